@@ -1,0 +1,128 @@
+// C-ABI layer of libmoe_gg.so: argument validation, kernel-variant choice, launches.
+#include "../../include/moe_gg.h"
+#include "kernels.h"
+#include "tile_sched.h"
+
+#include <atomic>
+#include <mutex>
+
+namespace {
+
+struct DeviceInfo {
+  int cus = 0;
+  int xcds = 8;
+  bool ok = false;
+};
+
+constexpr int kMaxDevices = 16;
+DeviceInfo g_dev[kMaxDevices];
+std::once_flag g_dev_once[kMaxDevices];
+std::atomic<int> g_variant[8] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
+
+int current_device_info(const DeviceInfo** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return MOE_GG_EDEVICE;
+  std::call_once(g_dev_once[dev], [dev]() {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return;
+    g_dev[dev].cus = prop.multiProcessorCount;
+    g_dev[dev].xcds = 8;  // MI355X: 8 XCDs x 32 CUs, workgroups dealt round-robin over XCDs
+    g_dev[dev].ok = prop.multiProcessorCount > 0;
+  });
+  if (!g_dev[dev].ok) return MOE_GG_EDEVICE;
+  *out = &g_dev[dev];
+  return MOE_GG_OK;
+}
+
+bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+int moe_gg_abi_version(void) { return MOE_GG_ABI_VERSION; }
+
+const char* moe_gg_strerror(int code) {
+  switch (code) {
+    case MOE_GG_OK: return "success";
+    case MOE_GG_EINVAL: return "invalid argument (null pointer, negative size or bad enum)";
+    case MOE_GG_ESHAPE: return "inconsistent dimensions";
+    case MOE_GG_EALIGN: return "pointer or leading dimension not sufficiently aligned";
+    case MOE_GG_EUNSUPPORTED: return "request outside the supported range of the kernels";
+    case MOE_GG_EDEVICE: return "no usable gfx950 device";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "unknown moe_gg error";
+}
+
+int moe_gg_set_variant(int op, int variant) {
+  if (op < 0 || op >= 8) return MOE_GG_EINVAL;
+  g_variant[op].store(variant);
+  return MOE_GG_OK;
+}
+
+int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
+                             int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream) {
+  if (G < 0 || M < 0 || N < 0 || K < 0) return MOE_GG_EINVAL;
+  if (out_layout != MOE_GG_OUT_MN && out_layout != MOE_GG_OUT_BLOCK) return MOE_GG_EINVAL;
+  if (M > INT32_MAX || (int64_t)G * N > INT32_MAX || ldy > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  const int64_t min_ld = out_layout == MOE_GG_OUT_BLOCK ? (int64_t)N * G : (int64_t)N;
+  if (ldy < min_ld) return MOE_GG_ESHAPE;
+  if (G == 0 || M == 0 || N == 0) return MOE_GG_OK;  // nothing to compute
+  if (!x || !w || !y || !m_sizes) return MOE_GG_EINVAL;
+  if (K == 0) return MOE_GG_ESHAPE;
+  if (G > MOE_GG_MAX_GROUPS_ABI) return MOE_GG_EUNSUPPORTED;
+  if (!aligned(m_sizes, 4) || !aligned(x, 2) || !aligned(w, 2) || !aligned(y, 2)) return MOE_GG_EALIGN;
+
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != MOE_GG_OK) return rc;
+
+  GgParams p{};
+  p.x = x; p.w = w; p.y = y; p.m_sizes = m_sizes;
+  p.G = G; p.M = (int)M; p.N = N; p.K = K;
+  p.ldy = (int)ldy;
+  p.col_block = out_layout == MOE_GG_OUT_BLOCK ? N : 0;
+  p.vec_store = aligned(y, 8) && ldy % 4 == 0 && N % 4 == 0;
+  p.xcds = di->xcds;
+
+  hipStream_t s = (hipStream_t)stream;
+  const bool tiled_ok = K % 64 == 0 && aligned(x, 16) && aligned(w, 16);
+  if (!tiled_ok) return (int)gg_bf16_generic_launch(p, s);
+
+  int variant = g_variant[MOE_GG_OP_GG_BF16].load();
+  if (variant < 0) variant = 0;
+  if (gg_bf16_prefill_block_m(variant) == 0) return MOE_GG_EINVAL;
+  int num_wg = di->cus - di->cus % p.xcds;
+  if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
+  return (int)gg_bf16_prefill_launch(p, variant, num_wg, s);
+}
+
+int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
+                                int block_n, int num_workgroups, int xcds, int32_t* out,
+                                int max_tiles) {
+  if (!m_sizes_host || !out || G <= 0 || G > MOE_GG_MAX_GROUPS_ABI || block_m <= 0 || block_n <= 0 ||
+      num_workgroups <= 0 || xcds <= 0 || num_workgroups % xcds != 0 || M < 0 || N <= 0)
+    return MOE_GG_EINVAL;
+  static thread_local int32_t row_off[MOE_GG_MAX_GROUPS_ABI + 1], tile_off[MOE_GG_MAX_GROUPS_ABI + 1];
+  const int ntn = moe_gg_cdiv(N, block_n);
+  const int total = moe_gg_build_tables(m_sizes_host, G, M, block_m, ntn, row_off, tile_off);
+  int written = 0;
+  for (int wg = 0; wg < num_workgroups; ++wg) {
+    for (int round = 0; round * num_workgroups < total; ++round) {
+      const int L = moe_gg_tile_of(wg, num_workgroups, xcds, round);
+      if (L >= total) continue;
+      if (written >= max_tiles) return written;
+      MoeGgTile t = moe_gg_decode_tile(row_off, tile_off, G, L, block_m);
+      int32_t* o = out + (size_t)written * 5;
+      o[0] = wg; o[1] = t.g; o[2] = t.tm; o[3] = t.tn; o[4] = t.row0;
+      ++written;
+    }
+  }
+  return written;
+}
+
+}  // extern "C"

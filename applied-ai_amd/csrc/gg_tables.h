@@ -1,0 +1,65 @@
+// In-kernel construction of the row-offset and tile-offset tables of tile_sched.h.
+// One wavefront scans m_sizes with a shuffle prefix sum; the result is identical to
+// moe_gg_build_tables (row offsets are min(prefix, M), which equals the serial clamped walk).
+#pragma once
+#include "common.h"
+#include "tile_sched.h"
+
+DEVINL long long wave_incl_scan_i64(long long x) {
+  const int l = lane_id();
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    long long v = __shfl_up(x, d, 64);
+    if (l >= d) x += v;
+  }
+  return x;
+}
+
+// Must be called by every thread of the workgroup (it contains barriers).
+// row_off / tile_off: LDS arrays of G + 1 entries, G <= MOE_GG_MAX_GROUPS.
+DEVINL void build_group_tables(const int32_t* __restrict__ m_sizes, int G, int M, int BM, int n_tiles_n,
+                               int32_t* row_off, int32_t* tile_off) {
+  const int per = (G + 63) >> 6;
+  if (wave_id() == 0) {
+    const int g0 = lane_id() * per;
+    long long s = 0;
+    for (int i = 0; i < per; ++i) {
+      int g = g0 + i;
+      if (g < G) {
+        int m = m_sizes[g];
+        m = m < 0 ? 0 : (m > M ? M : m);
+        s += m;
+      }
+    }
+    long long run = wave_incl_scan_i64(s) - s;
+    for (int i = 0; i < per; ++i) {
+      int g = g0 + i;
+      if (g < G) {
+        row_off[g] = (int32_t)(run > M ? M : run);
+        int m = m_sizes[g];
+        m = m < 0 ? 0 : (m > M ? M : m);
+        run += m;
+      }
+    }
+    if (lane_id() == 63) row_off[G] = (int32_t)(run > M ? M : run);
+  }
+  __syncthreads();
+  if (wave_id() == 0) {
+    const int g0 = lane_id() * per;
+    long long s = 0;
+    for (int i = 0; i < per; ++i) {
+      int g = g0 + i;
+      if (g < G) s += moe_gg_cdiv(row_off[g + 1] - row_off[g], BM) * n_tiles_n;
+    }
+    long long run = wave_incl_scan_i64(s) - s;
+    for (int i = 0; i < per; ++i) {
+      int g = g0 + i;
+      if (g < G) {
+        tile_off[g] = (int32_t)run;
+        run += moe_gg_cdiv(row_off[g + 1] - row_off[g], BM) * n_tiles_n;
+      }
+    }
+    if (lane_id() == 63) tile_off[G] = (int32_t)run;
+  }
+  __syncthreads();
+}

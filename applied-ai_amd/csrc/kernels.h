@@ -1,0 +1,25 @@
+// Internal launch interface between the C-ABI layer (api.hip) and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// Arguments of the grouped GEMM kernels. x is [M, K] row-major, w is [G * N, K] row-major
+// (expert g owns rows g*N .. (g+1)*N), y has leading dimension ldy; expert g writes its rows at
+// column offset g * col_block (0 for the [M, N] layout, N for the [M, N*G] block layout).
+struct GgParams {
+  const void* x;
+  const void* w;
+  void* y;
+  const int32_t* m_sizes;  // device, G entries
+  const float* x_scale;    // fp8 only
+  const float* w_scale;    // fp8 only
+  int G, M, N, K;
+  int ldy;
+  int col_block;
+  int vec_store;  // 1 when 8-byte aligned row segments can be stored as one dwordx2
+  int xcds;       // number of XCDs the persistent grid is spread over
+};
+
+hipError_t gg_bf16_prefill_launch(const GgParams& p, int variant, int num_wg, hipStream_t stream);
+int gg_bf16_prefill_block_m(int variant);
+hipError_t gg_bf16_generic_launch(const GgParams& p, hipStream_t stream);

@@ -1,0 +1,88 @@
+// Tile scheduler for the grouped GEMM: walks the m_sizes offset table.
+//
+// Restates the persistent tile walk of the reference kernel
+// (dev/triton_groupGEMM/groupgemm.py:159-254): groups are visited in order, empty groups
+// contribute no tiles, and inside a group the linear tile index runs M-fastest
+// (tile_m = idx % num_m_tiles, tile_n = idx / num_m_tiles; groupgemm.py:190-191).
+// Instead of every workgroup re-scanning all G sizes per tile, two exclusive prefix tables
+// are built once per launch (row offsets = groupgemm.py:161-165's running M offset, and tile
+// offsets) and a tile id is mapped to its group with a binary search.
+//
+// The same code compiles for the host (used by the scheduler tests) and the device.
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define MOE_GG_HD __host__ __device__ inline
+#else
+#define MOE_GG_HD inline
+#endif
+
+struct MoeGgTile {
+  int g;      // group (expert) index
+  int tm;     // tile index along the group's rows
+  int tn;     // tile index along N
+  int row0;   // first row of the group in x / y
+  int rows;   // number of rows of the group (m_sizes[g] after clamping)
+};
+
+// Rows a group may use: negative sizes count as empty and the running sum never passes M,
+// so a corrupt m_sizes cannot make a kernel read or write out of bounds.
+MOE_GG_HD int moe_gg_clamp_rows(int m, int64_t row0, int64_t M) {
+  if (m < 0) m = 0;
+  int64_t left = M - row0;
+  if (left < 0) left = 0;
+  return (int64_t)m > left ? (int)left : m;
+}
+
+MOE_GG_HD int moe_gg_cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// Serial construction of both tables; row_off and tile_off have G + 1 entries.
+// Returns the total number of tiles.
+MOE_GG_HD int moe_gg_build_tables(const int32_t* m_sizes, int G, int64_t M, int BM, int n_tiles_n,
+                                  int32_t* row_off, int32_t* tile_off) {
+  int64_t r = 0;
+  int t = 0;
+  for (int g = 0; g < G; ++g) {
+    row_off[g] = (int32_t)r;
+    tile_off[g] = t;
+    int m = moe_gg_clamp_rows(m_sizes[g], r, M);
+    r += m;
+    t += moe_gg_cdiv(m, BM) * n_tiles_n;
+  }
+  row_off[G] = (int32_t)r;
+  tile_off[G] = t;
+  return t;
+}
+
+// Largest g with tile_off[g] <= L, skipping empty groups (their range is empty). L < tile_off[G].
+MOE_GG_HD int moe_gg_find_group(const int32_t* tile_off, int G, int L) {
+  int lo = 0, hi = G;  // invariant: tile_off[lo] <= L < tile_off[hi]
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (tile_off[mid] <= L) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+MOE_GG_HD MoeGgTile moe_gg_decode_tile(const int32_t* row_off, const int32_t* tile_off, int G, int L,
+                                       int BM) {
+  MoeGgTile t;
+  t.g = moe_gg_find_group(tile_off, G, L);
+  t.row0 = row_off[t.g];
+  t.rows = row_off[t.g + 1] - t.row0;
+  int idx = L - tile_off[t.g];
+  int nmt = moe_gg_cdiv(t.rows, BM);
+  t.tm = idx % nmt;
+  t.tn = idx / nmt;
+  return t;
+}
+
+// Linear tile id handled by persistent workgroup `wg` (of `nwg`, a multiple of `xcds`) in round
+// `round`. Workgroups are dealt to the chip's XCDs round-robin (wg % xcds), each XCD with a
+// private L2; giving an XCD a contiguous run of nwg / xcds tile ids per round makes the
+// workgroups that share an L2 also share weight and activation tiles.
+MOE_GG_HD int moe_gg_tile_of(int wg, int nwg, int xcds, int round) {
+  int per = nwg / xcds;
+  return round * nwg + (wg % xcds) * per + wg / xcds;
+}

@@ -1,0 +1,77 @@
+"""Host-side mirror of the reference's Python entry functions for the MoE grouped-GEMM path.
+
+Same names, argument meaning and return values as the reference launchers; the work is done by
+hand-written gfx950 kernels behind the C ABI in include/moe_gg.h. torch is used for device
+memory and the current stream only.
+"""
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+OUT_MN = 0
+OUT_BLOCK = 1
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_cuda(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                "applied_ai_amd ops run on a HIP device only (got a %s tensor); there is no CPU path"
+                % t.device.type
+            )
+        if t.device != dev:
+            raise RuntimeError("all tensors must be on the same device")
+    return dev
+
+
+def _grouped_gemm_bf16(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, out_layout: int) -> torch.Tensor:
+    # Mirrors _grouped_gemm (dev/triton_groupGEMM/groupgemm.py:407-427): contiguity asserts,
+    # G from m_sizes, N = w.shape[0] // G, K check, torch.empty output.
+    assert x.is_contiguous()
+    assert w.is_contiguous()
+    assert m_sizes.is_contiguous()
+    if x.dim() != 2 or w.dim() != 2 or m_sizes.dim() != 1:
+        raise ValueError("x must be [M, K], w must be [G*N, K], m_sizes must be [G]")
+    G = m_sizes.shape[0]
+    M, K = x.shape
+    if G == 0 or w.shape[0] % G != 0:
+        raise ValueError(f"w.shape[0]={w.shape[0]} is not a multiple of G={G}")
+    N = w.shape[0] // G
+    assert K == w.shape[1], f"K mismatch: x has {K}, w has {w.shape[1]}"
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ValueError("grouped_gemm takes bf16 x and w")
+    if m_sizes.dtype != torch.int32:
+        raise ValueError("m_sizes must be int32")
+    dev = _require_cuda(x, w, m_sizes)
+    cols = N * G if out_layout == OUT_BLOCK else N
+    y = torch.empty((M, cols), device=dev, dtype=torch.bfloat16)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_grouped_gemm_bf16(
+            x.data_ptr(), w.data_ptr(), y.data_ptr(), m_sizes.data_ptr(), G, M, N, K, cols, out_layout,
+            _stream_ptr(dev),
+        )
+    _lib.check(rc, "moe_gg_grouped_gemm_bf16")
+    return y
+
+
+def grouped_gemm(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor) -> torch.Tensor:
+    """y[off_g:off_g+m_g] = x[off_g:off_g+m_g] @ w[g*N:(g+1)*N].T for every expert g; y is [M, N] bf16.
+
+    Drop-in for grouped_gemm (dev/triton_groupGEMM/groupgemm.py:518-521). Rows at or beyond
+    sum(m_sizes) are left uninitialised, as in the reference (torch.empty, groupgemm.py:427).
+    """
+    return _grouped_gemm_bf16(x, w, m_sizes, OUT_MN)
+
+
+def grouped_gemm_forward(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor) -> torch.Tensor:
+    """Same product with the [M, N*G] output of the MoE-training copy: expert g writes columns
+    [g*N, (g+1)*N) of its own rows (kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:626-629,
+    280-289); everything else is left uninitialised."""
+    return _grouped_gemm_bf16(x, w, m_sizes, OUT_BLOCK)

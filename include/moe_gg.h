@@ -1,0 +1,79 @@
+/*
+ * moe_gg.h - C ABI of libmoe_gg.so: MI355X (gfx950) MoE grouped-GEMM inference path.
+ *
+ * Plain pointers and sizes only; no torch types. Every pointer marked "device" must be HIP device
+ * memory on the current device. All entry points are asynchronous: they enqueue kernels on `stream`
+ * (a hipStream_t passed as void*; NULL = the default stream) and return without synchronising.
+ * The library keeps no per-call state, never allocates device memory and never synchronises.
+ *
+ * Return value: 0 on success, a negative MOE_GG_E* code for a rejected argument (nothing was
+ * launched), or a positive hipError_t from the HIP runtime.
+ *
+ * The boundary follows the reference's own native pattern: an extern "C" launcher taking raw
+ * pointers + dims + stream and returning an error code
+ * (kernels/blackwell/cute_gemm_01/sm100_gemm.h:33-35), wrapped by host code that checks
+ * device / dtype / contiguity / shape (kernels/blackwell/cute_gemm_01/sm100_gemm_pytorch.cpp:49-100).
+ */
+#ifndef MOE_GG_H
+#define MOE_GG_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE_GG_ABI_VERSION 1
+
+#define MOE_GG_OK 0
+#define MOE_GG_EINVAL (-1)       /* null pointer, negative size, bad enum value */
+#define MOE_GG_ESHAPE (-2)       /* dimensions inconsistent with each other */
+#define MOE_GG_EALIGN (-3)       /* pointer or leading dimension not aligned as required */
+#define MOE_GG_EUNSUPPORTED (-4) /* valid request outside what the kernels cover (e.g. G > 1024) */
+#define MOE_GG_EDEVICE (-5)      /* no usable gfx950 device */
+
+#define MOE_GG_MAX_GROUPS_ABI 1024 /* largest G the grouped kernels accept */
+
+/* Output layouts of the grouped GEMM. */
+#define MOE_GG_OUT_MN 0     /* y is [M, N]: dev/triton_groupGEMM/groupgemm.py:427 */
+#define MOE_GG_OUT_BLOCK 1  /* y is [M, N*G], expert g writes columns [g*N, (g+1)*N):
+                               kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:280-289 */
+
+int moe_gg_abi_version(void);
+const char* moe_gg_strerror(int code);
+
+/*
+ * bf16 grouped GEMM forward. Replaces grouped_gemm -> _grouped_gemm -> _kernel_grouped_gemm
+ * (dev/triton_groupGEMM/groupgemm.py:518-521, 407-515, 130-254) and, with
+ * out_layout = MOE_GG_OUT_BLOCK, grouped_gemm_forward
+ * (kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:626-629).
+ *
+ *   x        device, bf16 [M, K] row-major, rows sorted by expert
+ *   w        device, bf16 [G*N, K] row-major (stacked expert weights)
+ *   y        device, bf16, leading dimension ldy elements; rows >= sum(m_sizes) are not written
+ *   m_sizes  device, int32 [G]; rows per expert. Consumed on the device (no host copy, no sync).
+ *            Negative entries count as 0 and the running sum is clamped at M.
+ * fp32 accumulation, round-to-nearest-even bf16 output.
+ */
+int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
+                             int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream);
+
+/*
+ * Test / tuning hooks (no counterpart in the reference).
+ * moe_gg_set_variant pins the kernel variant used by an op (-1 = automatic choice).
+ * moe_gg_host_enumerate_tiles runs the kernels' tile scheduler on the host: for a host copy of
+ * m_sizes it writes, for every persistent workgroup in launch order, the tiles it would visit as
+ * int32 quintuples (workgroup, group, tile_m, tile_n, first_row_of_group). Returns the number of
+ * tiles written (<= max_tiles), or a negative error.
+ */
+#define MOE_GG_OP_GG_BF16 0
+int moe_gg_set_variant(int op, int variant);
+int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
+                                int block_n, int num_workgroups, int xcds, int32_t* out,
+                                int max_tiles);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_GG_H */
