@@ -1,0 +1,215 @@
+"""numpy front end of the C oracle (moe_oracle.c) plus the torch per-expert loop used as CPU baseline.
+
+TEST INFRASTRUCTURE ONLY - see the header of moe_oracle.c. All functions take and return numpy arrays
+(bf16 / fp8 data is passed as float32 values or uint8 codes); nothing here touches a GPU.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libmoe_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    if force:
+        subprocess.run(["make", "-C", _HERE, "clean"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+    return _SO
+
+
+def _l():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        _lib = ctypes.CDLL(_SO)
+        _lib.orc_e4m3_to_f32.restype = ctypes.c_float
+        _lib.orc_e4m3_to_f32.argtypes = [ctypes.c_uint8]
+        _lib.orc_f32_to_e4m3.restype = ctypes.c_uint8
+        _lib.orc_f32_to_e4m3.argtypes = [ctypes.c_float]
+        _lib.orc_round_bf16.restype = ctypes.c_float
+        _lib.orc_round_bf16.argtypes = [ctypes.c_float]
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def offsets(m_sizes):
+    """Exclusive prefix sum [G+1] of m_sizes (groupgemm.py:159-165)."""
+    m = _i32(m_sizes)
+    out = np.empty(m.shape[0] + 1, dtype=np.int32)
+    _l().orc_offsets(_p(m), ctypes.c_int(m.shape[0]), _p(out))
+    return out
+
+
+def grouped_gemm(x, w, m_sizes, block_layout=False, fill=np.nan):
+    """fp32 per-expert x_g @ w_g^T (unit_tests.py:49-55). Unwritten entries hold `fill`."""
+    x, w, m = _f32(x), _f32(w), _i32(m_sizes)
+    G = m.shape[0]
+    M, K = x.shape
+    N = w.shape[0] // G
+    cols = N * G if block_layout else N
+    y = np.full((M, cols), fill, dtype=np.float32)
+    _l().orc_grouped_gemm(_p(x), _p(w), _p(m), ctypes.c_int(G), ctypes.c_int64(M), ctypes.c_int(N),
+                          ctypes.c_int(K), _p(y), ctypes.c_int64(cols), ctypes.c_int(N if block_layout else 0))
+    return y
+
+
+def topk(logits, k):
+    """Top-k expert ids per token, descending score, ties to the lower index (test_moe_gemm.py:54-57)."""
+    lg = _f32(logits)
+    T, E = lg.shape
+    ids = np.empty((T, k), dtype=np.int32)
+    _l().orc_topk(_p(lg), ctypes.c_int64(T), ctypes.c_int(E), ctypes.c_int(k), _p(ids))
+    return ids
+
+
+def route(topk_ids, num_experts):
+    """(perm, m_sizes): flat indices grouped by ascending expert, stable (v0_moe_fused.py:141-166)."""
+    flat = _i32(np.asarray(topk_ids).reshape(-1))
+    perm = np.empty(flat.shape[0], dtype=np.int32)
+    m = np.empty(num_experts, dtype=np.int32)
+    _l().orc_route(_p(flat), ctypes.c_int64(flat.shape[0]), ctypes.c_int(num_experts), _p(perm), _p(m))
+    return perm, m
+
+
+def moe_align_block_size(topk_ids, block_size, num_experts):
+    flat = _i32(np.asarray(topk_ids).reshape(-1))
+    n = flat.shape[0]
+    sorted_ids = np.full(n + num_experts * (block_size - 1), n, dtype=np.int32)
+    expert_ids = np.full(n + num_experts, -1, dtype=np.int32)
+    post = np.zeros(1, dtype=np.int32)
+    _l().orc_moe_align_block_size(_p(flat), ctypes.c_int64(n), ctypes.c_int(num_experts),
+                                  ctypes.c_int(block_size), _p(sorted_ids), _p(expert_ids), _p(post))
+    return sorted_ids, expert_ids, int(post[0])
+
+
+def w4_dequant(qweight, scales, qzeros, group_size=128, zero_offset=1):
+    """[K, N] fp32 weights from GPTQ-packed int4 (splitk_dequant_gemm.py:56-77)."""
+    qw, s, qz = _i32(qweight), _f32(scales), _i32(qzeros)
+    K, N = qw.shape[0] * 8, qw.shape[1]
+    out = np.empty((K, N), dtype=np.float32)
+    _l().orc_w4_dequant(_p(qw), _p(s), _p(qz), ctypes.c_int(K), ctypes.c_int(N), ctypes.c_int(group_size),
+                        ctypes.c_int(zero_offset), _p(out))
+    return out
+
+
+def w4a16_gemm(a, qweight, scales, qzeros, group_size=128, zero_offset=1):
+    a, qw, s, qz = _f32(a), _i32(qweight), _f32(scales), _i32(qzeros)
+    M, K = a.shape
+    N = qw.shape[1]
+    c = np.empty((M, N), dtype=np.float32)
+    _l().orc_w4a16_gemm(_p(a), _p(qw), _p(s), _p(qz), ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(K),
+                        ctypes.c_int(group_size), ctypes.c_int(zero_offset), _p(c))
+    return c
+
+
+def e4m3_to_f32(codes):
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    lut = np.array([_l().orc_e4m3_to_f32(i) for i in range(256)], dtype=np.float32)
+    return lut[codes]
+
+
+def f32_to_e4m3(x):
+    x = _f32(x)
+    out = np.empty(x.shape, dtype=np.uint8)
+    flat_in, flat_out = x.reshape(-1), out.reshape(-1)
+    f = _l().orc_f32_to_e4m3
+    for i in range(flat_in.shape[0]):
+        flat_out[i] = f(float(flat_in[i]))
+    return out
+
+
+def fp8_groupwise_quant(x, block=128):
+    """(codes uint8 like x, scales [..., K/block] fp32) - float8_groupwise_quant.py:36-50."""
+    x = _f32(x)
+    q = np.empty(x.shape, dtype=np.uint8)
+    scales = np.empty(x.shape[:-1] + (x.shape[-1] // block,), dtype=np.float32)
+    _l().orc_fp8_groupwise_quant(_p(x), ctypes.c_int64(x.size), ctypes.c_int(block), _p(q), _p(scales))
+    return q, scales
+
+
+def fp8_block_quant_weight(w, block=128):
+    """128x128 block quantiser for [rows, K] weights (defined by this oracle; parity unpinned)."""
+    w = _f32(w)
+    rows, K = w.shape
+    q = np.empty(w.shape, dtype=np.uint8)
+    scales = np.empty((rows // block, K // block), dtype=np.float32)
+    _l().orc_fp8_block_quant_weight(_p(w), ctypes.c_int64(rows), ctypes.c_int(K), ctypes.c_int(block), _p(q), _p(scales))
+    return q, scales
+
+
+def grouped_gemm_fp8(xq, wq, x_scale, w_scale, m_sizes, scale_mode, block_layout=False, fill=np.nan):
+    """fp8 grouped GEMM oracle; scale_mode 0 = row-wise (base_testing.py:83-88), 1 = 1x128 / 128x128 blocks."""
+    xq = np.ascontiguousarray(xq, dtype=np.uint8)
+    wq = np.ascontiguousarray(wq, dtype=np.uint8)
+    xs, ws, m = _f32(x_scale), _f32(w_scale), _i32(m_sizes)
+    G = m.shape[0]
+    M, K = xq.shape
+    N = wq.shape[0] // G
+    cols = N * G if block_layout else N
+    y = np.full((M, cols), fill, dtype=np.float32)
+    _l().orc_grouped_gemm_fp8(_p(xq), _p(wq), _p(xs), _p(ws), ctypes.c_int(scale_mode), _p(m), ctypes.c_int(G),
+                              ctypes.c_int64(M), ctypes.c_int(N), ctypes.c_int(K), _p(y), ctypes.c_int64(cols),
+                              ctypes.c_int(N if block_layout else 0))
+    return y
+
+
+def round_bf16(x):
+    """fp32 -> bf16 -> fp32, round-to-nearest-even (vectorised restatement of orc_round_bf16)."""
+    u = _f32(x).view(np.uint32).astype(np.uint64)
+    lsb = (u >> 16) & 1
+    r = ((u + 0x7FFF + lsb) & 0xFFFF0000).astype(np.uint32)
+    return r.view(np.float32).reshape(np.shape(x))
+
+
+def pack_int4_along_k(q):
+    """[K, N] values 0..15 -> int32 [K/8, N], nibble j of a word = row 8*i + j (splitk_dequant_gemm.py:56,76)."""
+    q = np.asarray(q, dtype=np.uint32)
+    K, N = q.shape
+    out = np.zeros((K // 8, N), dtype=np.uint32)
+    for j in range(8):
+        out |= q[j::8, :] << np.uint32(4 * j)
+    return out.view(np.int32)
+
+
+def pack_int4_along_n(z):
+    """[G, N] values 0..15 -> int32 [G, N/8], nibble j of a word = column 8*i + j (splitk_dequant_gemm.py:57,70)."""
+    z = np.asarray(z, dtype=np.uint32)
+    G, N = z.shape
+    out = np.zeros((G, N // 8), dtype=np.uint32)
+    for j in range(8):
+        out |= z[:, j::8] << np.uint32(4 * j)
+    return out.view(np.int32)
+
+
+def grouped_gemm_torch_loop(x, w, m_sizes):
+    """The reference's CPU-expressible path: a per-expert torch.matmul loop over the expert-sorted rows
+    (dev/triton_groupGEMM/testing/unit_tests.py:49-55), fp32 on the host cores. Used by tests as a second
+    opinion on the C oracle and by bench.py as the timed CPU baseline."""
+    import torch
+
+    G = len(m_sizes)
+    N = w.shape[0] // G
+    y = torch.zeros((x.shape[0], N), dtype=torch.float32)
+    start = 0
+    for g in range(G):
+        m = int(m_sizes[g])
+        if m > 0:
+            y[start:start + m] = x[start:start + m] @ w[g * N:(g + 1) * N].T
+        start += m
+    return y

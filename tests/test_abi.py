@@ -1,0 +1,103 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol the header declares, rejects bad
+arguments without launching, and its tile scheduler covers every output tile exactly once."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "moe_gg.h")
+I32P = ctypes.POINTER(ctypes.c_int32)
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(moe_gg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound(lib):
+    import applied_ai_amd
+
+    names = declared_symbols()
+    assert "moe_gg_grouped_gemm_bf16" in names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/moe_gg.h but not exported"
+        assert n in applied_ai_amd._lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert sorted(applied_ai_amd._lib.SIGNATURES) == names
+
+
+def test_abi_version_and_strerror(lib):
+    assert lib.moe_gg_abi_version() == 1
+    assert lib.moe_gg_strerror(0) == b"success"
+    for code in (-1, -2, -3, -4, -5):
+        assert len(lib.moe_gg_strerror(code)) > 0
+
+
+def test_argument_errors_are_rejected_before_any_launch(lib):
+    f = lib.moe_gg_grouped_gemm_bf16
+    # negative size, bad layout, too small leading dimension, too many groups, null pointers
+    assert f(None, None, None, None, -1, 8, 8, 8, 8, 0, None) == -1
+    assert f(None, None, None, None, 2, 8, 8, 8, 8, 7, None) == -1
+    assert f(None, None, None, None, 2, 8, 8, 8, 4, 0, None) == -2
+    assert f(None, None, None, None, 2, 8, 8, 8, 8, 1, None) == -2   # block layout needs ldy >= N*G
+    assert f(None, None, None, None, 2, 8, 8, 8, 8, 0, None) == -1   # null pointers with work to do
+    assert f(None, None, None, None, 2, 0, 8, 8, 8, 0, None) == 0    # M == 0: nothing to do
+
+
+def enumerate_tiles(lib, m_sizes, M, N, bm, bn, nwg, xcds):
+    ms = np.ascontiguousarray(m_sizes, dtype=np.int32)
+    cap = 1 << 16
+    out = np.zeros((cap, 5), dtype=np.int32)
+    n = lib.moe_gg_host_enumerate_tiles(ms.ctypes.data_as(I32P), len(ms), M, N, bm, bn, nwg, xcds,
+                                        out.ctypes.data_as(I32P), cap)
+    assert n >= 0
+    return out[:n]
+
+
+@pytest.mark.parametrize("m_sizes,N,bm,bn,nwg", [
+    ([25, 50, 25], 512, 16, 256, 8),
+    ([0, 300, 1, 399], 328, 256, 256, 256),
+    ([1026, 1002, 1065, 981, 1034, 1000, 1036, 1048], 14336, 256, 256, 256),
+    ([0] * 7 + [64], 4096, 128, 128, 16),
+    ([3, 0, 0, 9, 16, 0, 11, 25], 14336, 256, 256, 256),
+])
+def test_scheduler_is_an_exact_cover(lib, m_sizes, N, bm, bn, nwg):
+    M = sum(m_sizes)
+    tiles = enumerate_tiles(lib, m_sizes, M, N, bm, bn, nwg, 8)
+    off = O.offsets(m_sizes)
+    expect = set()
+    for g, m in enumerate(m_sizes):
+        for tm in range(-(-m // bm)):
+            for tn in range(-(-N // bn)):
+                expect.add((g, tm, tn))
+    got = [tuple(t[1:4]) for t in tiles.tolist()]
+    assert len(got) == len(set(got)) == len(expect)      # no duplicates
+    assert set(got) == expect                            # nothing missing, empty groups skipped
+    for wg, g, tm, tn, row0 in tiles.tolist():
+        assert row0 == off[g]
+    # a workgroup's tile ids ascend, and workgroups of one XCD (wg % 8) share a contiguous id range
+    if len(tiles) >= nwg:
+        per_wg = {}
+        for i, t in enumerate(tiles.tolist()):
+            per_wg.setdefault(t[0], []).append(i)
+        assert max(len(v) for v in per_wg.values()) - min(len(v) for v in per_wg.values()) <= 1
+
+
+def test_scheduler_clamps_corrupt_sizes(lib):
+    # negative sizes count as empty; a running sum beyond M is cut at M, so no tile starts past M
+    tiles = enumerate_tiles(lib, [10, -5, 100, 7], 50, 64, 16, 64, 8, 8)
+    got = sorted(set((g, tm) for _, g, tm, _, _ in tiles.tolist()))
+    assert got == [(0, 0), (2, 0), (2, 1), (2, 2)]       # group 2 is cut to 40 rows, group 3 to 0
+
+
+def test_scheduler_rejects_bad_arguments(lib):
+    ms = np.array([1, 2], dtype=np.int32)
+    out = np.zeros((8, 5), dtype=np.int32)
+    args = (ms.ctypes.data_as(I32P), 2, 3, 64, 16, 64)
+    assert lib.moe_gg_host_enumerate_tiles(*args, 6, 4, out.ctypes.data_as(I32P), 8) == -1  # 6 % 4 != 0
+    assert lib.moe_gg_host_enumerate_tiles(*args, 0, 1, out.ctypes.data_as(I32P), 8) == -1

@@ -1,0 +1,163 @@
+"""GPU parity of the bf16 grouped GEMM (through the C ABI) against the CPU oracle.
+Tolerance: rtol 1e-2 / atol 1e-2 against the fp32 per-expert product (the bar of
+kernels/MoE/group_GEMM/triton/testing/fast_verification.py:111-122)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.gpu_util import bf16_inputs, random_m_sizes, to_np
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+def run(x, w, m_sizes, fn=None):
+    import applied_ai_amd as A
+
+    fn = fn or A.grouped_gemm
+    ms = torch.tensor(m_sizes, dtype=torch.int32, device="cuda")
+    y = fn(x.cuda(), w.cuda(), ms)
+    torch.cuda.synchronize()
+    return y
+
+
+def check(x, w, m_sizes):
+    print(f"case G={len(m_sizes)} M={x.shape[0]} K={x.shape[1]} N={w.shape[0] // len(m_sizes)} m_sizes={m_sizes[:16]}", flush=True)
+    y = to_np(run(x, w, m_sizes))
+    ref = O.grouped_gemm(to_np(x), to_np(w), m_sizes)
+    tot = sum(m_sizes)
+    np.testing.assert_allclose(y[:tot], ref[:tot], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("G", [1, 4, 16])
+@pytest.mark.parametrize("M", [64, 512])
+def test_reference_base_shapes(G, M):
+    # dev/triton_groupGEMM/testing/base_testing.py:135-138: N = K = 256
+    x, w, gen = bf16_inputs(G, M, 256, 256, seed=G * 1000 + M)
+    check(x, w, random_m_sizes(G, M, gen))
+
+
+@pytest.mark.parametrize("G", [4, 8])
+@pytest.mark.parametrize("M", [128, 256])
+@pytest.mark.parametrize("N,K", [(128, 256), (256, 128), (64, 64)])
+def test_reference_various_dimensions(G, M, N, K):
+    # dev/triton_groupGEMM/testing/unit_tests.py:99-103
+    x, w, gen = bf16_inputs(G, M, N, K, seed=7 + G + M + N)
+    check(x, w, random_m_sizes(G, M, gen))
+
+
+@pytest.mark.parametrize("G,M,N,K,m_sizes", [
+    (1, 32, 32, 32, [32]),              # unit_tests.py:110-116
+    (3, 100, 32, 32, [25, 50, 25]),     # unit_tests.py:119-134
+    (2, 8, 8, 8, [4, 4]),               # unit_tests.py:136-149
+    (32, 32 * 4, 16, 16, [4] * 32),     # unit_tests.py:151-166 (G=32, N=K=16)
+    (4, 128, 64, 128, [32] * 4),        # unit_tests.py:224
+    (4, 700, 328, 192, [0, 300, 1, 399]),
+    (5, 70, 100, 72, [0, 0, 70, 0, 0]),  # K not a multiple of 64: generic kernel
+    (3, 50, 33, 40, [20, 10, 20]),       # odd N
+])
+def test_edge_cases(G, M, N, K, m_sizes):
+    x, w, _ = bf16_inputs(G, M, N, K, seed=11)
+    check(x, w, m_sizes)
+
+
+def test_large_two_groups():
+    # unit_tests.py:235-256: (G, M, N, K) = (2, 2048, 512, 1024), m_sizes [1024, 1024]
+    x, w, _ = bf16_inputs(2, 2048, 512, 1024, seed=12)
+    check(x, w, [1024, 1024])
+
+
+def test_fast_verification_shape_and_block_layout():
+    # kernels/MoE/group_GEMM/triton/testing/fast_verification.py:31-48,83-96: G=20, M=1024, N=512, K=256
+    import applied_ai_amd as A
+
+    G, M, N, K = 20, 1024, 512, 256
+    m_sizes = [52] * 4 + [51] * 16
+    x, w, _ = bf16_inputs(G, M, N, K, seed=13)
+    check(x, w, m_sizes)
+    ms = torch.tensor(m_sizes, dtype=torch.int32, device="cuda")
+    yb = torch.full((M, N * G), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = A._lib.lib().moe_gg_grouped_gemm_bf16(x.cuda().data_ptr(), w.cuda().data_ptr(), yb.data_ptr(), ms.data_ptr(),
+                                               G, M, N, K, N * G, 1, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ref = O.grouped_gemm(to_np(x), to_np(w), m_sizes, block_layout=True)
+    got = to_np(yb)
+    written = ~np.isnan(ref)
+    np.testing.assert_allclose(got[written], ref[written], rtol=RTOL, atol=ATOL)
+    assert np.isnan(got[~written]).all()  # other experts' column blocks are not touched
+    yf = A.grouped_gemm_forward(x.cuda(), w.cuda(), ms)
+    assert yf.shape == (M, N * G)
+    np.testing.assert_allclose(to_np(yf)[written], ref[written], rtol=RTOL, atol=ATOL)
+
+
+def test_rows_beyond_sum_are_untouched():
+    import applied_ai_amd as A
+
+    G, M, N, K = 3, 96, 64, 64
+    x, w, _ = bf16_inputs(G, M, N, K, seed=14)
+    ms = torch.tensor([10, 0, 30], dtype=torch.int32, device="cuda")
+    y = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    rc = A._lib.lib().moe_gg_grouped_gemm_bf16(x.cuda().data_ptr(), w.cuda().data_ptr(), y.data_ptr(), ms.data_ptr(),
+                                               G, M, N, K, N, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert (to_np(y)[40:] == 7.0).all()
+
+
+def test_bitwise_deterministic():
+    # unit_tests.py:214-233
+    x, w, _ = bf16_inputs(4, 128, 64, 128, seed=15)
+    a = run(x, w, [32] * 4)
+    b = run(x, w, [32] * 4)
+    assert torch.equal(a, b)
+
+
+def test_config1_plumbing_from_golden_fixture():
+    # BASELINE config 1 (8 experts, K=256, N=512, 256 tokens top-2) run in bf16 against the committed vectors
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "cfg1.npz"))
+    x = torch.from_numpy(z["x_sorted_bf16_bits"].astype(np.int16)).view(torch.bfloat16)
+    w = torch.from_numpy(z["w_bf16_bits"].astype(np.int16)).view(torch.bfloat16)
+    y = to_np(run(x, w, z["m_sizes"].tolist()))
+    np.testing.assert_allclose(y, z["y_bf16_inputs"], rtol=RTOL, atol=ATOL)
+
+
+def test_invalid_inputs_raise():
+    import applied_ai_amd as A
+
+    x = torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(16, 32, dtype=torch.bfloat16, device="cuda")
+    ms = torch.tensor([4, 4], dtype=torch.int32, device="cuda")
+    with pytest.raises(AssertionError):       # K mismatch: dev/triton_groupGEMM/groupgemm.py:425
+        A.grouped_gemm(x, w, ms)
+    with pytest.raises(ValueError):
+        A.grouped_gemm(x, torch.zeros(15, 64, dtype=torch.bfloat16, device="cuda"), ms)
+    with pytest.raises(RuntimeError):         # host tensors: no CPU path
+        A.grouped_gemm(x.cpu(), w.cpu(), ms.cpu())
+
+
+def test_mixtral_prefill_shape_sampled_rows():
+    """BASELINE config 2 at full size (T=4096 top-2, K=4096, N=14336, 8 experts); the oracle checks 8 sampled rows
+    per expert over all columns, and linearity checks the rest: y(2x) == 2 y(x) exactly in bf16."""
+    from applied_ai_amd import configs
+
+    c = configs.cfg2()
+    m_sizes = c["m_sizes"].tolist()
+    xs = c["x_sorted"].cuda(); wd = c["w"].cuda()
+    ms = c["m_sizes"].cuda()
+    import applied_ai_amd as A
+    y = A.grouped_gemm(xs, wd, ms)
+    y2 = A.grouped_gemm(xs * 2, wd, ms)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y * 2)
+    off = O.offsets(m_sizes)
+    rng = np.random.default_rng(0)
+    N = 14336
+    for g in range(8):
+        rows = np.unique(np.concatenate([[off[g], off[g + 1] - 1], rng.integers(off[g], off[g + 1], 6)]))
+        xr = c["x_sorted"][rows].float().numpy()
+        ref = O.grouped_gemm(xr, c["w"][g * N:(g + 1) * N].float().numpy(), [len(rows)])
+        np.testing.assert_allclose(to_np(y[rows]), ref, rtol=RTOL, atol=ATOL)
