@@ -95,10 +95,19 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
 
   int variant = g_variant[MOE_GG_OP_GG_BF16].load();
   if (variant < 0) variant = 0;
-  if (gg_bf16_prefill_block_m(variant) == 0) return MOE_GG_EINVAL;
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
+  if (variant >= 20) return (int)gg_bf16_pingpong_launch(p, variant - 20, num_wg, s);
+  if (gg_bf16_prefill_block_m(variant) == 0) return MOE_GG_EINVAL;
   return (int)gg_bf16_prefill_launch(p, variant, num_wg, s);
+}
+
+int moe_gg_debug_read_ts(long long* out256) { gg_debug_read_ts(out256); return 0; }
+
+int moe_gg_debug_read_clock(long long* cycles_and_100mhz_ticks) {
+  if (!cycles_and_100mhz_ticks) return MOE_GG_EINVAL;
+  gg_debug_read_clock(cycles_and_100mhz_ticks);
+  return MOE_GG_OK;
 }
 
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,

@@ -2,10 +2,17 @@
 //
 // Replaces the reference's _kernel_grouped_gemm (dev/triton_groupGEMM/groupgemm.py:130-254).
 // One workgroup per CU walks the tile list of tile_sched.h. Per tile, BM x 64 (activations) and
-// BN x 64 (weights) bf16 slabs are staged through double-buffered, XOR-swizzled LDS with 128-bit
-// global loads, and consumed by v_mfma_f32_16x16x32_bf16. The weight fragment is the MFMA "A"
-// operand and the activation fragment the "B" operand, so a lane ends up holding four consecutive
-// output columns of one output row and the epilogue stores 8 bytes per lane.
+// BN x 64 (weights) bf16 slabs are brought into double-buffered, XOR-swizzled LDS by
+// global_load_lds_dwordx4 (no VGPR staging) and consumed by v_mfma_f32_16x16x32_bf16.
+// The weight fragment is the MFMA "A" operand and the activation fragment the "B" operand, so a
+// lane ends up holding four consecutive output columns of one output row and the epilogue stores
+// 8 bytes per lane.
+//
+// K loop (one barrier per 64-wide K step): the fragments of the two 32-wide halves of a K step live
+// in two register sets F0/F1. While the MFMAs of one half run, the ds_reads of the next half are in
+// flight; the barrier in the middle of the step both publishes slab kt+1 and frees slab kt's buffer,
+// into which the loads of slab kt+2 are issued at once. A one-dword-per-line load into a scratch LDS
+// area runs PF_DIST steps ahead so that the slab loads hit in L2 instead of waiting for HBM.
 #include "common.h"
 #include "gg_tables.h"
 #include "kernels.h"
@@ -15,45 +22,80 @@ namespace {
 template <int BM_, int BN_, int WM_, int WN_>
 struct Cfg {
   static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
-  static constexpr int NT = 64 * WM * WN;       // threads per workgroup
-  static constexpr int FM = BM / 16 / WM;       // activation fragments per wave
-  static constexpr int FN = BN / 16 / WN;       // weight fragments per wave
-  static constexpr int XL = BM * 8 / NT;        // 16-byte chunks of the x slab per thread
-  static constexpr int WL = BN * 8 / NT;        // 16-byte chunks of the w slab per thread
+  static constexpr int NT = 64 * WM * WN;  // threads per workgroup
+  static constexpr int NW = NT / 64;
+  static constexpr int FM = BM / 16 / WM;  // activation fragments per wave
+  static constexpr int FN = BN / 16 / WN;  // weight fragments per wave
+  static constexpr int XI = BM / 8 / NW;   // slab-load instructions per wave (8 rows each), x
+  static constexpr int WI = BN / 8 / NW;   // same, w
   static constexpr int X_BYTES = BM * 128;
   static constexpr int W_BYTES = BN * 128;
   static constexpr int STAGE = X_BYTES + W_BYTES;
-  static_assert((NT / 8) % 16 == 0, "row step of the loader must keep the swizzle phase");
+  static constexpr int NLOAD = XI + WI;
+  static_assert(NW % 2 == 0, "swizzle phase of a wave's rows relies on an even wave count");
   static_assert(BM % (16 * WM) == 0 && BN % (16 * WN) == 0, "tile must split evenly over waves");
+  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "slab rows must split evenly over waves");
 };
 
-template <class C>
+// 64 lanes x 16 B from global memory straight into LDS: lane l's 16 bytes land at lds_addr + 16 l.
+// Issued from inline assembly so that the compiler does not serialise the in-flight slab against
+// the LDS reads of the slab being consumed; completion is tracked by hand with vmcnt.
+DEVINL void dma16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory");
+}
+// One dword per lane; used to pull 64 different cache lines towards L2 ahead of time.
+DEVINL void dma4(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory");
+}
+template <int N>
+DEVINL void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ long long g_clk[4];
+
+template <class C, int PF_DIST, int DBG = 0>
 __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
-  __shared__ __attribute__((aligned(16))) char lds[2 * C::STAGE];
+  __shared__ __attribute__((aligned(1024))) char lds[2 * C::STAGE];
+  __shared__ __attribute__((aligned(256))) char pf_sink[C::NW * 256];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t tile_off[MOE_GG_MAX_GROUPS + 1];
+  constexpr int NW = C::NW;
+  constexpr int NPF = PF_DIST > 0 ? (C::BM + C::BN + C::NT - 1) / C::NT : 0;  // prefetch instrs / wave / K step
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % C::WM;
   const int wn = wave / C::WM;
   const int K = p.K, N = p.N;
   const int n_tiles_n = moe_gg_cdiv(N, C::BN);
 
+  const long long dbg_c0 = __builtin_readcyclecounter(), dbg_w0 = wall_clock64();
   build_group_tables(p.m_sizes, p.G, p.M, C::BM, n_tiles_n, row_off, tile_off);
   const int total = tile_off[p.G];
   const int KT = K / 64;
 
-  // Loader geometry: chunk id = i * NT + tid -> (row, 16-byte chunk of the 128-byte row).
-  const int ld_row = tid >> 3, ld_c = tid & 7;
-  const int ld_lds = lds_swizzle_off(ld_row, ld_c);
-  // Fragment reads: row = frag * 16 + lane % 16, chunk = kk * 4 + lane / 16.
+  // Slab-load geometry: instruction i of wave w fills rows (i * NW + w) * 8 + lane / 8; the lane's
+  // physical 16-byte slot is lane % 8 and must hold logical chunk slot ^ ((row >> 1) & 7).
+  const int d_r = lane >> 3;
+  const int d_c = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const uint32_t lds_wave = lds_base + wave * 1024;
+  const uint32_t sink = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)pf_sink + wave * 256;
+
+  // Fragment reads: row = frag * 16 + lane % 16, chunk = kk * 4 + lane / 16 (swizzled).
   const int fr = lane & 15, fq = lane >> 4;
   const int rd0 = fr * 128 + ((fq ^ (fr >> 1)) << 4);  // kk = 0; kk = 1 is rd0 ^ 64
 
-  const bf16_t* __restrict__ xp = (const bf16_t*)p.x;
-  const bf16_t* __restrict__ wp = (const bf16_t*)p.w;
+  const char* xp = (const char*)p.x;
+  const char* wp = (const char*)p.w;
   bf16_t* __restrict__ yp = (bf16_t*)p.y;
 
   for (int round = 0; round * (int)gridDim.x < total; ++round) {
@@ -65,28 +107,46 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
     const int n0 = t.tn * C::BN;
     const int cols_valid = min(N - n0, C::BN);
 
-    const bf16_t* xg = xp + (int64_t)(t.row0 + m0) * K + ld_c * 8;
-    const bf16_t* wg = wp + ((int64_t)t.g * N + n0) * K + ld_c * 8;
-    int xoff[C::XL], woff[C::WL];
+    const char* xg = xp + (int64_t)(t.row0 + m0) * K * 2;
+    const char* wg = wp + ((int64_t)t.g * N + n0) * K * 2;
+    if (DBG == 2) { xg = xp; wg = wp; }
+    uint32_t xoff[C::XI], woff[C::WI];
 #pragma unroll
-    for (int i = 0; i < C::XL; ++i) xoff[i] = min(ld_row + i * (C::NT / 8), rows_valid - 1) * K;
+    for (int i = 0; i < C::XI; ++i)
+      xoff[i] = (uint32_t)min((i * NW + wave) * 8 + d_r, rows_valid - 1) * (uint32_t)(K * 2) + d_c * 16;
 #pragma unroll
-    for (int i = 0; i < C::WL; ++i) woff[i] = min(ld_row + i * (C::NT / 8), cols_valid - 1) * K;
+    for (int i = 0; i < C::WI; ++i)
+      woff[i] = (uint32_t)min((i * NW + wave) * 8 + d_r, cols_valid - 1) * (uint32_t)(K * 2) + d_c * 16;
 
-    u32x4_t xr[C::XL], wr[C::WL];
-    auto gload = [&](int kt) {
+    // Prefetch lanes: slab row r = tid + i * NT; rows < BM are x rows, the next BN are w rows.
+    uint32_t pf_off[NPF > 0 ? NPF : 1];
+    bool pf_is_x[NPF > 0 ? NPF : 1];
 #pragma unroll
-      for (int i = 0; i < C::XL; ++i) xr[i] = *(const u32x4_t*)(xg + xoff[i] + kt * 64);
+    for (int i = 0; i < NPF; ++i) {
+      const int r = tid + i * C::NT;
+      pf_is_x[i] = r < C::BM;
+      const int row = pf_is_x[i] ? min(r, rows_valid - 1) : min(min(r - C::BM, C::BN - 1), cols_valid - 1);
+      pf_off[i] = (uint32_t)row * (uint32_t)(K * 2);
+    }
+
+    auto dma = [&](int kt, int buf) {
+      if (DBG == 2) kt &= 15;
+      const char* xs = xg + kt * 128;
+      const char* ws = wg + kt * 128;
+      const uint32_t lb = lds_wave + buf * C::STAGE;
 #pragma unroll
-      for (int i = 0; i < C::WL; ++i) wr[i] = *(const u32x4_t*)(wg + woff[i] + kt * 64);
+      for (int i = 0; i < C::XI; ++i) dma16(xs, xoff[i], lb + i * NW * 1024);
+#pragma unroll
+      for (int i = 0; i < C::WI; ++i) dma16(ws, woff[i], lb + C::X_BYTES + i * NW * 1024);
     };
-    auto lstore = [&](int buf) {
-      char* xs = lds + buf * C::STAGE + ld_lds;
-      char* ws = xs + C::X_BYTES;
+    auto prefetch = [&](int kt) {
+      const int k = min(kt, KT - 1) * 128;
 #pragma unroll
-      for (int i = 0; i < C::XL; ++i) *(u32x4_t*)(xs + i * (C::NT / 8) * 128) = xr[i];
-#pragma unroll
-      for (int i = 0; i < C::WL; ++i) *(u32x4_t*)(ws + i * (C::NT / 8) * 128) = wr[i];
+      for (int i = 0; i < NPF; ++i) {
+        // x and w rows never share a wave when BM is a multiple of 64, so the base is wave-uniform
+        const char* base = __builtin_amdgcn_readfirstlane((int)pf_is_x[i]) ? xg : wg;
+        dma4(base + k, pf_off[i], sink);
+      }
     };
 
     f32x4_t acc[C::FN][C::FM];
@@ -95,32 +155,65 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
 #pragma unroll
       for (int i = 0; i < C::FM; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    gload(0);
-    lstore(0);
+    bf16x8_t wf0[C::FN], xf0[C::FM], wf1[C::FN], xf1[C::FM];
+    auto read_frags = [&](int buf, int kk, bf16x8_t (&wf)[C::FN], bf16x8_t (&xf)[C::FM]) {
+      const char* xs = lds + buf * C::STAGE + wm * (C::FM * 16 * 128);
+      const char* ws = lds + buf * C::STAGE + C::X_BYTES + wn * (C::FN * 16 * 128);
+      const int ro = kk ? (rd0 ^ 64) : rd0;
+#pragma unroll
+      for (int j = 0; j < C::FN; ++j) wf[j] = *(const bf16x8_t*)(ws + j * 2048 + ro);
+#pragma unroll
+      for (int i = 0; i < C::FM; ++i) xf[i] = *(const bf16x8_t*)(xs + i * 2048 + ro);
+    };
+    auto mma = [&](bf16x8_t (&wf)[C::FN], bf16x8_t (&xf)[C::FM]) {
+#pragma unroll
+      for (int j = 0; j < C::FN; ++j)
+#pragma unroll
+        for (int i = 0; i < C::FM; ++i)
+          acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[i], acc[j][i], 0, 0, 0);
+    };
+    // Ask the scheduler to spread the fragment reads of the next half over the MFMAs of this one.
+    auto interleave = [&]() {
+      constexpr int NR = C::FN + C::FM, NM = C::FN * C::FM;
+      constexpr int PER = NM / NR > 0 ? NM / NR : 1;
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * NR > 0 ? NM - PER * NR : 0, 0);
+    };
+
+    // Prologue: slabs 0 and 1 in flight, prefetch of the following ones, F0 <- (slab 0, half 0).
+    dma(0, 0);
+    if (KT > 1) dma(1, 1);
+    prefetch(2 + PF_DIST - 1);
+    if (KT > 1) wait_vmcnt<C::NLOAD + NPF>(); else wait_vmcnt<NPF>();
     __syncthreads();
+    read_frags(0, 0, wf0, xf0);
+    if (DBG == 4) read_frags(0, 1, wf1, xf1);
 
     for (int kt = 0; kt < KT; ++kt) {
       const int cur = kt & 1;
-      if (kt + 1 < KT) gload(kt + 1);
-      const char* xs = lds + cur * C::STAGE + wm * (C::FM * 16 * 128);
-      const char* ws = lds + cur * C::STAGE + C::X_BYTES + wn * (C::FN * 16 * 128);
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const int ro = kk ? (rd0 ^ 64) : rd0;
-        bf16x8_t wf[C::FN], xf[C::FM];
-#pragma unroll
-        for (int j = 0; j < C::FN; ++j) wf[j] = *(const bf16x8_t*)(ws + j * 2048 + ro);
-#pragma unroll
-        for (int i = 0; i < C::FM; ++i) xf[i] = *(const bf16x8_t*)(xs + i * 2048 + ro);
-#pragma unroll
-        for (int j = 0; j < C::FN; ++j)
-#pragma unroll
-          for (int i = 0; i < C::FM; ++i)
-            acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[i], acc[j][i], 0, 0, 0);
-      }
-      if (kt + 1 < KT) lstore(cur ^ 1);
-      __syncthreads();
+      if (DBG != 4) read_frags(cur, 1, wf1, xf1);
+      mma(wf0, xf0);
+      interleave();
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave has read all of slab kt
+      wait_vmcnt<NPF>();                                   // this wave's share of slab kt+1 has landed
+      if (DBG < 3) __syncthreads();
+      if ((DBG == 0 || DBG == 2) && kt + 2 < KT) dma(kt + 2, cur);
+      if (DBG == 0 || DBG == 2) prefetch(kt + 2 + PF_DIST);
+      __builtin_amdgcn_sched_barrier(0);
+      if (DBG != 4 && kt + 1 < KT) read_frags(cur ^ 1, 0, wf0, xf0);
+      mma(wf1, xf1);
+      interleave();
+      __builtin_amdgcn_sched_barrier(0);
     }
+    // All LDS reads of this tile were consumed by the MFMAs above; the next tile's prologue may
+    // overwrite both buffers only after every wave got here.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
 
     // Epilogue: lane holds y[m][n .. n+3] for m = frag_m * 16 + lane % 16, n = frag_n * 16 + 4 * (lane / 16).
     bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + (int64_t)t.g * p.col_block + n0;
@@ -148,11 +241,15 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
       }
     }
   }
+  if (DBG != 0 && blockIdx.x == 0 && threadIdx.x == 0) {
+    g_clk[0] = __builtin_readcyclecounter() - dbg_c0;
+    g_clk[1] = wall_clock64() - dbg_w0;
+  }
 }
 
-template <class C>
+template <class C, int PF, int DBG = 0>
 hipError_t launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  hipLaunchKernelGGL(gg_bf16_persistent<C>, dim3(num_wg), dim3(C::NT), 0, stream, p);
+  hipLaunchKernelGGL((gg_bf16_persistent<C, PF, DBG>), dim3(num_wg), dim3(C::NT), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -160,19 +257,32 @@ hipError_t launch(const GgParams& p, int num_wg, hipStream_t stream) {
 
 hipError_t gg_bf16_prefill_launch(const GgParams& p, int variant, int num_wg, hipStream_t stream) {
   switch (variant) {
-    case 0: return launch<Cfg<256, 256, 2, 2>>(p, num_wg, stream);
-    case 1: return launch<Cfg<256, 256, 2, 4>>(p, num_wg, stream);
-    case 2: return launch<Cfg<128, 256, 2, 2>>(p, num_wg, stream);
-    case 3: return launch<Cfg<128, 128, 2, 2>>(p, num_wg, stream);
-    case 4: return launch<Cfg<256, 128, 2, 2>>(p, num_wg, stream);
+    case 0: return launch<Cfg<256, 256, 2, 4>, 3>(p, num_wg, stream);
+    case 1: return launch<Cfg<256, 256, 2, 4>, 0>(p, num_wg, stream);
+    case 2: return launch<Cfg<256, 256, 2, 2>, 3>(p, num_wg, stream);
+    case 3: return launch<Cfg<256, 256, 2, 2>, 0>(p, num_wg, stream);
+    case 4: return launch<Cfg<256, 256, 4, 2>, 3>(p, num_wg, stream);
+    case 5: return launch<Cfg<128, 128, 2, 2>, 3>(p, num_wg, stream);
+    case 6: return launch<Cfg<256, 256, 2, 4>, 2>(p, num_wg, stream);
+    case 7: return launch<Cfg<256, 256, 2, 4>, 4>(p, num_wg, stream);
+    case 8: return launch<Cfg<256, 256, 2, 4>, 0, 1>(p, num_wg, stream);
+    case 9: return launch<Cfg<256, 256, 2, 4>, 0, 2>(p, num_wg, stream);
+    case 10: return launch<Cfg<256, 256, 2, 2>, 0, 1>(p, num_wg, stream);
+    case 11: return launch<Cfg<256, 256, 2, 2>, 0, 2>(p, num_wg, stream);
+    case 12: return launch<Cfg<256, 256, 2, 4>, 0, 3>(p, num_wg, stream);
+    case 13: return launch<Cfg<256, 256, 2, 4>, 0, 4>(p, num_wg, stream);
+    case 14: return launch<Cfg<256, 256, 2, 2>, 0, 3>(p, num_wg, stream);
+    case 15: return launch<Cfg<256, 256, 2, 2>, 0, 4>(p, num_wg, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
+void gg_debug_read_clock(long long* out) { (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_clk), 16); }
+
 int gg_bf16_prefill_block_m(int variant) {
   switch (variant) {
-    case 0: case 1: case 4: return 256;
-    case 2: case 3: return 128;
+    case 0: case 1: case 2: case 3: case 4: case 6: case 7: case 8: case 9: case 10: case 11: case 12: case 13: case 14: case 15: return 256;
+    case 5: return 128;
     default: return 0;
   }
 }

@@ -23,3 +23,6 @@ struct GgParams {
 hipError_t gg_bf16_prefill_launch(const GgParams& p, int variant, int num_wg, hipStream_t stream);
 int gg_bf16_prefill_block_m(int variant);
 hipError_t gg_bf16_generic_launch(const GgParams& p, hipStream_t stream);
+hipError_t gg_bf16_pingpong_launch(const GgParams& p, int variant, int num_wg, hipStream_t stream);
+void gg_debug_read_clock(long long* out);
+void gg_debug_read_ts(long long* out);
