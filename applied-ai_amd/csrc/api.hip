@@ -91,23 +91,28 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
 
   hipStream_t s = (hipStream_t)stream;
   const bool tiled_ok = K % 64 == 0 && aligned(x, 16) && aligned(w, 16);
-  if (!tiled_ok) return (int)gg_bf16_generic_launch(p, s);
-
   int variant = g_variant[MOE_GG_OP_GG_BF16].load();
-  if (variant < 0) variant = 0;
+  if (!tiled_ok || variant == MOE_GG_GG_GENERIC) return (int)gg_bf16_generic_launch(p, s);
+
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
-  if (variant >= 20) return (int)gg_bf16_pingpong_launch(p, variant - 20, num_wg, s);
-  if (gg_bf16_prefill_block_m(variant) == 0) return MOE_GG_EINVAL;
-  return (int)gg_bf16_prefill_launch(p, variant, num_wg, s);
-}
-
-int moe_gg_debug_read_ts(long long* out256) { gg_debug_read_ts(out256); return 0; }
-
-int moe_gg_debug_read_clock(long long* cycles_and_100mhz_ticks) {
-  if (!cycles_and_100mhz_ticks) return MOE_GG_EINVAL;
-  gg_debug_read_clock(cycles_and_100mhz_ticks);
-  return MOE_GG_OK;
+  if (variant < 0) {
+    // m_sizes lives on the device and is never copied back, so the tile shape is picked from the
+    // average rows per expert and a rough tile count (each expert adds about half a partial tile).
+    const int64_t avg = M / G;
+    const int64_t t256 = (M / 256 + (G + 1) / 2) * ((N + 255) / 256);
+    const int64_t t128 = (M / 128 + (G + 1) / 2) * ((N + 127) / 128);
+    if (avg >= 160 && t256 * 4 >= (int64_t)num_wg * 3) variant = MOE_GG_GG_PINGPONG_256;
+    else if (avg >= 80 && t128 * 2 >= num_wg) variant = MOE_GG_GG_TILED_128;
+    else variant = MOE_GG_GG_TILED_64;
+  }
+  switch (variant) {
+    case MOE_GG_GG_PINGPONG_256: return (int)gg_bf16_pingpong_launch(p, num_wg, s);
+    case MOE_GG_GG_TILED_256: return (int)gg_bf16_tiled_launch(p, 256, num_wg, s);
+    case MOE_GG_GG_TILED_128: return (int)gg_bf16_tiled_launch(p, 128, num_wg, s);
+    case MOE_GG_GG_TILED_64: return (int)gg_bf16_tiled_launch(p, 64, num_wg, s);
+    default: return MOE_GG_EINVAL;
+  }
 }
 
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,

@@ -11,8 +11,10 @@
 // K loop (one barrier per 64-wide K step): the fragments of the two 32-wide halves of a K step live
 // in two register sets F0/F1. While the MFMAs of one half run, the ds_reads of the next half are in
 // flight; the barrier in the middle of the step both publishes slab kt+1 and frees slab kt's buffer,
-// into which the loads of slab kt+2 are issued at once. A one-dword-per-line load into a scratch LDS
-// area runs PF_DIST steps ahead so that the slab loads hit in L2 instead of waiting for HBM.
+// into which the loads of slab kt+2 are issued at once.
+//
+// This is the general tiled kernel (tile shapes 256x256, 128x128 and 64x128); the 256x256 ping-pong
+// kernel in gg_bf16_pp.hip is preferred when a launch has enough 256x256 tiles to fill the chip.
 #include "common.h"
 #include "gg_tables.h"
 #include "kernels.h"
@@ -46,28 +48,17 @@ DEVINL void dma16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
                : "s"(lds_addr), "v"(voff), "s"(sbase)
                : "memory");
 }
-// One dword per lane; used to pull 64 different cache lines towards L2 ahead of time.
-DEVINL void dma4(const void* sbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n"
-               :
-               : "s"(lds_addr), "v"(voff), "s"(sbase)
-               : "memory");
-}
 template <int N>
 DEVINL void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-__device__ long long g_clk[4];
-
-template <class C, int PF_DIST, int DBG = 0>
+template <class C>
 __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[2 * C::STAGE];
-  __shared__ __attribute__((aligned(256))) char pf_sink[C::NW * 256];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t tile_off[MOE_GG_MAX_GROUPS + 1];
   constexpr int NW = C::NW;
-  constexpr int NPF = PF_DIST > 0 ? (C::BM + C::BN + C::NT - 1) / C::NT : 0;  // prefetch instrs / wave / K step
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -77,7 +68,6 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
   const int K = p.K, N = p.N;
   const int n_tiles_n = moe_gg_cdiv(N, C::BN);
 
-  const long long dbg_c0 = __builtin_readcyclecounter(), dbg_w0 = wall_clock64();
   build_group_tables(p.m_sizes, p.G, p.M, C::BM, n_tiles_n, row_off, tile_off);
   const int total = tile_off[p.G];
   const int KT = K / 64;
@@ -88,7 +78,6 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
   const int d_c = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
   const uint32_t lds_wave = lds_base + wave * 1024;
-  const uint32_t sink = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)pf_sink + wave * 256;
 
   // Fragment reads: row = frag * 16 + lane % 16, chunk = kk * 4 + lane / 16 (swizzled).
   const int fr = lane & 15, fq = lane >> 4;
@@ -109,7 +98,6 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
 
     const char* xg = xp + (int64_t)(t.row0 + m0) * K * 2;
     const char* wg = wp + ((int64_t)t.g * N + n0) * K * 2;
-    if (DBG == 2) { xg = xp; wg = wp; }
     uint32_t xoff[C::XI], woff[C::WI];
 #pragma unroll
     for (int i = 0; i < C::XI; ++i)
@@ -118,19 +106,7 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
     for (int i = 0; i < C::WI; ++i)
       woff[i] = (uint32_t)min((i * NW + wave) * 8 + d_r, cols_valid - 1) * (uint32_t)(K * 2) + d_c * 16;
 
-    // Prefetch lanes: slab row r = tid + i * NT; rows < BM are x rows, the next BN are w rows.
-    uint32_t pf_off[NPF > 0 ? NPF : 1];
-    bool pf_is_x[NPF > 0 ? NPF : 1];
-#pragma unroll
-    for (int i = 0; i < NPF; ++i) {
-      const int r = tid + i * C::NT;
-      pf_is_x[i] = r < C::BM;
-      const int row = pf_is_x[i] ? min(r, rows_valid - 1) : min(min(r - C::BM, C::BN - 1), cols_valid - 1);
-      pf_off[i] = (uint32_t)row * (uint32_t)(K * 2);
-    }
-
     auto dma = [&](int kt, int buf) {
-      if (DBG == 2) kt &= 15;
       const char* xs = xg + kt * 128;
       const char* ws = wg + kt * 128;
       const uint32_t lb = lds_wave + buf * C::STAGE;
@@ -139,16 +115,6 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
 #pragma unroll
       for (int i = 0; i < C::WI; ++i) dma16(ws, woff[i], lb + C::X_BYTES + i * NW * 1024);
     };
-    auto prefetch = [&](int kt) {
-      const int k = min(kt, KT - 1) * 128;
-#pragma unroll
-      for (int i = 0; i < NPF; ++i) {
-        // x and w rows never share a wave when BM is a multiple of 64, so the base is wave-uniform
-        const char* base = __builtin_amdgcn_readfirstlane((int)pf_is_x[i]) ? xg : wg;
-        dma4(base + k, pf_off[i], sink);
-      }
-    };
-
     f32x4_t acc[C::FN][C::FM];
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
@@ -184,28 +150,25 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
       __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * NR > 0 ? NM - PER * NR : 0, 0);
     };
 
-    // Prologue: slabs 0 and 1 in flight, prefetch of the following ones, F0 <- (slab 0, half 0).
+    // Prologue: slabs 0 and 1 in flight, F0 <- (slab 0, half 0).
     dma(0, 0);
     if (KT > 1) dma(1, 1);
-    prefetch(2 + PF_DIST - 1);
-    if (KT > 1) wait_vmcnt<C::NLOAD + NPF>(); else wait_vmcnt<NPF>();
+    if (KT > 1) wait_vmcnt<C::NLOAD>(); else wait_vmcnt<0>();
     __syncthreads();
     read_frags(0, 0, wf0, xf0);
-    if (DBG == 4) read_frags(0, 1, wf1, xf1);
 
     for (int kt = 0; kt < KT; ++kt) {
       const int cur = kt & 1;
-      if (DBG != 4) read_frags(cur, 1, wf1, xf1);
+      read_frags(cur, 1, wf1, xf1);
       mma(wf0, xf0);
       interleave();
       __builtin_amdgcn_sched_barrier(0);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave has read all of slab kt
-      wait_vmcnt<NPF>();                                   // this wave's share of slab kt+1 has landed
-      if (DBG < 3) __syncthreads();
-      if ((DBG == 0 || DBG == 2) && kt + 2 < KT) dma(kt + 2, cur);
-      if (DBG == 0 || DBG == 2) prefetch(kt + 2 + PF_DIST);
+      wait_vmcnt<0>();                                     // this wave's share of slab kt+1 has landed
+      __syncthreads();
+      if (kt + 2 < KT) dma(kt + 2, cur);
       __builtin_amdgcn_sched_barrier(0);
-      if (DBG != 4 && kt + 1 < KT) read_frags(cur ^ 1, 0, wf0, xf0);
+      if (kt + 1 < KT) read_frags(cur ^ 1, 0, wf0, xf0);
       mma(wf1, xf1);
       interleave();
       __builtin_amdgcn_sched_barrier(0);
@@ -241,48 +204,23 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
       }
     }
   }
-  if (DBG != 0 && blockIdx.x == 0 && threadIdx.x == 0) {
-    g_clk[0] = __builtin_readcyclecounter() - dbg_c0;
-    g_clk[1] = wall_clock64() - dbg_w0;
-  }
 }
 
-template <class C, int PF, int DBG = 0>
+template <class C>
 hipError_t launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  hipLaunchKernelGGL((gg_bf16_persistent<C, PF, DBG>), dim3(num_wg), dim3(C::NT), 0, stream, p);
+  hipLaunchKernelGGL((gg_bf16_persistent<C>), dim3(num_wg), dim3(C::NT), 0, stream, p);
   return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t gg_bf16_prefill_launch(const GgParams& p, int variant, int num_wg, hipStream_t stream) {
-  switch (variant) {
-    case 0: return launch<Cfg<256, 256, 2, 4>, 3>(p, num_wg, stream);
-    case 1: return launch<Cfg<256, 256, 2, 4>, 0>(p, num_wg, stream);
-    case 2: return launch<Cfg<256, 256, 2, 2>, 3>(p, num_wg, stream);
-    case 3: return launch<Cfg<256, 256, 2, 2>, 0>(p, num_wg, stream);
-    case 4: return launch<Cfg<256, 256, 4, 2>, 3>(p, num_wg, stream);
-    case 5: return launch<Cfg<128, 128, 2, 2>, 3>(p, num_wg, stream);
-    case 6: return launch<Cfg<256, 256, 2, 4>, 2>(p, num_wg, stream);
-    case 7: return launch<Cfg<256, 256, 2, 4>, 4>(p, num_wg, stream);
-    case 8: return launch<Cfg<256, 256, 2, 4>, 0, 1>(p, num_wg, stream);
-    case 9: return launch<Cfg<256, 256, 2, 4>, 0, 2>(p, num_wg, stream);
-    case 10: return launch<Cfg<256, 256, 2, 2>, 0, 1>(p, num_wg, stream);
-    case 11: return launch<Cfg<256, 256, 2, 2>, 0, 2>(p, num_wg, stream);
-    case 12: return launch<Cfg<256, 256, 2, 4>, 0, 3>(p, num_wg, stream);
-    case 13: return launch<Cfg<256, 256, 2, 4>, 0, 4>(p, num_wg, stream);
-    case 14: return launch<Cfg<256, 256, 2, 2>, 0, 3>(p, num_wg, stream);
-    case 15: return launch<Cfg<256, 256, 2, 2>, 0, 4>(p, num_wg, stream);
+hipError_t gg_bf16_tiled_launch(const GgParams& p, int block_m, int num_wg, hipStream_t stream) {
+  switch (block_m) {
+    case 256: return launch<Cfg<256, 256, 2, 4>>(p, num_wg, stream);
+    case 128: return launch<Cfg<128, 128, 2, 2>>(p, num_wg, stream);
+    case 64: return launch<Cfg<64, 128, 2, 2>>(p, num_wg, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
-void gg_debug_read_clock(long long* out) { (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_clk), 16); }
-
-int gg_bf16_prefill_block_m(int variant) {
-  switch (variant) {
-    case 0: case 1: case 2: case 3: case 4: case 6: case 7: case 8: case 9: case 10: case 11: case 12: case 13: case 14: case 15: return 256;
-    case 5: return 128;
-    default: return 0;
-  }
-}
+int gg_bf16_tiled_block_n(int block_m) { return block_m == 256 ? 256 : 128; }

@@ -20,9 +20,9 @@ struct GgParams {
   int xcds;       // number of XCDs the persistent grid is spread over
 };
 
-hipError_t gg_bf16_prefill_launch(const GgParams& p, int variant, int num_wg, hipStream_t stream);
-int gg_bf16_prefill_block_m(int variant);
+// block_m in {256, 128, 64}; the matching tile width is gg_bf16_tiled_block_n(block_m).
+hipError_t gg_bf16_tiled_launch(const GgParams& p, int block_m, int num_wg, hipStream_t stream);
+int gg_bf16_tiled_block_n(int block_m);
+// 256 x 256 tiles, ping-pong schedule.
+hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream);
 hipError_t gg_bf16_generic_launch(const GgParams& p, hipStream_t stream);
-hipError_t gg_bf16_pingpong_launch(const GgParams& p, int variant, int num_wg, hipStream_t stream);
-void gg_debug_read_clock(long long* out);
-void gg_debug_read_ts(long long* out);

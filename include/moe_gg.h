@@ -68,6 +68,12 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
  * tiles written (<= max_tiles), or a negative error.
  */
 #define MOE_GG_OP_GG_BF16 0
+/* variants of MOE_GG_OP_GG_BF16 */
+#define MOE_GG_GG_PINGPONG_256 0 /* 256x256 tiles, two wave groups alternating load / MFMA phases */
+#define MOE_GG_GG_TILED_256 1    /* 256x256 tiles, all waves in step */
+#define MOE_GG_GG_TILED_128 2    /* 128x128 tiles */
+#define MOE_GG_GG_TILED_64 3     /* 64x128 tiles */
+#define MOE_GG_GG_GENERIC 4      /* one thread per output element, any shape / alignment */
 int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,
