@@ -96,6 +96,16 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
 
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
+  const bool decode_ok = K % 128 == 0;
+  if (variant < 0 && decode_ok && M <= (int64_t)G * 40) variant = MOE_GG_GG_DECODE;
+  if (variant == MOE_GG_GG_DECODE) {
+    if (!decode_ok) return MOE_GG_EUNSUPPORTED;
+    const int64_t avg = (M + G - 1) / G;
+    const int mf = avg <= 10 ? 1 : (avg <= 24 ? 2 : 4);
+    int nf = ((int64_t)(N / 64) * G >= 4 * (int64_t)di->cus) ? 4 : 2;
+    if (mf == 4) nf = 2;
+    return (int)gg_bf16_decode_launch(p, nf, mf, s);
+  }
   if (variant < 0) {
     // m_sizes lives on the device and is never copied back, so the tile shape is picked from the
     // average rows per expert and a rough tile count (each expert adds about half a partial tile).

@@ -1,0 +1,147 @@
+// Small-M ("decode") bf16 grouped GEMM for gfx950: split-K inside the workgroup, weights streamed once.
+//
+// Same contract as the reference's _kernel_grouped_gemm (dev/triton_groupGEMM/groupgemm.py:130-254):
+// y[off_g : off_g + m_g, :] = x[off_g : ...] @ w[g]^T, but built for m_g of a few rows per expert,
+// where the time is the time to stream the active experts' weights from HBM once. The split-K
+// decode configurations of the reference's fused-MoE kernels are the model
+// (kernels/triton/inference/col_major_moe_gemm/v1_moe_fused.py:297-312).
+//
+// Grid: (N / (16 * NF), G). A workgroup owns 16 * NF weight rows of one expert and all of the
+// expert's (<= 16 * MF per pass) activation rows; its four waves split K four ways. Each wave loads
+// its weight fragments straight from global memory into the MFMA "A" operand layout (lane l holds
+// row l % 16, 16 bytes of K chunk l / 16 -> two consecutive K steps consume one 128-byte line per
+// row) with DEPTH K steps of loads in flight, multiplies them with the activation fragments
+// ("B" operand, L2-resident) by v_mfma_f32_16x16x32_bf16, and the four partial accumulators are
+// summed through LDS (fixed order: deterministic) before the bf16 store. Experts with m_g = 0 exit
+// at once, so their weights are never touched.
+#include "common.h"
+#include "kernels.h"
+#include "tile_sched.h"
+
+namespace {
+
+template <int NF, int MF, int WAVES, int DEPTH>
+__global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
+  __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MF][256];
+  __shared__ int s_row0, s_rows;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int g = blockIdx.y;
+  const int K = p.K, N = p.N;
+
+  // Row range of expert g: prefix sum of m_sizes[0 .. g) (clamped like tile_sched.h does).
+  if (wave == 0) {
+    long long s = 0;
+    for (int i = lane; i < g; i += 64) {
+      int m = p.m_sizes[i];
+      s += m < 0 ? 0 : (m > p.M ? p.M : m);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
+    if (lane == 0) {
+      const long long r0 = s > p.M ? p.M : s;
+      s_row0 = (int)r0;
+      s_rows = moe_gg_clamp_rows(p.m_sizes[g], r0, p.M);
+    }
+  }
+  __syncthreads();
+  const int row0 = s_row0, rows = s_rows;
+  if (rows == 0) return;
+
+  const int n0 = blockIdx.x * (16 * NF);
+  const int fr = lane & 15, fq = lane >> 4;
+  const int kw = K / WAVES;            // K range of this wave
+  const int steps = kw / 32;
+  const bf16_t* wbase = (const bf16_t*)p.w + ((int64_t)g * N + n0) * K + wave * kw + fq * 8;
+  const bf16_t* xbase = (const bf16_t*)p.x + (int64_t)row0 * K + wave * kw + fq * 8;
+  int64_t woff[NF];
+#pragma unroll
+  for (int j = 0; j < NF; ++j) woff[j] = (int64_t)min(j * 16 + fr, N - n0 - 1) * K;
+
+  for (int mb = 0; mb < rows; mb += 16 * MF) {  // one pass unless the expert has more than 16 * MF rows
+    int64_t xoff[MF];
+#pragma unroll
+    for (int i = 0; i < MF; ++i) xoff[i] = (int64_t)min(mb + i * 16 + fr, rows - 1) * K;
+
+    f32x4_t acc[NF][MF];
+#pragma unroll
+    for (int j = 0; j < NF; ++j)
+#pragma unroll
+      for (int i = 0; i < MF; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    bf16x8_t wb[DEPTH][NF], xb[DEPTH][MF];
+    auto load = [&](int d, int t) {
+#pragma unroll
+      for (int j = 0; j < NF; ++j) wb[d][j] = *(const bf16x8_t*)(wbase + woff[j] + t * 32);
+#pragma unroll
+      for (int i = 0; i < MF; ++i) xb[d][i] = *(const bf16x8_t*)(xbase + xoff[i] + t * 32);
+    };
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (d < steps) load(d, d);
+    for (int t0 = 0; t0 < steps; t0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        if (t0 + d < steps) {
+#pragma unroll
+          for (int j = 0; j < NF; ++j)
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+              acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[d][j], xb[d][i], acc[j][i], 0, 0, 0);
+          if (t0 + d + DEPTH < steps) load(d, t0 + d + DEPTH);
+        }
+      }
+    }
+
+    // Split-K reduction through LDS, then the store: lane holds y[m][n .. n+3] for
+    // m = mb + i * 16 + lane % 16, n = n0 + j * 16 + 4 * (lane / 16).
+#pragma unroll
+    for (int j = 0; j < NF; ++j)
+#pragma unroll
+      for (int i = 0; i < MF; ++i) *(f32x4_t*)&red[wave][j * MF + i][lane * 4] = acc[j][i];
+    __syncthreads();
+    for (int f = wave; f < NF * MF; f += WAVES) {
+      f32x4_t v = *(const f32x4_t*)&red[0][f][lane * 4];
+#pragma unroll
+      for (int w2 = 1; w2 < WAVES; ++w2) v += *(const f32x4_t*)&red[w2][f][lane * 4];
+      const int j = f / MF, i = f % MF;
+      const int m = mb + i * 16 + fr;
+      const int n = n0 + j * 16 + fq * 4;
+      if (m < rows) {
+        bf16_t* yrow = (bf16_t*)p.y + (int64_t)(row0 + m) * p.ldy + (int64_t)g * p.col_block;
+        if (p.vec_store && n + 3 < N) {
+          u32x2_t o;
+          o[0] = pack_bf16x2(v[0], v[1]);
+          o[1] = pack_bf16x2(v[2], v[3]);
+          *(u32x2_t*)(yrow + n) = o;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < N) yrow[n + r] = (bf16_t)v[r];
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <int NF, int MF, int DEPTH>
+hipError_t launch(const GgParams& p, hipStream_t stream) {
+  dim3 grid((p.N + 16 * NF - 1) / (16 * NF), p.G);
+  hipLaunchKernelGGL((gg_bf16_decode<NF, MF, 4, DEPTH>), grid, dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+// nf: 16-row weight fragments per wave (2 or 4); mf: 16-row activation fragments per pass (1, 2, 4).
+hipError_t gg_bf16_decode_launch(const GgParams& p, int nf, int mf, hipStream_t stream) {
+  if (nf == 2 && mf == 1) return launch<2, 1, 8>(p, stream);
+  if (nf == 4 && mf == 1) return launch<4, 1, 4>(p, stream);
+  if (nf == 2 && mf == 2) return launch<2, 2, 8>(p, stream);
+  if (nf == 4 && mf == 2) return launch<4, 2, 4>(p, stream);
+  if (nf == 2 && mf == 4) return launch<2, 4, 4>(p, stream);
+  return hipErrorInvalidValue;
+}

@@ -26,3 +26,6 @@ int gg_bf16_tiled_block_n(int block_m);
 // 256 x 256 tiles, ping-pong schedule.
 hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream);
 hipError_t gg_bf16_generic_launch(const GgParams& p, hipStream_t stream);
+// Small-M split-K kernel; nf = 16-row weight fragments per wave (2 or 4), mf = 16-row activation
+// fragments per pass (1, 2 or 4). Needs K % 128 == 0 and 16-byte aligned x and w.
+hipError_t gg_bf16_decode_launch(const GgParams& p, int nf, int mf, hipStream_t stream);

@@ -74,6 +74,7 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
 #define MOE_GG_GG_TILED_128 2    /* 128x128 tiles */
 #define MOE_GG_GG_TILED_64 3     /* 64x128 tiles */
 #define MOE_GG_GG_GENERIC 4      /* one thread per output element, any shape / alignment */
+#define MOE_GG_GG_DECODE 5       /* small-M path: weights streamed once, split-K inside the workgroup */
 int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,
