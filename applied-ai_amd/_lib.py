@@ -26,6 +26,11 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_i64, _c_int,
          _c_void_p],
     ),
+    "moe_gg_w4a16_splitk": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_void_p],
+    ),
     "moe_gg_host_enumerate_tiles": (
         _c_int,
         [_i32_p, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _i32_p, _c_int],

@@ -125,6 +125,25 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
   }
 }
 
+int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                        void* c, int M, int N, int K, int group_size, int zero_offset, int dtype,
+                        void* stream) {
+  if (M < 0 || N < 0 || K < 0 || group_size <= 0) return MOE_GG_EINVAL;
+  if (zero_offset != 0 && zero_offset != 1) return MOE_GG_EINVAL;
+  if (dtype != MOE_GG_DTYPE_BF16 && dtype != MOE_GG_DTYPE_FP16) return MOE_GG_EINVAL;
+  if (M == 0 || N == 0) return MOE_GG_OK;
+  if (!a || !qweight || !scales || !qzeros || !c) return MOE_GG_EINVAL;
+  if (K == 0 || K % group_size != 0 || K % 8 != 0 || N % 8 != 0) return MOE_GG_ESHAPE;
+  if (group_size % 32 != 0 || N % 64 != 0) return MOE_GG_EUNSUPPORTED;
+  if (!aligned(a, 16) || !aligned(qweight, 16) || !aligned(scales, 16) || !aligned(qzeros, 8) || !aligned(c, 2))
+    return MOE_GG_EALIGN;
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != MOE_GG_OK) return rc;
+  W4Params p{a, qweight, scales, qzeros, c, M, N, K, group_size, zero_offset};
+  return (int)w4a16_splitk_launch(p, dtype == MOE_GG_DTYPE_FP16, (hipStream_t)stream);
+}
+
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,
                                 int max_tiles) {

@@ -29,3 +29,16 @@ hipError_t gg_bf16_generic_launch(const GgParams& p, hipStream_t stream);
 // Small-M split-K kernel; nf = 16-row weight fragments per wave (2 or 4), mf = 16-row activation
 // fragments per pass (1, 2 or 4). Needs K % 128 == 0 and 16-byte aligned x and w.
 hipError_t gg_bf16_decode_launch(const GgParams& p, int nf, int mf, hipStream_t stream);
+
+// W4A16 split-K dequant GEMM (w4a16.hip). a, scales, c share one 16-bit float type.
+struct W4Params {
+  const void* a;           // [M, K]
+  const int32_t* qweight;  // [K/8, N]
+  const void* scales;      // [K/group_size, N]
+  const int32_t* qzeros;   // [K/group_size, N/8]
+  void* c;                 // [M, N]
+  int M, N, K;
+  int group_size;
+  int zero_offset;
+};
+hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream);

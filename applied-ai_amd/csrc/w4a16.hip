@@ -1,0 +1,338 @@
+// W4A16 split-K dequant GEMM for gfx950: c[M, N] = a[M, K] @ dequant(qweight, scales, qzeros).
+//
+// Replaces matmul_split_k / matmul_split_k_kernel
+// (kernels/triton/inference/gptq/splitk_dequant_gemm.py:91-141, 23-89). Data layout as there:
+//   qweight [K/8, N] int32, nibble j of a word = row 8*i + j            (:56, :76)
+//   scales  [K/group, N] (same 16-bit float type as a)
+//   qzeros  [K/group, N/8] int32, nibble j of a word = column 8*i + j   (:57, :70)
+//   w(k, n) = (q(k, n) - (z(g, n) + zero_offset)) * s(g, n),  g = k / group   (:73-77)
+//
+// A workgroup of eight waves owns 64 output columns; the waves split K by quantisation group
+// (wave w takes groups w, w+8, ...: the interleaved K split of the reference, :45,80-81) and their
+// partial sums are added through LDS in a fixed order, so no atomics, no zero-initialised output and
+// bit-identical results run to run.
+//
+// Per 32-wide K step a lane loads one dwordx4 of qweight: 4 adjacent columns x 8 consecutive k.
+// Word j becomes the MFMA "A" fragment of column n0 + 4*(lane%16) + j without any arithmetic:
+// ((word >> 4t) & 0x000F000F) | MAGIC puts nibble t in the low and nibble t+4 in the high half of a
+// dword as the floats BIAS + q (BIAS = 128 for bf16, 1024 for fp16, exact). The activation fragment is
+// permuted to the same k order (0,4,1,5,2,6,3,7). One extra MFMA per step with an all-ones A fragment
+// gives S = sum_k x[k]; after each group the lane folds scale and zero point in fp32:
+//   total += s * (acc_group - (BIAS + z + zero_offset) * S).
+// With the four words of a lane feeding four MFMAs, a lane ends up with 16 consecutive output
+// columns of one output row.
+#include "common.h"
+#include "kernels.h"
+
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+
+template <bool FP16>
+struct Elem;
+template <>
+struct Elem<false> {  // bf16
+  static constexpr uint32_t MAGIC = 0x43004300u;  // 128.0 | 128.0
+  static constexpr uint32_t ONES = 0x3F803F80u;
+  static constexpr float BIAS = 128.f;
+  static DEVINL f32x4_t mfma(u32x4_t a, u32x4_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+  static DEVINL float to_f32(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
+  static DEVINL uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+};
+template <>
+struct Elem<true> {  // fp16
+  static constexpr uint32_t MAGIC = 0x64006400u;  // 1024.0 | 1024.0
+  static constexpr uint32_t ONES = 0x3C003C00u;
+  static constexpr float BIAS = 1024.f;
+  static DEVINL f32x4_t mfma(u32x4_t a, u32x4_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+  static DEVINL float to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+  static DEVINL uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+};
+
+constexpr int WAVES = 8;
+constexpr int DEPTH = 8;  // K steps of qweight loads in flight per wave
+
+// Any group size that is a multiple of 32; scales / zeros are loaded where they are used.
+template <bool FP16, int MF>
+__global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) {
+  using E = Elem<FP16>;
+  __shared__ __attribute__((aligned(16))) float red[WAVES][MF][64 * 16];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int fr = lane & 15, fq = lane >> 4;
+  const int N = p.N, K = p.K, M = p.M;
+  const int n0 = blockIdx.x * 64;
+  const int spg = p.group_size / 32;               // K steps per quantisation group
+  const int ngroups = K / p.group_size;
+  const int my_groups = ngroups > wave ? (ngroups - wave + WAVES - 1) / WAVES : 0;
+  const int steps = my_groups * spg;               // K steps of this wave
+
+  // step t of this wave -> absolute K step
+  auto kstep = [&](int t) { return ((t / spg) * WAVES + wave) * spg + t % spg; };
+
+  // qweight: lane reads words of columns n0 + 4*fr .. + 3 (clamped at the right edge), k-word row 4*step + fq
+  const int wcol = min(n0 + 4 * fr, N - 4);
+  const int32_t* qw = p.qweight + wcol;
+  // output / scale columns of this lane: n0 + 16*fq + 0..15
+  const int ocol = n0 + 16 * fq;
+  const int ocol_c = min(ocol, N - 16 >= 0 ? N - 16 : 0);
+
+  for (int mb = 0; mb < M; mb += 16 * MF) {
+    const uint16_t* arow[MF];
+#pragma unroll
+    for (int i = 0; i < MF; ++i) arow[i] = (const uint16_t*)p.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
+
+    f32x4_t total[MF][4];  // [m fragment][j]: rows n-local 4*ii + j ... see epilogue
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) total[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    u32x4_t wb[DEPTH];
+    auto loadw = [&](int d, int t) { wb[d] = *(const u32x4_t*)(qw + (int64_t)(kstep(t) * 4 + fq) * N); };
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (d < steps) loadw(d, d);
+
+    f32x4_t accg[MF][4], accs[MF];
+    for (int t0 = 0; t0 < steps; t0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int t = t0 + d;
+        if (t < steps) {
+          if (t % spg == 0) {
+#pragma unroll
+            for (int i = 0; i < MF; ++i) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) accg[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+              accs[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            }
+          }
+          const int ks = kstep(t);
+          // activation fragments, permuted to the k order the nibble unpack produces
+          u32x4_t xb[MF];
+#pragma unroll
+          for (int i = 0; i < MF; ++i) {
+            const u32x4_t v = *(const u32x4_t*)(arow[i] + ks * 32);
+            xb[i][0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // k 0, 4
+            xb[i][1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // k 1, 5
+            xb[i][2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // k 2, 6
+            xb[i][3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // k 3, 7
+          }
+          const u32x4_t w4 = wb[d];
+          if (t + DEPTH < steps) loadw(d, t + DEPTH);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            u32x4_t af;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) af[e] = ((w4[j] >> (4 * e)) & 0x000F000Fu) | E::MAGIC;
+#pragma unroll
+            for (int i = 0; i < MF; ++i) accg[i][j] = E::mfma(af, xb[i], accg[i][j]);
+          }
+          const u32x4_t ones = {E::ONES, E::ONES, E::ONES, E::ONES};
+#pragma unroll
+          for (int i = 0; i < MF; ++i) accs[i] = E::mfma(ones, xb[i], accs[i]);
+
+          if (t % spg == spg - 1) {
+            // fold scale and zero point of this group: lane's columns are ocol + 4*ii + j
+            const int g = ks / spg;
+            const u32x4_t s0 = *(const u32x4_t*)((const uint16_t*)p.scales + (int64_t)g * N + ocol_c);
+            const u32x4_t s1 = *(const u32x4_t*)((const uint16_t*)p.scales + (int64_t)g * N + ocol_c + 8);
+            const u32x2_t zw = *(const u32x2_t*)(p.qzeros + (int64_t)g * (N / 8) + ocol_c / 8);
+#pragma unroll
+            for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const int c = 4 * ii + j;  // column offset inside the lane's 16
+                const uint32_t sw = c < 8 ? s0[c >> 1] : s1[(c - 8) >> 1];
+                const float s = E::to_f32((uint16_t)((c & 1) ? (sw >> 16) : (sw & 0xFFFFu)));
+                const uint32_t z = (zw[c >> 3] >> (4 * (c & 7))) & 0xFu;
+                const float zz = E::BIAS + (float)(int)(z + (uint32_t)p.zero_offset);
+#pragma unroll
+                for (int i = 0; i < MF; ++i) total[i][j][ii] += s * (accg[i][j][ii] - zz * accs[i][ii]);
+              }
+          }
+        }
+      }
+    }
+
+    // Cross-wave (split-K) reduction, fixed order. red[wave][i][(m_local * 64) + col_local]
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii) red[wave][i][fr * 64 + 16 * fq + 4 * ii + j] = total[i][j][ii];
+    __syncthreads();
+    for (int o = tid; o < MF * 16 * 64; o += 64 * WAVES) {
+      const int i = o / 1024, rem = o % 1024;
+      const int m = mb + i * 16 + rem / 64, n = n0 + rem % 64;
+      float v = red[0][i][rem];
+#pragma unroll
+      for (int w2 = 1; w2 < WAVES; ++w2) v += red[w2][i][rem];
+      if (m < M && n < N) ((uint16_t*)p.c)[(int64_t)m * N + n] = E::from_f32(v);
+    }
+    __syncthreads();
+  }
+}
+
+// group_size == 128 (four K steps per group). Every load - qweight, activations, scales, zeros - is
+// issued two groups (eight K steps) ahead of its use and consumed in issue order, because vector
+// memory loads return in order: a late-issued small load would otherwise wait for all the weight
+// loads queued before it.
+template <bool FP16, int MF, int GA>  // GA = groups kept in flight
+__global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_g128(W4Params p) {
+  using E = Elem<FP16>;
+  constexpr int SPG = 4, D = SPG * GA;
+  __shared__ __attribute__((aligned(16))) float red[WAVES][MF][64 * 16];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int fr = lane & 15, fq = lane >> 4;
+  const int N = p.N, K = p.K, M = p.M;
+  const int n0 = blockIdx.x * 64;
+  const int ngroups = K / 128;
+  const int my_groups = ngroups > wave ? (ngroups - wave + WAVES - 1) / WAVES : 0;
+  const int steps = my_groups * SPG;
+  auto kstep = [&](int t) { return ((t / SPG) * WAVES + wave) * SPG + t % SPG; };
+
+  const int32_t* qw = p.qweight + n0 + 4 * fr;
+  const int ocol = n0 + 16 * fq;
+  const uint16_t* sc = (const uint16_t*)p.scales + ocol;
+  const int32_t* zp = p.qzeros + ocol / 8;
+
+  for (int mb = 0; mb < M; mb += 16 * MF) {
+    const uint16_t* arow[MF];
+#pragma unroll
+    for (int i = 0; i < MF; ++i) arow[i] = (const uint16_t*)p.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
+
+    f32x4_t total[MF][4];
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) total[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    u32x4_t wb[D], xr[D][MF], s0[GA], s1[GA];
+    u32x2_t zw[GA];
+    auto load_step = [&](int d, int t) {
+      const int ks = kstep(t);
+      wb[d] = *(const u32x4_t*)(qw + (int64_t)(ks * 4 + fq) * N);
+#pragma unroll
+      for (int i = 0; i < MF; ++i) xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
+    };
+    auto load_group = [&](int q, int gi) {  // gi = index among this wave's groups
+      const int64_t g = (int64_t)gi * WAVES + wave;
+      s0[q] = *(const u32x4_t*)(sc + g * N);
+      s1[q] = *(const u32x4_t*)(sc + g * N + 8);
+      zw[q] = *(const u32x2_t*)(zp + g * (N / 8));
+    };
+#pragma unroll
+    for (int q = 0; q < GA; ++q) {
+#pragma unroll
+      for (int e = 0; e < SPG; ++e)
+        if (q * SPG + e < steps) load_step(q * SPG + e, q * SPG + e);
+      if (q < my_groups) load_group(q, q);
+    }
+
+    f32x4_t accg[MF][4], accs[MF];
+    for (int t0 = 0; t0 < steps; t0 += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const int t = t0 + d;
+        if (t < steps) {
+          if (d % SPG == 0) {
+#pragma unroll
+            for (int i = 0; i < MF; ++i) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) accg[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+              accs[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            }
+          }
+          u32x4_t xb[MF];
+#pragma unroll
+          for (int i = 0; i < MF; ++i) {
+            const u32x4_t v = xr[d][i];
+            xb[i][0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // k 0, 4
+            xb[i][1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // k 1, 5
+            xb[i][2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // k 2, 6
+            xb[i][3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // k 3, 7
+          }
+          const u32x4_t w4 = wb[d];
+          if (t + D < steps) load_step(d, t + D);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            u32x4_t af;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) af[e] = ((w4[j] >> (4 * e)) & 0x000F000Fu) | E::MAGIC;
+#pragma unroll
+            for (int i = 0; i < MF; ++i) accg[i][j] = E::mfma(af, xb[i], accg[i][j]);
+          }
+          const u32x4_t ones = {E::ONES, E::ONES, E::ONES, E::ONES};
+#pragma unroll
+          for (int i = 0; i < MF; ++i) accs[i] = E::mfma(ones, xb[i], accs[i]);
+
+          if (d % SPG == SPG - 1) {
+            const int q = d / SPG;
+            const u32x4_t sa = s0[q], sb = s1[q];
+            const u32x2_t zq = zw[q];
+            if (t / SPG + GA < my_groups) load_group(q, t / SPG + GA);
+#pragma unroll
+            for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const int c = 4 * ii + j;
+                const uint32_t sw = c < 8 ? sa[c >> 1] : sb[(c - 8) >> 1];
+                const float s = E::to_f32((uint16_t)((c & 1) ? (sw >> 16) : (sw & 0xFFFFu)));
+                const uint32_t z = (zq[c >> 3] >> (4 * (c & 7))) & 0xFu;
+                const float zz = E::BIAS + (float)(int)(z + (uint32_t)p.zero_offset);
+#pragma unroll
+                for (int i = 0; i < MF; ++i) total[i][j][ii] += s * (accg[i][j][ii] - zz * accs[i][ii]);
+              }
+          }
+        }
+      }
+    }
+
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii) red[wave][i][fr * 64 + 16 * fq + 4 * ii + j] = total[i][j][ii];
+    __syncthreads();
+    for (int o = tid; o < MF * 16 * 64; o += 64 * WAVES) {
+      const int i = o / 1024, rem = o % 1024;
+      const int m = mb + i * 16 + rem / 64, n = n0 + rem % 64;
+      float v = red[0][i][rem];
+#pragma unroll
+      for (int w2 = 1; w2 < WAVES; ++w2) v += red[w2][i][rem];
+      if (m < M && n < N) ((uint16_t*)p.c)[(int64_t)m * N + n] = E::from_f32(v);
+    }
+    __syncthreads();
+  }
+}
+
+template <bool FP16>
+hipError_t launch(const W4Params& p, hipStream_t stream) {
+  dim3 grid((p.N + 63) / 64), block(64 * WAVES);
+  // M <= 16: one activation fragment, everything prefetched (group size 128 only). Larger M keeps up
+  // to four activation fragments per pass so that the weights are unpacked once per four fragments.
+  if (p.M <= 16 && p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 2>), grid, block, 0, stream, p);
+  else if (p.M <= 16) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 1>), grid, block, 0, stream, p);
+  else if (p.M <= 32) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 2>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 4>), grid, block, 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream) {
+  return fp16 ? launch<true>(p, stream) : launch<false>(p, stream);
+}

@@ -75,3 +75,39 @@ def grouped_gemm_forward(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor
     [g*N, (g+1)*N) of its own rows (kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:626-629,
     280-289); everything else is left uninitialised."""
     return _grouped_gemm_bf16(x, w, m_sizes, OUT_BLOCK)
+
+
+def matmul_split_k(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
+                   zero_offset: int = 1, groupsize: Optional[int] = None) -> torch.Tensor:
+    """W4A16 split-K dequant GEMM: c = a @ dequant(b, scales, zeros).
+
+    Drop-in for matmul_split_k (kernels/triton/inference/gptq/splitk_dequant_gemm.py:91-141):
+    a [M, K] fp16 or bf16; b [K/8, N] int32 (8 nibbles along K, LSB = lowest k); scales [K/g, N] in a's
+    dtype; zeros [K/g, N/8] int32 (8 nibbles along N); returns c [M, N] in a's dtype.
+    w = (q - (z + zero_offset)) * s with zero_offset = 1 as in the reference (:73-74); zero_offset = 0 gives
+    (q - z) * s. The group size defaults to K // scales.shape[0] (128 in the reference, :94).
+    Unlike the reference there is no atomic accumulation: the result is deterministic and c needs no
+    zero-initialisation."""
+    if a.dim() != 2 or b.dim() != 2 or scales.dim() != 2 or zeros.dim() != 2:
+        raise ValueError("a, b, scales and zeros must be 2-D")
+    m, k = a.shape
+    kw, n = b.shape
+    if kw * 8 != k:
+        raise ValueError(f"b has {kw} packed rows, expected K/8 = {k // 8}")
+    if b.dtype != torch.int32 or zeros.dtype != torch.int32:
+        raise ValueError("b and zeros must be int32")
+    if a.dtype not in (torch.bfloat16, torch.float16) or scales.dtype != a.dtype:
+        raise ValueError("a and scales must both be bf16 or both fp16")
+    g = groupsize if groupsize is not None else k // scales.shape[0]
+    if scales.shape != (k // g, n) or zeros.shape != (k // g, n // 8):
+        raise ValueError("scales must be [K/g, N] and zeros [K/g, N/8]")
+    dev = _require_cuda(a, b, scales, zeros)
+    a, b, scales, zeros = a.contiguous(), b.contiguous(), scales.contiguous(), zeros.contiguous()
+    c = torch.empty((m, n), device=dev, dtype=a.dtype)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_w4a16_splitk(
+            a.data_ptr(), b.data_ptr(), scales.data_ptr(), zeros.data_ptr(), c.data_ptr(), m, n, k, g,
+            zero_offset, 1 if a.dtype == torch.float16 else 0, _stream_ptr(dev),
+        )
+    _lib.check(rc, "moe_gg_w4a16_splitk")
+    return c

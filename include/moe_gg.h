@@ -59,6 +59,27 @@ const char* moe_gg_strerror(int code);
 int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
                              int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream);
 
+#define MOE_GG_DTYPE_BF16 0
+#define MOE_GG_DTYPE_FP16 1
+
+/*
+ * W4A16 split-K dequant GEMM. Replaces matmul_split_k -> matmul_split_k_kernel
+ * (kernels/triton/inference/gptq/splitk_dequant_gemm.py:91-141, 23-89).
+ *
+ *   a        device, [M, K] row-major, bf16 or fp16 (dtype)
+ *   qweight  device, int32 [K/8, N]; nibble j of a word is row 8*i + j (LSB = lowest k)
+ *   scales   device, [K/group_size, N], same 16-bit type as a
+ *   qzeros   device, int32 [K/group_size, N/8]; nibble j of a word is column 8*i + j
+ *   c        device, [M, N], same type as a; fully overwritten (no zero-initialisation needed)
+ *   w(k, n) = (q(k, n) - (z(k/group_size, n) + zero_offset)) * s(k/group_size, n);
+ *   zero_offset = 1 is the reference's convention (splitk_dequant_gemm.py:73-74), 0 gives (q - z) * s.
+ * K is split over the eight waves of a workgroup and reduced in a fixed order (deterministic, no
+ * atomics). Requires N % 64 == 0 and group_size % 32 == 0.
+ */
+int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                        void* c, int M, int N, int K, int group_size, int zero_offset, int dtype,
+                        void* stream);
+
 /*
  * Test / tuning hooks (no counterpart in the reference).
  * moe_gg_set_variant pins the kernel variant used by an op (-1 = automatic choice).
