@@ -26,11 +26,20 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_i64, _c_int,
          _c_void_p],
     ),
+    "moe_gg_grouped_gemm_fp8": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_i64, _c_int, _c_int,
+         _c_i64, _c_int, _c_void_p],
+    ),
     "moe_gg_w4a16_splitk": (
         _c_int,
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
          _c_void_p],
     ),
+    "moe_gg_route_topk": (_c_int, [_c_void_p, _c_i64, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "moe_gg_route_group": (_c_int, [_c_void_p, _c_i64, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
+    "moe_gg_gather_rows": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_i64, _c_i64, _c_void_p]),
+    "moe_gg_fp8_groupwise_quant": (_c_int, [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_i64, _c_void_p]),
     "moe_gg_host_enumerate_tiles": (
         _c_int,
         [_i32_p, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _i32_p, _c_int],

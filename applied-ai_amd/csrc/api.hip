@@ -125,6 +125,38 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
   }
 }
 
+int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* x_scale, const float* w_scale,
+                            int scale_mode, const int32_t* m_sizes, int G, int64_t M, int N, int K,
+                            int64_t ldy, int out_layout, void* stream) {
+  if (G < 0 || M < 0 || N < 0 || K < 0) return MOE_GG_EINVAL;
+  if (out_layout != MOE_GG_OUT_MN && out_layout != MOE_GG_OUT_BLOCK) return MOE_GG_EINVAL;
+  if (scale_mode != MOE_GG_SCALE_ROWWISE && scale_mode != MOE_GG_SCALE_BLOCK128) return MOE_GG_EINVAL;
+  if (M > INT32_MAX || (int64_t)G * N > INT32_MAX || ldy > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  const int64_t min_ld = out_layout == MOE_GG_OUT_BLOCK ? (int64_t)N * G : (int64_t)N;
+  if (ldy < min_ld) return MOE_GG_ESHAPE;
+  if (G == 0 || M == 0 || N == 0) return MOE_GG_OK;
+  if (!x || !w || !y || !m_sizes || !x_scale || !w_scale) return MOE_GG_EINVAL;
+  if (K == 0) return MOE_GG_ESHAPE;
+  if (G > MOE_GG_MAX_GROUPS_ABI) return MOE_GG_EUNSUPPORTED;
+  if (K % 128 != 0 || (scale_mode == MOE_GG_SCALE_BLOCK128 && N % 128 != 0)) return MOE_GG_EUNSUPPORTED;
+  if (!aligned(x, 16) || !aligned(w, 16) || !aligned(y, 2) || !aligned(x_scale, 4) || !aligned(w_scale, 4) ||
+      !aligned(m_sizes, 4))
+    return MOE_GG_EALIGN;
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != MOE_GG_OK) return rc;
+  GgParams p{};
+  p.x = x; p.w = w; p.y = y; p.m_sizes = m_sizes; p.x_scale = x_scale; p.w_scale = w_scale;
+  p.G = G; p.M = (int)M; p.N = N; p.K = K;
+  p.ldy = (int)ldy;
+  p.col_block = out_layout == MOE_GG_OUT_BLOCK ? N : 0;
+  p.vec_store = aligned(y, 8) && ldy % 4 == 0 && N % 4 == 0;
+  p.xcds = di->xcds;
+  int num_wg = di->cus - di->cus % p.xcds;
+  if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
+  return (int)gg_fp8_launch(p, scale_mode, num_wg, (hipStream_t)stream);
+}
+
 int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros,
                         void* c, int M, int N, int K, int group_size, int zero_offset, int dtype,
                         void* stream) {
@@ -142,6 +174,45 @@ int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scale
   if (rc != MOE_GG_OK) return rc;
   W4Params p{a, qweight, scales, qzeros, c, M, N, K, group_size, zero_offset};
   return (int)w4a16_splitk_launch(p, dtype == MOE_GG_DTYPE_FP16, (hipStream_t)stream);
+}
+
+int moe_gg_route_topk(const float* logits, int64_t T, int E, int k, int32_t* ids, int32_t* perm, int32_t* m_sizes,
+                      int32_t* offsets, void* stream) {
+  if (T < 0 || E <= 0 || k <= 0 || k > E) return MOE_GG_EINVAL;
+  if (E > MOE_GG_MAX_ROUTE_EXPERTS || T * k > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (!m_sizes || !perm || (T > 0 && (!logits || !ids))) return MOE_GG_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e = route_topk_launch(logits, (int)T, E, k, ids, s);
+  if (e != hipSuccess) return (int)e;
+  return (int)route_group_launch(ids, (int)(T * k), E, perm, m_sizes, offsets, s);
+}
+
+int moe_gg_route_group(const int32_t* flat_ids, int64_t n, int E, int32_t* perm, int32_t* m_sizes, int32_t* offsets,
+                       void* stream) {
+  if (n < 0 || E <= 0) return MOE_GG_EINVAL;
+  if (E > MOE_GG_MAX_ROUTE_EXPERTS || n > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (!m_sizes || !perm || (n > 0 && !flat_ids)) return MOE_GG_EINVAL;
+  return (int)route_group_launch(flat_ids, (int)n, E, perm, m_sizes, offsets, (hipStream_t)stream);
+}
+
+int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int64_t n, int64_t row_bytes,
+                       void* stream) {
+  if (n < 0 || k <= 0 || row_bytes < 0) return MOE_GG_EINVAL;
+  if (n == 0 || row_bytes == 0) return MOE_GG_OK;
+  if (!x || !perm || !out) return MOE_GG_EINVAL;
+  if (n > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (row_bytes % 16 != 0 || !aligned(x, 16) || !aligned(out, 16)) return MOE_GG_EALIGN;
+  return (int)gather_rows_launch(x, perm, k, out, (int)n, row_bytes, (hipStream_t)stream);
+}
+
+int moe_gg_fp8_groupwise_quant(const void* in, int dtype, void* out, float* scales, int64_t numel, void* stream) {
+  if (numel < 0) return MOE_GG_EINVAL;
+  if (dtype != MOE_GG_DTYPE_BF16 && dtype != MOE_GG_DTYPE_FP32) return MOE_GG_EINVAL;
+  if (numel % 128 != 0) return MOE_GG_ESHAPE;
+  if (numel == 0) return MOE_GG_OK;
+  if (!in || !out || !scales) return MOE_GG_EINVAL;
+  if (!aligned(in, 8) || !aligned(out, 2) || !aligned(scales, 4)) return MOE_GG_EALIGN;
+  return (int)fp8_groupwise_quant_launch(in, dtype == MOE_GG_DTYPE_BF16, out, scales, numel / 128, (hipStream_t)stream);
 }
 
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,

@@ -42,3 +42,17 @@ struct W4Params {
   int zero_offset;
 };
 hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream);
+
+// fp8 e4m3 grouped GEMM (gg_fp8.hip). scale_mode 0: x_scale [M], w_scale [G*N]; 1: x_scale [M, K/128],
+// w_scale [G*N/128, K/128]. Needs K % 128 == 0 (and N % 128 == 0 in block mode), 16-byte aligned x, w.
+hipError_t gg_fp8_launch(const GgParams& p, int scale_mode, int num_wg, hipStream_t stream);
+
+// Routing (routing.hip). E <= MOE_GG_MAX_ROUTE_EXPERTS; ids are int32.
+hipError_t route_topk_launch(const float* logits, int T, int E, int k, int32_t* ids, hipStream_t stream);
+hipError_t route_group_launch(const int32_t* flat, int n, int E, int32_t* perm, int32_t* m_sizes, int32_t* offsets,
+                              hipStream_t stream);
+hipError_t gather_rows_launch(const void* x, const int32_t* perm, int k, void* out, int n, int64_t row_bytes,
+                              hipStream_t stream);
+// 1 x 128 fp8 quantiser (quant.hip); `groups` groups of 128 consecutive elements.
+hipError_t fp8_groupwise_quant_launch(const void* in, bool bf16_in, void* out, float* scales, int64_t groups,
+                                      hipStream_t stream);

@@ -111,3 +111,62 @@ def matmul_split_k(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros
         )
     _lib.check(rc, "moe_gg_w4a16_splitk")
     return c
+
+
+SCALE_ROWWISE = 0
+SCALE_BLOCK128 = 1
+
+
+def _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, scale_mode: int) -> torch.Tensor:
+    # Mirrors _grouped_gemm with scales (dev/triton_groupGEMM/groupgemm.py:407-427, 478-494).
+    assert x.is_contiguous()
+    assert w.is_contiguous()
+    assert m_sizes.is_contiguous()
+    assert x_scale.is_contiguous()
+    assert w_scale.is_contiguous()
+    if x.dim() != 2 or w.dim() != 2 or m_sizes.dim() != 1:
+        raise ValueError("x must be [M, K], w must be [G*N, K], m_sizes must be [G]")
+    G = m_sizes.shape[0]
+    M, K = x.shape
+    if G == 0 or w.shape[0] % G != 0:
+        raise ValueError(f"w.shape[0]={w.shape[0]} is not a multiple of G={G}")
+    N = w.shape[0] // G
+    assert K == w.shape[1], f"K mismatch: x has {K}, w has {w.shape[1]}"
+    if x.dtype != torch.float8_e4m3fn or w.dtype != torch.float8_e4m3fn:
+        raise ValueError("x and w must be torch.float8_e4m3fn (gfx950 computes in OCP e4m3)")
+    if x_scale.dtype != torch.float32 or w_scale.dtype != torch.float32 or m_sizes.dtype != torch.int32:
+        raise ValueError("scales must be float32 and m_sizes int32")
+    if scale_mode == SCALE_ROWWISE:
+        want_x, want_w = (M,), (G * N,)
+    else:
+        if K % 128 or (G * N) % 128:
+            raise ValueError("block scales need K and G*N to be multiples of 128")
+        want_x, want_w = (M, K // 128), (G * N // 128, K // 128)
+    if tuple(x_scale.shape) != want_x or tuple(w_scale.shape) != want_w:
+        raise ValueError(f"scale shapes must be {want_x} and {want_w}")
+    dev = _require_cuda(x, w, m_sizes, x_scale, w_scale)
+    y = torch.empty((M, N), device=dev, dtype=torch.bfloat16)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_grouped_gemm_fp8(
+            x.data_ptr(), w.data_ptr(), y.data_ptr(), x_scale.data_ptr(), w_scale.data_ptr(), scale_mode,
+            m_sizes.data_ptr(), G, M, N, K, N, OUT_MN, _stream_ptr(dev),
+        )
+    _lib.check(rc, "moe_gg_grouped_gemm_fp8")
+    return y
+
+
+def grouped_gemm_fp8_rowwise(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, x_scale: torch.Tensor,
+                             w_scale: torch.Tensor) -> torch.Tensor:
+    """fp8 grouped GEMM with one scale per activation row and per weight row:
+    y = (x @ w_g.T) * x_scale[:, None] * w_scale[g*N:(g+1)*N][None, :], bf16 out.
+    Drop-in for grouped_gemm_fp8_rowwise (dev/triton_groupGEMM/groupgemm.py:524-531)."""
+    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_ROWWISE)
+
+
+def grouped_gemm_fp8_blockwise(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, x_scale: torch.Tensor,
+                               w_scale: torch.Tensor) -> torch.Tensor:
+    """fp8 grouped GEMM with 1x128 activation scales x_scale[M, K/128] (the output layout of
+    float8_groupwise_quantize, kernels/triton/inference/fp8/float8_groupwise_quant.py:53-91) and 128x128
+    weight scales w_scale[G*N/128, K/128]; bf16 out. No counterpart in the reference (its fp8 grouped GEMM is
+    row-wise only); it is the block-scaled extension of that entry point."""
+    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_BLOCK128)

@@ -1,0 +1,66 @@
+"""Routing in front of the grouped GEMM: top-k expert choice, expert-sorted permutation, m_sizes, offsets.
+
+The host-side mirror of what the reference's MoE tests do with torch.topk
+(kernels/triton/inference/col_major_moe_gemm/test_moe_gemm.py:54-57) plus the grouping of the external
+moe_align_block_size op (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:141-166, without its
+padding); the work runs in the HIP kernels behind include/moe_gg.h."""
+from typing import Tuple
+
+import torch
+
+from . import _lib
+from .ops import _require_cuda, _stream_ptr
+
+
+def route_topk(logits: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """logits [T, E] fp32 -> (ids [T, k] int32, perm [T*k] int32, m_sizes [E] int32, offsets [E+1] int32).
+
+    ids are the k best experts per token in descending score (ties to the lower id); perm lists the flat
+    positions token*k + j grouped by ascending expert, stable, so sorted row i comes from token perm[i] // k;
+    m_sizes / offsets are what grouped_gemm consumes."""
+    if logits.dim() != 2 or logits.dtype != torch.float32:
+        raise ValueError("logits must be fp32 [T, E]")
+    dev = _require_cuda(logits)
+    logits = logits.contiguous()
+    T, E = logits.shape
+    ids = torch.empty((T, k), dtype=torch.int32, device=dev)
+    perm = torch.empty((T * k,), dtype=torch.int32, device=dev)
+    m_sizes = torch.empty((E,), dtype=torch.int32, device=dev)
+    offsets = torch.empty((E + 1,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_route_topk(logits.data_ptr(), T, E, k, ids.data_ptr(), perm.data_ptr(),
+                                          m_sizes.data_ptr(), offsets.data_ptr(), _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_route_topk")
+    return ids, perm, m_sizes, offsets
+
+
+def route_group(topk_ids: torch.Tensor, num_experts: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Grouping only, for expert ids chosen elsewhere: topk_ids int32 [T, k] -> (perm, m_sizes, offsets)."""
+    if topk_ids.dtype != torch.int32:
+        raise ValueError("topk_ids must be int32")
+    dev = _require_cuda(topk_ids)
+    flat = topk_ids.contiguous().reshape(-1)
+    n = flat.shape[0]
+    perm = torch.empty((n,), dtype=torch.int32, device=dev)
+    m_sizes = torch.empty((num_experts,), dtype=torch.int32, device=dev)
+    offsets = torch.empty((num_experts + 1,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_route_group(flat.data_ptr(), n, num_experts, perm.data_ptr(), m_sizes.data_ptr(),
+                                           offsets.data_ptr(), _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_route_group")
+    return perm, m_sizes, offsets
+
+
+def gather_sorted(x: torch.Tensor, perm: torch.Tensor, k: int) -> torch.Tensor:
+    """x_sorted[i] = x[perm[i] // k]: the token rows in expert-sorted order."""
+    if x.dim() != 2 or perm.dtype != torch.int32:
+        raise ValueError("x must be 2-D and perm int32")
+    dev = _require_cuda(x, perm)
+    x = x.contiguous()
+    n = perm.shape[0]
+    out = torch.empty((n, x.shape[1]), dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_gather_rows(x.data_ptr(), perm.data_ptr(), k, out.data_ptr(), n,
+                                           x.shape[1] * x.element_size(), _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_gather_rows")
+    return out

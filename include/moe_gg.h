@@ -59,8 +59,27 @@ const char* moe_gg_strerror(int code);
 int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
                              int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream);
 
+#define MOE_GG_SCALE_ROWWISE 0  /* x_scale [M], w_scale [G*N] */
+#define MOE_GG_SCALE_BLOCK128 1 /* x_scale [M, K/128], w_scale [G*N/128, K/128] */
+
+/*
+ * fp8 (OCP e4m3fn) grouped GEMM forward, bf16 output, fp32 accumulation and scales.
+ * scale_mode = MOE_GG_SCALE_ROWWISE replaces grouped_gemm_fp8_rowwise -> _kernel_grouped_gemm_fp8_rowwise
+ * (dev/triton_groupGEMM/groupgemm.py:524-531, 269-404): y = (x @ w_g^T) * x_scale[m] * w_scale[g*N + n].
+ * scale_mode = MOE_GG_SCALE_BLOCK128 is the block-scaled extension used by the DeepSeek-V3-style
+ * configuration: per-1x128 activation scales as produced by float8_groupwise_quantize
+ * (kernels/triton/inference/fp8/float8_groupwise_quant.py:53-91) and per-128x128 weight scales; each
+ * 128-wide K block is scaled by x_scale[m, kb] * w_scale[(g*N + n) / 128, kb] before it is summed.
+ * x, w: device fp8 [M, K] / [G*N, K]; other arguments as for moe_gg_grouped_gemm_bf16.
+ * Requires K % 128 == 0 (and N % 128 == 0 for block scales).
+ */
+int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* x_scale, const float* w_scale,
+                            int scale_mode, const int32_t* m_sizes, int G, int64_t M, int N, int K,
+                            int64_t ldy, int out_layout, void* stream);
+
 #define MOE_GG_DTYPE_BF16 0
 #define MOE_GG_DTYPE_FP16 1
+#define MOE_GG_DTYPE_FP32 2
 
 /*
  * W4A16 split-K dequant GEMM. Replaces matmul_split_k -> matmul_split_k_kernel
@@ -79,6 +98,41 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
 int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros,
                         void* c, int M, int N, int K, int group_size, int zero_offset, int dtype,
                         void* stream);
+
+#define MOE_GG_MAX_ROUTE_EXPERTS 768
+
+/*
+ * Routing: top-k expert choice, expert histogram, offsets and the stable expert-sorted permutation.
+ * Replaces torch.topk as used by the reference's MoE test
+ * (kernels/triton/inference/col_major_moe_gemm/test_moe_gemm.py:54-57) and the grouping of the external
+ * moe_align_block_size op (semantics: kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:141-166),
+ * without its padding.
+ *   logits   device, fp32 [T, E]
+ *   ids      device out, int32 [T, k]: the k largest entries of each row, descending, ties to the lower id
+ *   perm     device out, int32 [T*k]: flat positions p = token*k + j grouped by ascending expert, stable;
+ *            the source token of sorted row i is perm[i] / k
+ *   m_sizes  device out, int32 [E]: rows per expert (the m_sizes argument of the grouped GEMMs)
+ *   offsets  device out, int32 [E+1] or NULL: exclusive prefix sum of m_sizes
+ *            (dev/triton_groupGEMM/groupgemm.py:159-165)
+ * moe_gg_route_group does the grouping for ids chosen elsewhere (flat_ids int32 [n]; ids outside [0, E) are
+ * dropped). E <= MOE_GG_MAX_ROUTE_EXPERTS.
+ */
+int moe_gg_route_topk(const float* logits, int64_t T, int E, int k, int32_t* ids, int32_t* perm, int32_t* m_sizes,
+                      int32_t* offsets, void* stream);
+int moe_gg_route_group(const int32_t* flat_ids, int64_t n, int E, int32_t* perm, int32_t* m_sizes, int32_t* offsets,
+                       void* stream);
+/* out[i, :] = x[perm[i] / k, :] for i < n; rows of row_bytes bytes (multiple of 16), x and out 16-byte aligned. */
+int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int64_t n, int64_t row_bytes,
+                       void* stream);
+
+/*
+ * 1 x 128 group-wise fp8 e4m3fn quantiser. Replaces float8_groupwise_quantize
+ * (kernels/triton/inference/fp8/float8_groupwise_quant.py:53-91): per 128 consecutive elements
+ * s = max(amax|x|, 1e-12) / 448, q = clamp(x / s, -448, 448) -> e4m3fn (RNE).
+ *   in  device, bf16 or fp32 (dtype), numel elements, numel % 128 == 0;  out device, numel bytes;
+ *   scales device out, fp32 [numel / 128].
+ */
+int moe_gg_fp8_groupwise_quant(const void* in, int dtype, void* out, float* scales, int64_t numel, void* stream);
 
 /*
  * Test / tuning hooks (no counterpart in the reference).
