@@ -180,7 +180,7 @@ int moe_gg_route_topk(const float* logits, int64_t T, int E, int k, int32_t* ids
                       int32_t* offsets, void* stream) {
   if (T < 0 || E <= 0 || k <= 0 || k > E) return MOE_GG_EINVAL;
   if (E > MOE_GG_MAX_ROUTE_EXPERTS || T * k > INT32_MAX) return MOE_GG_EUNSUPPORTED;
-  if (!m_sizes || !perm || (T > 0 && (!logits || !ids))) return MOE_GG_EINVAL;
+  if (!m_sizes || (T > 0 && (!logits || !ids || !perm))) return MOE_GG_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   hipError_t e = route_topk_launch(logits, (int)T, E, k, ids, s);
   if (e != hipSuccess) return (int)e;
@@ -191,7 +191,7 @@ int moe_gg_route_group(const int32_t* flat_ids, int64_t n, int E, int32_t* perm,
                        void* stream) {
   if (n < 0 || E <= 0) return MOE_GG_EINVAL;
   if (E > MOE_GG_MAX_ROUTE_EXPERTS || n > INT32_MAX) return MOE_GG_EUNSUPPORTED;
-  if (!m_sizes || !perm || (n > 0 && !flat_ids)) return MOE_GG_EINVAL;
+  if (!m_sizes || (n > 0 && (!flat_ids || !perm))) return MOE_GG_EINVAL;
   return (int)route_group_launch(flat_ids, (int)n, E, perm, m_sizes, offsets, (hipStream_t)stream);
 }
 

@@ -1,0 +1,134 @@
+"""GPU parity of the fp8 grouped GEMM (row-wise and block scales) and of the 1x128 quantiser.
+GEMM: relative Frobenius error <= 2e-2 against the dequantise-then-matmul oracle; quantiser: bit-exact."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.gpu_util import rel_fro, to_np
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+F8 = torch.float8_e4m3fn
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def f8(codes):
+    return torch.from_numpy(np.ascontiguousarray(codes)).view(F8)
+
+
+def run(xq, wq, xs, ws, m_sizes, mode):
+    import applied_ai_amd as A
+
+    fn = A.grouped_gemm_fp8_blockwise if mode == 1 else A.grouped_gemm_fp8_rowwise
+    y = fn(f8(xq).cuda(), f8(wq).cuda(), torch.tensor(m_sizes, dtype=torch.int32, device="cuda"),
+           torch.from_numpy(np.ascontiguousarray(xs, dtype=np.float32)).cuda(), torch.from_numpy(np.ascontiguousarray(ws, dtype=np.float32)).cuda())
+    torch.cuda.synchronize()
+    return y
+
+
+def test_golden_fixture_block_and_rowwise():
+    z = np.load(os.path.join(GOLD, "fp8_tiny.npz"))
+    m = z["m_sizes"].tolist()
+    tot = sum(m)
+    y = run(z["xq"], z["wq"], z["xs"], z["ws"], m, 1)
+    assert rel_fro(to_np(y)[:tot], z["y_block"][:tot]) <= TOL
+    y = run(z["xq_row"], z["wq_row"], z["xs_row"], z["ws_row"], m, 0)
+    assert rel_fro(to_np(y)[:tot], z["y_row"][:tot]) <= TOL
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("G,N,K,m_sizes", [
+    (1, 128, 128, [16]),
+    (2, 128, 256, [100, 28]),
+    (4, 256, 512, [0, 300, 1, 83]),
+    (8, 512, 1024, [7, 130, 64, 0, 255, 129, 33, 2]),
+    (3, 384, 7168, [5, 200, 60]),
+])
+def test_against_oracle(mode, G, N, K, m_sizes):
+    print(f"case mode={mode} G={G} N={N} K={K} m_sizes={m_sizes}", flush=True)
+    rng = np.random.default_rng(G + N + K)
+    M = sum(m_sizes)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((G * N, K)) * 0.05).astype(np.float32)
+    if mode == 1:
+        xq, xs = O.fp8_groupwise_quant(x); wq, ws = O.fp8_block_quant_weight(w)
+    else:
+        xs = np.abs(x).max(axis=1) / 448.0; ws = np.abs(w).max(axis=1) / 448.0
+        xq = torch.from_numpy(np.clip(x / xs[:, None], -448, 448)).to(F8).view(torch.uint8).numpy()
+        wq = torch.from_numpy(np.clip(w / ws[:, None], -448, 448)).to(F8).view(torch.uint8).numpy()
+    y = run(xq, wq, xs, ws, m_sizes, mode)
+    ref = O.grouped_gemm_fp8(xq, wq, xs, ws, m_sizes, mode)
+    assert rel_fro(to_np(y), ref) <= TOL
+
+
+def test_unit_scales_equal_plain_fp8_product():
+    """All scales = 1: block-scaled and row-wise kernels must agree bit for bit with each other
+    (same MFMA sums, scaling by 1.0 is exact) - the invariant that ties the block extension to the reference's
+    row-wise kernel (dev/triton_groupGEMM/groupgemm.py:374-384)."""
+    rng = np.random.default_rng(21)
+    G, N, K = 2, 256, 512
+    m_sizes = [37, 91]
+    M = sum(m_sizes)
+    xq = rng.integers(0, 0x60, size=(M, K)).astype(np.uint8) | (rng.integers(0, 2, size=(M, K)) * 0x80).astype(np.uint8)
+    wq = rng.integers(0, 0x50, size=(G * N, K)).astype(np.uint8) | (rng.integers(0, 2, size=(G * N, K)) * 0x80).astype(np.uint8)
+    yb = run(xq, wq, np.ones((M, K // 128)), np.ones((G * N // 128, K // 128)), m_sizes, 1)
+    yr = run(xq, wq, np.ones(M), np.ones(G * N), m_sizes, 0)
+    ref = O.grouped_gemm(O.e4m3_to_f32(xq), O.e4m3_to_f32(wq), m_sizes)
+    assert rel_fro(to_np(yr), ref) <= 4e-3
+    assert rel_fro(to_np(yb), ref) <= 4e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_quantiser_bit_exact(dtype):
+    import applied_ai_amd as A
+
+    gen = torch.Generator().manual_seed(4)
+    x = (torch.randn(300, 1024, generator=gen) * torch.rand(300, 1, generator=gen) * 5).to(dtype)
+    x[0, :128] = 0          # all-zero group: scale 1e-12 / 448, codes 0
+    x[1, 5] = 1000.0        # outlier dominates its group
+    q, s = A.float8_groupwise_quantize(x.cuda())
+    torch.cuda.synchronize()
+    oq, os_ = O.fp8_groupwise_quant(x.float().numpy())
+    assert q.dtype == F8 and s.shape == (300, 8)
+    assert np.array_equal(q.view(torch.uint8).cpu().numpy(), oq)
+    assert np.array_equal(s.cpu().numpy(), os_)
+    with pytest.raises(ValueError):
+        A.float8_groupwise_quantize(torch.zeros(4, 100, device="cuda"))
+
+
+def test_config5_shape_sampled_experts():
+    """BASELINE config 5 at full K and N (7168, 4096) with its Zipf routing, on a sample of experts (largest,
+    smallest, two in between): activations quantised by the GPU quantiser, weights by the block quantiser,
+    oracle on a 256-column slice."""
+    import applied_ai_amd as A
+    from applied_ai_amd import configs
+
+    _, _, _, m_all = configs.cfg5_routing()
+    order = np.argsort(-m_all.numpy())
+    pick = [int(order[0]), int(order[40]), int(order[128]), int(order[-1])]
+    m_sizes = [min(int(m_all[g]), 700) for g in pick]
+    print(f"cfg5 sample experts {pick} rows {m_sizes}", flush=True)
+    G, N, K = len(pick), 4096, 7168
+    gen = torch.Generator().manual_seed(1005)
+    x = torch.randn(sum(m_sizes), K, generator=gen)
+    w = torch.randn(G * N, K, generator=gen) * 0.02
+    xq, xs = A.float8_groupwise_quantize(x.cuda())
+    wq, ws = A.float8_blockwise_quantize_weight(w.cuda())
+    y = A.grouped_gemm_fp8_blockwise(xq, wq, torch.tensor(m_sizes, dtype=torch.int32, device="cuda"), xs, ws)
+    torch.cuda.synchronize()
+    off = O.offsets(m_sizes)
+    xq_h = xq.view(torch.uint8).cpu().numpy(); xs_h = xs.cpu().numpy()
+    wq_h = wq.view(torch.uint8).cpu().numpy(); ws_h = ws.cpu().numpy()
+    for gi in range(G):
+        rows = slice(off[gi], min(off[gi + 1], off[gi] + 64))
+        wr = slice(gi * N + 1024, gi * N + 1280)
+        ref = O.grouped_gemm_fp8(xq_h[rows], wq_h[wr], xs_h[rows], ws_h[(gi * N + 1024) // 128:(gi * N + 1280) // 128],
+                                 [rows.stop - rows.start], 1)
+        assert rel_fro(to_np(y[rows, 1024:1280]), ref) <= TOL
+    # quantised result is close to the unquantised product too
+    g0 = slice(off[0], off[0] + 32)
+    exact = x[g0].double() @ w[1024:1280].double().T
+    assert rel_fro(to_np(y[g0, 1024:1280]), exact.numpy()) <= 6e-2
