@@ -1,11 +1,14 @@
 """Benchmark of the MoE grouped-GEMM hot path on one MI355X.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill]
-A step is one pass of the hot path over one batch of synthetic, HBM-resident input. The default workload is the
-configuration the headline metric is quoted on: Mixtral 8x7B w1 grouped GEMM, bf16, T=4096 tokens top-2 (8192
-expert-sorted rows), K=4096, N=14336, 8 experts. Prints ONE JSON line.
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu-baseline]
+
+A step is one pass of the hot path over one batch of synthetic, HBM-resident input. The headline workload is the
+configuration the metric is quoted on: Mixtral 8x7B w1 grouped GEMM, bf16, T=4096 tokens top-2 (8192 expert-sorted
+rows), K=4096, N=14336, 8 experts. Prints ONE JSON line; the other benchmark configurations (decode, W4A16, fp8)
+are measured in the same run and reported under "secondary" with their own rooflines.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -15,7 +18,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+# HBM traffic per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what the
+# same counters read for a plain copy of known size (profiles/gg_bf16_pingpong_mixtral_prefill_traffic.md):
+# 2.06 GB fetched + 0.245 GB written.
+PREFILL_TRAFFIC_BYTES = 2.30e9
 
 
 def cpu_baseline_prefill(c, n_experts_sample=2):
@@ -40,12 +49,124 @@ def cpu_baseline_prefill(c, n_experts_sample=2):
         times.append(time.perf_counter() - t0)
     t = min(times)
     return {
-        "value": 2.0 * rows * N * K / t / 1e12,
+        "value": round(2.0 * rows * N * K / t / 1e12, 3),
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"first {n_experts_sample} of 8 experts ({rows} of {sum(c['m_sizes'].tolist())} rows), fp32 torch.matmul loop, best of 2",
+        "sample": f"first {n_experts_sample} of 8 experts ({rows} of {sum(c['m_sizes'].tolist())} rows), fp32 per-expert torch.matmul loop, best of 2",
     }
+
+
+def event_time_ms(torch, fn, iters, warmup):
+    """Average duration of fn() over `iters` back-to-back calls, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    s = torch.cuda.Event(enable_timing=True)
+    e = torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters
+
+
+def secondary_workloads(torch, A, dev):
+    """Decode (config 3), W4A16 (config 4) and fp8 block-scaled (config 5) shapes: HBM-bound kernels, reported as
+    GB/s of algorithmic bytes against the 8 TB/s HBM peak. Weights rotate over enough distinct copies that the
+    footprint exceeds the 256 MB Infinity Cache. Calls go straight through the C ABI so that the ~10 us kernels
+    are not timed through Python allocation overhead."""
+    from applied_ai_amd import configs
+
+    lib = A._lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    out = []
+
+    # ---- config 3: Mixtral decode, bf16, 64 rows over 8 experts ----
+    c3 = configs.cfg3()
+    m_sizes = c3["m_sizes"].tolist()
+    ms_dev = c3["m_sizes"].to(dev)
+    active = sum(1 for m in m_sizes if m > 0)
+    for name, K, N in (("up-proj K=4096 N=14336", 4096, 14336), ("down-proj K=14336 N=4096", 14336, 4096)):
+        x = torch.randn(64, K, device=dev).to(torch.bfloat16)
+        ws = [(torch.randn(8 * N, K, device=dev) * 0.02).to(torch.bfloat16) for _ in range(2)]
+        y = torch.empty(64, N, device=dev, dtype=torch.bfloat16)
+        state = {"i": 0}
+
+        def call():
+            w = ws[state["i"] & 1]
+            state["i"] += 1
+            lib.moe_gg_grouped_gemm_bf16(x.data_ptr(), w.data_ptr(), y.data_ptr(), ms_dev.data_ptr(), 8, 64, N, K, N, 0, stream)
+
+        ms = event_time_ms(torch, call, 40, 6)
+        byt = active * N * K * 2 + 64 * K * 2 + 64 * N * 2
+        out.append({"workload": f"Mixtral decode bf16, T=32 top-2 (64 rows, m_sizes {m_sizes}), {name}",
+                    "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
+                    "roofline": {"bound": "hbm", "kernel": "gg_bf16_decode", "achieved": round(byt / ms / 1e6, 1),
+                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                 "traffic": None}})
+        del ws
+
+    # ---- config 4: W4A16 split-K, K=4096, N=14336, group 128, (q - z) * s ----
+    K, N, copies = 4096, 14336, 12
+    qws = [torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device=dev) for _ in range(copies)]
+    sc = (torch.rand(K // 128, N, device=dev) * 0.015 + 0.005).to(torch.bfloat16)
+    qz = torch.randint(-2**31, 2**31 - 1, (K // 128, N // 8), dtype=torch.int32, device=dev)
+    for M in (1, 16, 64):
+        a = torch.randn(M, K, device=dev).to(torch.bfloat16)
+        c = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+        state = {"i": 0}
+
+        def call():
+            qw = qws[state["i"] % copies]
+            state["i"] += 1
+            lib.moe_gg_w4a16_splitk(a.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), c.data_ptr(), M, N, K, 128, 0, 0, stream)
+
+        ms = event_time_ms(torch, call, 120, 24)
+        byt = K * N // 2 + (K // 128) * N * 2 + (K // 128) * N // 2 + M * K * 2 + M * N * 2
+        out.append({"workload": f"W4A16 split-K M={M} K=4096 N=14336 group 128",
+                    "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
+                    "roofline": {"bound": "hbm", "kernel": "w4a16_splitk", "achieved": round(byt / ms / 1e6, 1),
+                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                 "traffic": None}})
+    del qws
+
+    # ---- config 5: DeepSeek-V3-style fp8 block-scaled, 256 experts top-8, Zipf(1.1) routing ----
+    _, _, _, m5 = configs.cfg5_routing()
+    G, N, K = 256, 4096, 7168
+    M = int(m5.sum())
+    f8 = torch.float8_e4m3fn
+
+    def rand_fp8(rows):
+        t = torch.randint(0, 256, (rows, K), dtype=torch.uint8, device=dev)
+        return torch.where((t & 0x7F) == 0x7F, t & 0xF0, t)  # no NaN codes
+
+    xq = rand_fp8(M).view(f8)
+    wq = torch.empty(G * N, K, dtype=torch.uint8, device=dev)
+    for g in range(G):
+        wq[g * N:(g + 1) * N] = rand_fp8(N)
+    wq = wq.view(f8)
+    xs = torch.rand(M, K // 128, device=dev) * 0.01 + 0.001
+    ws = torch.rand(G * N // 128, K // 128, device=dev) * 0.01 + 0.001
+    y = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+    ms_dev = m5.to(dev)
+
+    def call():
+        lib.moe_gg_grouped_gemm_fp8(xq.data_ptr(), wq.data_ptr(), y.data_ptr(), xs.data_ptr(), ws.data_ptr(), 1,
+                                    ms_dev.data_ptr(), G, M, N, K, N, 0, stream)
+
+    ms = event_time_ms(torch, call, 5, 2)
+    active = int((m5 > 0).sum())
+    byt = M * K + active * N * K + M * N * 2 + M * (K // 128) * 4 + active * (N // 128) * (K // 128) * 4
+    flop = 2.0 * M * N * K
+    out.append({"workload": "DeepSeek-V3-style fp8 e4m3 block-scaled grouped GEMM: 256 experts top-8, T=4096 (32768 rows, Zipf 1.1), K=7168, N=4096",
+                "ms_per_launch": round(ms, 3), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
+                "tflops": round(flop / ms / 1e9, 1),
+                "roofline": {"bound": "hbm", "kernel": "gg_fp8_persistent", "achieved": round(byt / ms / 1e6, 1),
+                             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
+                             "traffic": None}})
+    return out
 
 
 def main():
@@ -54,6 +175,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy, so that a rocprofv3 --pmc run of this command sees a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -115,18 +239,28 @@ def main():
         "pct_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
         "roofline": {
             "bound": "mfma",
-            "kernel": "gg_bf16_persistent",
+            "kernel": "gg_bf16_pingpong",
             "achieved": round(achieved, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": PREFILL_TRAFFIC_BYTES,
             "kernel_ms": {"avg": round(avg_kernel_ms, 4), "p20": round(kern_ms[len(kern_ms) // 5], 4),
                           "p50": round(kern_ms[len(kern_ms) // 2], 4), "p80": round(kern_ms[(len(kern_ms) * 4) // 5], 4)},
         },
     }
+    del x, w, y
+    if args.copy_calibration:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_prefill(c)
+    if not args.no_secondary:
+        out["secondary"] = secondary_workloads(torch, A, dev)
     print(json.dumps(out))
 
 
