@@ -154,6 +154,12 @@ int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* 
   p.xcds = di->xcds;
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
+  // Experts with a few rows are weight-streaming problems: they go to the split-K streaming kernel, the
+  // tiled kernel takes the rest. m_sizes stays on the device, so both are always launched; a kernel whose
+  // share is empty exits after reading m_sizes.
+  hipError_t e = gg_fp8_stream_launch(p, scale_mode, (hipStream_t)stream);
+  if (e != hipSuccess) return (int)e;
+  p.skip_rows = gg_fp8_stream_max_rows();
   return (int)gg_fp8_launch(p, scale_mode, num_wg, (hipStream_t)stream);
 }
 

@@ -28,6 +28,8 @@
 // Group 0 waits for its loads at the end of C(s); group 1 waits for W0(s+1) at the end of L(s), with
 // the W0(s+2) instructions it has just issued still in flight. The slab sequence runs straight
 // through tile boundaries, so the next tile's first slabs are in flight during the epilogue.
+#include <type_traits>
+
 #include "common.h"
 #include "gg_tables.h"
 #include "kernels.h"
@@ -131,6 +133,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   };
   // Block b (8 rows) of the cursor slab's activation / weight rows.
   auto dma_x = [&](int b) {
+    if (b * 8 > c.x_last) return;  // block entirely below the tile's last row: its fragments are never used
     const uint32_t off = (uint32_t)min(b * 8 + d_r, c.x_last) * K2 + d_c16;
     dma16(c.xg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + b * 1024);
   };
@@ -170,72 +173,109 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const int m0 = t.tm * BM, n0 = t.tn * BN;
     const int rows_valid = min(t.rows - m0, BM);
     const int cols_valid = min(N - n0, BN);
+    // Activation fragments of this wave that hold at least one valid row (fragments are dealt
+    // alternately to wm = 0 / 1, so a short tile shortens every wave's C phase alike).
+    const int nfm = min(FM, max(0, ((rows_valid + 15) / 16 - wm + WM - 1) / WM));
 
-    f32x4_t acc[FN][FM];
+    // The tile body exists twice: for full-height tiles (all 64 MFMAs per step, no branches) and for
+    // short tiles, which skip the MFMAs of activation fragments that hold no valid row. Each copy has
+    // its own accumulators, so the two K loops do not have to agree on a register assignment.
+    auto do_tile = [&](auto short_tag) {
+      constexpr bool SHORT = decltype(short_tag)::value;
+      f32x4_t acc[FN][FM];
 #pragma unroll
-    for (int j = 0; j < FN; ++j)
+      for (int j = 0; j < FN; ++j)
 #pragma unroll
-      for (int i = 0; i < FM; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < FM; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int kt = 0; kt < KT; ++kt, ++step) {
-      // ---------------- L phase: 24 fragment reads interleaved with this wave's slab loads ----------------
-      // Activation fragment i covers tile rows (i * WM + wm) * 16 .. + 15; weight fragment j covers
-      // tile columns (wn * FN + j) * 16 .. + 15.
-      const char* xs = sh.lds + (step & 1) * STAGE + wm * 2048;
-      const char* ws = sh.lds + (step & 1) * STAGE + X_BYTES + wn * (FN * 2048);
-      bf16x8_t wf[2][FN], xf[2][FM];
-      constexpr int READS_PER_DMA = 24 / NDMA;
+      for (int kt = 0; kt < KT; ++kt, ++step) {
+        // ---------------- L phase: 24 fragment reads interleaved with this wave's slab loads ----------------
+        // Activation fragment i covers tile rows (i * WM + wm) * 16 .. + 15; weight fragment j covers
+        // tile columns (wn * FN + j) * 16 .. + 15.
+        const char* xs = sh.lds + (step & 1) * STAGE + wm * 2048;
+        const char* ws = sh.lds + (step & 1) * STAGE + X_BYTES + wn * (FN * 2048);
+        bf16x8_t wf[2][FN], xf[2][FM];
+        constexpr int READS_PER_DMA = 24 / NDMA;
 #pragma unroll
-      for (int q = 0; q < 24; ++q) {
-        if (q % READS_PER_DMA == 0) {
-          __builtin_amdgcn_sched_barrier(0);
-          dma_one(q / READS_PER_DMA);
-          __builtin_amdgcn_sched_barrier(0);
+        for (int q = 0; q < 24; ++q) {
+          if (q % READS_PER_DMA == 0) {
+            __builtin_amdgcn_sched_barrier(0);
+            dma_one(q / READS_PER_DMA);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          const int kk = q / 12, f = q % 12;
+          const int ro = kk ? (rd0 ^ 64) : rd0;
+          if (f < FN) wf[kk][f] = *(const bf16x8_t*)(ws + f * 2048 + ro);
+          else xf[kk][f - FN] = *(const bf16x8_t*)(xs + (f - FN) * (WM * 2048) + ro);
         }
-        const int kk = q / 12, f = q % 12;
-        const int ro = kk ? (rd0 ^ 64) : rd0;
-        if (f < FN) wf[kk][f] = *(const bf16x8_t*)(ws + f * 2048 + ro);
-        else xf[kk][f - FN] = *(const bf16x8_t*)(xs + (f - FN) * (WM * 2048) + ro);
+        __builtin_amdgcn_sched_barrier(0);
+        wait_lgkm0();  // all of slab `step` is in this wave's registers
+        if (GRP == 1) wait_vm<NDMA>();  // W0(step + 1) has landed; W0(step + 2) may still be in flight
+        __syncthreads();
+        // ---------------- C phase: 64 MFMAs ----------------
+        __builtin_amdgcn_s_setprio(1);
+        if (!SHORT) {
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+              for (int i = 0; i < FM; ++i)
+                acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[kk][j], xf[kk][i], acc[j][i], 0, 0, 0);
+        } else {
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+            if (i < nfm) {
+#pragma unroll
+              for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                  acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[kk][j], xf[kk][i], acc[j][i], 0, 0, 0);
+            }
+          }
+        }
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (GRP == 0) wait_vm<0>();  // X(step + 1), W1(step + 1): issued at the start of this step
+        __syncthreads();
       }
-      __builtin_amdgcn_sched_barrier(0);
-      wait_lgkm0();  // all of slab `step` is in this wave's registers
-      if (GRP == 1) wait_vm<NDMA>();  // W0(step + 1) has landed; W0(step + 2) may still be in flight
-      __syncthreads();
-      // ---------------- C phase: 64 MFMAs ----------------
-      __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int i = 0; i < FM; ++i)
-            acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[kk][j], xf[kk][i], acc[j][i], 0, 0, 0);
-      __builtin_amdgcn_s_setprio(0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (GRP == 0) wait_vm<0>();  // X(step + 1), W1(step + 1): issued at the start of this step
-      __syncthreads();
-    }
 
-    // Epilogue: lane holds y[m][n .. n+3] for m = (i * WM + wm) * 16 + lane % 16,
-    // n = (wn * FN + j) * 16 + 4 * (lane / 16).
-    bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + (int64_t)t.g * p.col_block + n0;
-    {
-      const bool vec_ok = p.vec_store;
+      // Epilogue: lane holds y[m][n .. n+3] for m = (i * WM + wm) * 16 + lane % 16,
+      // n = (wn * FN + j) * 16 + 4 * (lane / 16). Addresses are a per-fragment uniform base plus one
+      // 32-bit lane offset, so nothing has to stay in registers across the K loop.
+      // The lane indices pass through an empty asm so that the address arithmetic is redone here for
+      // every tile instead of being hoisted out of the tile loop, where it would occupy (and spill)
+      // registers during the K loop.
+      bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + (int64_t)t.g * p.col_block + n0;
+      int er = fr, eq = fq;
+      asm volatile("" : "+v"(er), "+v"(eq));
+      if (p.vec_store && cols_valid == BN && p.ldy < (1 << 24)) {
+        const uint32_t voff = (uint32_t)er * (uint32_t)p.ldy + (uint32_t)(wn * FN * 16 + eq * 4);
 #pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        const int m = (i * WM + wm) * 16 + fr;
-        if (m < rows_valid) {
-          bf16_t* yrow = yg + (int64_t)m * p.ldy;
+        for (int i = 0; i < FM; ++i) {
+          const int mrow = (i * WM + wm) * 16;
+          bf16_t* ybase = yg + (int64_t)mrow * p.ldy;  // uniform
+          if (mrow + er < rows_valid) {
 #pragma unroll
-          for (int j = 0; j < FN; ++j) {
-            const int n = (wn * FN + j) * 16 + fq * 4;
-            const f32x4_t v = acc[j][i];
-            if (vec_ok && n + 3 < cols_valid) {
+            for (int j = 0; j < FN; ++j) {
+              const f32x4_t v = acc[j][i];
               u32x2_t o;
               o[0] = pack_bf16x2(v[0], v[1]);
               o[1] = pack_bf16x2(v[2], v[3]);
-              *(u32x2_t*)(yrow + n) = o;
-            } else {
+              *(u32x2_t*)(ybase + voff + j * 16) = o;
+            }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          const int m = (i * WM + wm) * 16 + er;
+          if (m < rows_valid) {
+            bf16_t* yrow = yg + (int64_t)m * p.ldy;
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+              const int n = (wn * FN + j) * 16 + eq * 4;
+              const f32x4_t v = acc[j][i];
 #pragma unroll
               for (int rr = 0; rr < 4; ++rr)
                 if (n + rr < cols_valid) yrow[n + rr] = (bf16_t)v[rr];
@@ -243,7 +283,9 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
           }
         }
       }
-    }
+    };
+    if (nfm == FM) do_tile(std::false_type{});
+    else do_tile(std::true_type{});
   }
   if (GRP == 0) __syncthreads();  // pairs with group 1's last barrier
   wait_vm<0>();                   // trailing (never read) slab loads must land before the LDS is released

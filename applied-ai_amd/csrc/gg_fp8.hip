@@ -70,7 +70,7 @@ __global__ __launch_bounds__(NT) void gg_fp8_persistent(GgParams p) {
   const int K = p.K, N = p.N;  // K in elements = bytes
   const int n_tiles_n = moe_gg_cdiv(N, BN);
 
-  build_group_tables(p.m_sizes, p.G, p.M, BM, n_tiles_n, row_off, tile_off);
+  build_group_tables(p.m_sizes, p.G, p.M, BM, n_tiles_n, row_off, tile_off, p.skip_rows);
   const int total = uni(tile_off[p.G]);
   const int KT = K / 128;
 

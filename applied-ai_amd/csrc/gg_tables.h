@@ -17,8 +17,11 @@ DEVINL long long wave_incl_scan_i64(long long x) {
 
 // Must be called by every thread of the workgroup (it contains barriers).
 // row_off / tile_off: LDS arrays of G + 1 entries, G <= MOE_GG_MAX_GROUPS.
+// Groups with at most skip_rows rows keep their rows in row_off but get no tiles (another kernel
+// of the same call computes them).
 DEVINL void build_group_tables(const int32_t* __restrict__ m_sizes, int G, int M, int BM, int n_tiles_n,
-                               int32_t* row_off, int32_t* tile_off) {
+                               int32_t* row_off, int32_t* tile_off, int skip_rows = 0) {
+  auto tiles_of = [&](int rows) { return rows > skip_rows ? moe_gg_cdiv(rows, BM) * n_tiles_n : 0; };
   const int per = (G + 63) >> 6;
   if (wave_id() == 0) {
     const int g0 = lane_id() * per;
@@ -49,14 +52,14 @@ DEVINL void build_group_tables(const int32_t* __restrict__ m_sizes, int G, int M
     long long s = 0;
     for (int i = 0; i < per; ++i) {
       int g = g0 + i;
-      if (g < G) s += moe_gg_cdiv(row_off[g + 1] - row_off[g], BM) * n_tiles_n;
+      if (g < G) s += tiles_of(row_off[g + 1] - row_off[g]);
     }
     long long run = wave_incl_scan_i64(s) - s;
     for (int i = 0; i < per; ++i) {
       int g = g0 + i;
       if (g < G) {
         tile_off[g] = (int32_t)run;
-        run += moe_gg_cdiv(row_off[g + 1] - row_off[g], BM) * n_tiles_n;
+        run += tiles_of(row_off[g + 1] - row_off[g]);
       }
     }
     if (lane_id() == 63) tile_off[G] = (int32_t)run;

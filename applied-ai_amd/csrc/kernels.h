@@ -18,6 +18,7 @@ struct GgParams {
   int col_block;
   int vec_store;  // 1 when 8-byte aligned row segments can be stored as one dwordx2
   int xcds;       // number of XCDs the persistent grid is spread over
+  int skip_rows;  // tiled fp8 kernel: experts with at most this many rows are left to the streaming kernel
 };
 
 // block_m in {256, 128, 64}; the matching tile width is gg_bf16_tiled_block_n(block_m).
@@ -46,6 +47,10 @@ hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream)
 // fp8 e4m3 grouped GEMM (gg_fp8.hip). scale_mode 0: x_scale [M], w_scale [G*N]; 1: x_scale [M, K/128],
 // w_scale [G*N/128, K/128]. Needs K % 128 == 0 (and N % 128 == 0 in block mode), 16-byte aligned x, w.
 hipError_t gg_fp8_launch(const GgParams& p, int scale_mode, int num_wg, hipStream_t stream);
+// Streaming split-K kernel for experts with 1 .. gg_fp8_stream_max_rows() rows (gg_fp8_stream.hip); experts
+// outside that range are not touched. Pair it with gg_fp8_launch and p.skip_rows = gg_fp8_stream_max_rows().
+hipError_t gg_fp8_stream_launch(const GgParams& p, int scale_mode, hipStream_t stream);
+int gg_fp8_stream_max_rows();
 
 // Routing (routing.hip). E <= MOE_GG_MAX_ROUTE_EXPERTS; ids are int32.
 hipError_t route_topk_launch(const float* logits, int T, int E, int k, int32_t* ids, hipStream_t stream);
