@@ -154,13 +154,19 @@ int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* 
   p.xcds = di->xcds;
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
-  // Experts with a few rows are weight-streaming problems: they go to the split-K streaming kernel, the
+  // Experts with a few rows are weight-streaming problems: they go to the split-K streaming kernel, a
   // tiled kernel takes the rest. m_sizes stays on the device, so both are always launched; a kernel whose
   // share is empty exits after reading m_sizes.
-  hipError_t e = gg_fp8_stream_launch(p, scale_mode, (hipStream_t)stream);
+  int variant = g_variant[MOE_GG_OP_GG_FP8].load();
+  if (variant < 0) variant = MOE_GG_FP8_STREAM_PINGPONG;
+  hipStream_t s = (hipStream_t)stream;
+  if (variant == MOE_GG_FP8_TILED_128) return (int)gg_fp8_launch(p, scale_mode, num_wg, s);
+  if (variant != MOE_GG_FP8_STREAM_PINGPONG && variant != MOE_GG_FP8_STREAM_TILED) return MOE_GG_EINVAL;
+  hipError_t e = gg_fp8_stream_launch(p, scale_mode, s);
   if (e != hipSuccess) return (int)e;
   p.skip_rows = gg_fp8_stream_max_rows();
-  return (int)gg_fp8_launch(p, scale_mode, num_wg, (hipStream_t)stream);
+  if (variant == MOE_GG_FP8_STREAM_TILED) return (int)gg_fp8_launch(p, scale_mode, num_wg, s);
+  return (int)gg_fp8_pingpong_launch(p, scale_mode, num_wg, s);
 }
 
 int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros,

@@ -1,19 +1,26 @@
-// Persistent bf16 grouped GEMM for gfx950, "ping-pong" schedule.
+// Persistent grouped GEMM for gfx950, "ping-pong" schedule; bf16 or fp8 (OCP e4m3) operands, bf16 output.
 //
-// Replaces the reference's _kernel_grouped_gemm (dev/triton_groupGEMM/groupgemm.py:130-254):
+// bf16: replaces the reference's _kernel_grouped_gemm (dev/triton_groupGEMM/groupgemm.py:130-254):
 // y[off_g : off_g + m_g, :] = x[off_g : ...] @ w[g]^T with fp32 accumulation and bf16 output.
+// fp8, row-wise scales: _kernel_grouped_gemm_fp8_rowwise (groupgemm.py:269-404), scales applied in the
+// epilogue (groupgemm.py:374-384). fp8, block scales: 1 x 128 activation scales as produced by
+// kernels/triton/inference/fp8/float8_groupwise_quant.py:53-91 and 128 x 128 weight scales; a K step is
+// one 128-wide scale block whose MFMA result is multiplied by x_scale[m, kb] * w_scale[n / 128, kb]
+// before it is added to the accumulator.
 //
 // One 512-thread workgroup per CU walks the tile list of tile_sched.h; a tile is 256 x 256 outputs.
-// Per 64-wide K step a 256 x 64 activation slab and a 256 x 64 weight slab (32 KB each) are written
-// into one of two XOR-swizzled LDS stages by global_load_lds_dwordx4 (no VGPR staging) and consumed
-// by v_mfma_f32_16x16x32_bf16. The weight fragment is the MFMA "A" operand and the activation
-// fragment the "B" operand, so a lane ends up holding four consecutive output columns of one output
-// row and the epilogue stores 8 bytes per lane.
+// Per K step of 128 bytes per row (64 bf16 or 128 fp8 values) a 256-row activation slab and a 256-row
+// weight slab (32 KB each) are written into one of two XOR-swizzled LDS stages by
+// global_load_lds_dwordx4 (no VGPR staging) and consumed by v_mfma_f32_16x16x32_bf16 (two per fragment
+// pair and step) or v_mfma_f32_16x16x128_f8f6f4 (one; its 32-byte operand is the lane's two 16-byte
+// reads, the same for both operands, so the order of k inside the step does not matter). The weight
+// fragment is the MFMA "A" operand and the activation fragment the "B" operand, so a lane ends up
+// holding four consecutive output columns of one output row and the epilogue stores 8 bytes per lane.
 //
 // The eight waves form two groups of four (one wave of each group per SIMD); group 0 owns weight
 // rows 0-127 of the tile (W0), group 1 rows 128-255 (W1), both use all activation rows (X).
 // Every K step s has a load phase L(s) (all 24 fragment reads of the step into registers, plus all
-// slab-load instructions) and a compute phase C(s) (64 MFMAs, nothing else). The groups run half a
+// slab-load instructions) and a compute phase C(s) (the MFMAs, nothing else). The groups run half a
 // step apart, so that the matrix pipes always have exactly one wave per SIMD feeding them while
 // the other wave does the memory work; a workgroup barrier swaps the roles:
 //
@@ -28,6 +35,8 @@
 // Group 0 waits for its loads at the end of C(s); group 1 waits for W0(s+1) at the end of L(s), with
 // the W0(s+2) instructions it has just issued still in flight. The slab sequence runs straight
 // through tile boundaries, so the next tile's first slabs are in flight during the epilogue.
+// Block scales of step s+1 (256 activation scales, the tile's two weight-block scales) travel with
+// group 0's loads into a small per-stage LDS area.
 #include <type_traits>
 
 #include "common.h"
@@ -36,18 +45,30 @@
 
 namespace {
 
+typedef __attribute__((__vector_size__(8 * sizeof(int)))) int i32x8_t;
+
 constexpr int BM = 256, BN = 256;
 constexpr int NW = 8, NT = 64 * NW;
 constexpr int WM = 2;            // wave = wm + 2 * wn; group = wave >> 2 = wn >> 1
 constexpr int FM = 8, FN = 4;    // 16-row activation / weight fragments per wave
 constexpr int X_BYTES = BM * 128;
 constexpr int STAGE = (BM + BN) * 128;
+constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x 256 B of weight-block scales
 
-// 64 lanes x 16 B from global memory straight into LDS: lane l's 16 bytes land at lds_addr + 16 l.
-// Issued from inline assembly so that the compiler does not serialise the in-flight slab against
+// Operand kinds.
+constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2;
+
+// 64 lanes x 16 B (or 4 B) from global memory straight into LDS: lane l's bytes land at lds_addr + 16 l
+// (4 l). Issued from inline assembly so that the compiler does not serialise the in-flight slab against
 // the LDS reads of the slab being consumed; completion is tracked by hand with vmcnt.
 DEVINL void dma16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory");
+}
+DEVINL void dma4(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n"
                :
                : "s"(lds_addr), "v"(voff), "s"(sbase)
                : "memory");
@@ -80,23 +101,28 @@ struct Shared {
 struct Cursor {
   const char* xg;   // activation rows of the tile, K offset 0
   const char* wg;   // weight rows of the tile
+  const char* xsg;  // block mode: activation scales of the tile's first row, K block 0
+  const char* wsg;  // block mode: weight scales of the tile's first 128-column block, K block 0
   int x_last;       // last valid activation row of the tile (rows beyond it re-read this one)
   int w_last;       // last valid weight row of the tile
+  int ws_second;    // block mode: byte offset of the second column block's scales (0 if there is none)
   int round, kt, step;
 };
 
-template <int GRP>
+template <int GRP, int OP>
 DEVINL void run_group(const GgParams& p, const Shared& sh) {
+  constexpr bool FP8 = OP != OP_BF16;
+  constexpr bool BLOCK = OP == OP_FP8_BLOCK;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1;
   const int wn = wave >> 1;
   const int gw = wave & 3;  // wave index inside its group
-  const int K = p.K, N = p.N;
-  const int KT = K / 64;
+  const int N = p.N;
+  const uint32_t KROW = (uint32_t)p.K * (FP8 ? 1u : 2u);  // bytes per operand row
+  const int KT = (int)(KROW / 128u);
   const int nwg = gridDim.x;
-  const uint32_t K2 = (uint32_t)K * 2u;
 
   // Slab-load geometry: an instruction fills 8 rows (1 KB of LDS); lane -> row lane / 8, physical
   // 16-byte slot lane % 8, which must hold logical chunk slot ^ ((row >> 1) & 7). Inside a group the
@@ -104,6 +130,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   const int d_r = lane >> 3;
   const uint32_t d_c16 = (uint32_t)(((lane & 7) ^ (((gw & 1) << 2) | (lane >> 4))) << 4);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)sh.lds;
+  const uint32_t lds_scale = lds_base + 2 * STAGE;
 
   // Fragment reads: row = frag * 16 + lane % 16, chunk = kk * 4 + lane / 16 (swizzled).
   const int fr = lane & 15, fq = lane >> 4;
@@ -121,8 +148,13 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const int m0 = t.tm * BM, n0 = t.tn * BN;
     c.x_last = min(t.rows - m0, BM) - 1;
     c.w_last = min(N - n0, BN) - 1;
-    c.xg = uni_ptr(xp + (int64_t)(t.row0 + m0) * K2);
-    c.wg = uni_ptr(wp + ((int64_t)t.g * N + n0) * K2);
+    c.xg = uni_ptr(xp + (int64_t)(t.row0 + m0) * KROW);
+    c.wg = uni_ptr(wp + ((int64_t)t.g * N + n0) * KROW);
+    if (BLOCK) {
+      c.xsg = uni_ptr((const char*)(p.x_scale + (int64_t)(t.row0 + m0) * KT));
+      c.wsg = uni_ptr((const char*)(p.w_scale + (((int64_t)t.g * N + n0) / 128) * KT));
+      c.ws_second = n0 + 128 < N ? KT * 4 : 0;
+    }
   };
   auto cursor_next = [&]() {
     ++c.step;
@@ -134,19 +166,34 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   // Block b (8 rows) of the cursor slab's activation / weight rows.
   auto dma_x = [&](int b) {
     if (b * 8 > c.x_last) return;  // block entirely below the tile's last row: its fragments are never used
-    const uint32_t off = (uint32_t)min(b * 8 + d_r, c.x_last) * K2 + d_c16;
+    const uint32_t off = (uint32_t)min(b * 8 + d_r, c.x_last) * KROW + d_c16;
     dma16(c.xg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + b * 1024);
   };
   auto dma_w = [&](int b) {
-    const uint32_t off = (uint32_t)min(b * 8 + d_r, c.w_last) * K2 + d_c16;
+    const uint32_t off = (uint32_t)min(b * 8 + d_r, c.w_last) * KROW + d_c16;
     dma16(c.wg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + X_BYTES + b * 1024);
   };
+  // Block scales of the cursor slab: wave gw of group 0 fetches the activation scales of rows
+  // 64 gw .. 64 gw + 63 (one per lane) and a private copy of the two weight-block scales (lanes 0-31 the
+  // first column block, lanes 32-63 the second).
+  auto dma_xscale = [&]() {
+    const uint32_t off = (uint32_t)min(gw * 64 + lane, c.x_last) * (uint32_t)(KT * 4);
+    dma4(c.xsg + c.kt * 4, off, lds_scale + (c.step & 1) * SCALE_BYTES + gw * 256);
+  };
+  auto dma_wscale = [&]() {
+    const uint32_t off = lane < 32 ? 0u : (uint32_t)c.ws_second;
+    dma4(c.wsg + c.kt * 4, off, lds_scale + (c.step & 1) * SCALE_BYTES + 1024 + gw * 256);
+  };
   // Load instruction idx of this wave for the cursor slab; the last one advances the cursor.
-  // Group 0: 8 activation blocks (idx 0-7) + 4 blocks of W1 (idx 8-11). Group 1: 4 blocks of W0.
-  constexpr int NDMA = GRP == 0 ? 12 : 4;
+  // Group 0: 8 activation blocks (idx 0-7), 4 blocks of W1 (idx 8-11), block mode: the scales (12, 13).
+  // Group 1: 4 blocks of W0.
+  constexpr int NDMA = GRP == 0 ? (BLOCK ? 14 : 12) : 4;
   auto dma_one = [&](int idx) {
     if (GRP == 0) {
-      if (idx < 8) dma_x(idx * 4 + gw); else dma_w(16 + (idx - 8) * 4 + gw);
+      if (idx < 8) dma_x(idx * 4 + gw);
+      else if (idx < 12) dma_w(16 + (idx - 8) * 4 + gw);
+      else if (idx == 12) dma_xscale();
+      else dma_wscale();
     } else {
       dma_w(idx * 4 + gw);
     }
@@ -177,7 +224,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     // alternately to wm = 0 / 1, so a short tile shortens every wave's C phase alike).
     const int nfm = min(FM, max(0, ((rows_valid + 15) / 16 - wm + WM - 1) / WM));
 
-    // The tile body exists twice: for full-height tiles (all 64 MFMAs per step, no branches) and for
+    // The tile body exists twice: for full-height tiles (all MFMAs of a step, no branches) and for
     // short tiles, which skip the MFMAs of activation fragments that hold no valid row. Each copy has
     // its own accumulators, so the two K loops do not have to agree on a register assignment.
     auto do_tile = [&](auto short_tag) {
@@ -194,43 +241,71 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         // tile columns (wn * FN + j) * 16 .. + 15.
         const char* xs = sh.lds + (step & 1) * STAGE + wm * 2048;
         const char* ws = sh.lds + (step & 1) * STAGE + X_BYTES + wn * (FN * 2048);
-        bf16x8_t wf[2][FN], xf[2][FM];
-        constexpr int READS_PER_DMA = 24 / NDMA;
+        u32x4_t wf[2][FN], xf[2][FM];
+        int issued = 0;
 #pragma unroll
         for (int q = 0; q < 24; ++q) {
-          if (q % READS_PER_DMA == 0) {
+          // spread the NDMA load instructions evenly over the 24 reads
+          if (issued < NDMA && q * NDMA >= issued * 24) {
             __builtin_amdgcn_sched_barrier(0);
-            dma_one(q / READS_PER_DMA);
+            dma_one(issued);
+            ++issued;
+            if (issued < NDMA && q * NDMA >= issued * 24) { dma_one(issued); ++issued; }
             __builtin_amdgcn_sched_barrier(0);
           }
           const int kk = q / 12, f = q % 12;
           const int ro = kk ? (rd0 ^ 64) : rd0;
-          if (f < FN) wf[kk][f] = *(const bf16x8_t*)(ws + f * 2048 + ro);
-          else xf[kk][f - FN] = *(const bf16x8_t*)(xs + (f - FN) * (WM * 2048) + ro);
+          if (f < FN) wf[kk][f] = *(const u32x4_t*)(ws + f * 2048 + ro);
+          else xf[kk][f - FN] = *(const u32x4_t*)(xs + (f - FN) * (WM * 2048) + ro);
+        }
+        float sc[FM];
+        if (BLOCK) {
+          const float* sl = (const float*)(sh.lds + 2 * STAGE + (step & 1) * SCALE_BYTES);
+          const float sw = sl[256 + (wn >> 1) * 32];  // the wave's 64 columns lie in column block wn / 2 of the tile's two
+#pragma unroll
+          for (int i = 0; i < FM; ++i) sc[i] = sl[(i * WM + wm) * 16 + fr] * sw;
         }
         __builtin_amdgcn_sched_barrier(0);
         wait_lgkm0();  // all of slab `step` is in this wave's registers
         if (GRP == 1) wait_vm<NDMA>();  // W0(step + 1) has landed; W0(step + 2) may still be in flight
         __syncthreads();
-        // ---------------- C phase: 64 MFMAs ----------------
+        // ---------------- C phase: MFMAs only ----------------
         __builtin_amdgcn_s_setprio(1);
+        // bf16: one of the two MFMAs (K half kk) of fragment pair (j, i); fp8: its single MFMA.
+        auto mma = [&](int j, int i, int kk) {
+          if (!FP8) {
+            acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf[kk][j]),
+                                                               __builtin_bit_cast(bf16x8_t, xf[kk][i]), acc[j][i], 0, 0, 0);
+          } else {
+            const i32x8_t a = {(int)wf[0][j][0], (int)wf[0][j][1], (int)wf[0][j][2], (int)wf[0][j][3],
+                               (int)wf[1][j][0], (int)wf[1][j][1], (int)wf[1][j][2], (int)wf[1][j][3]};
+            const i32x8_t b = {(int)xf[0][i][0], (int)xf[0][i][1], (int)xf[0][i][2], (int)xf[0][i][3],
+                               (int)xf[1][i][0], (int)xf[1][i][1], (int)xf[1][i][2], (int)xf[1][i][3]};
+            if (BLOCK) {
+              const f32x4_t z = {0.f, 0.f, 0.f, 0.f};
+              const f32x4_t d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, z, 0, 0, 0, 0, 0, 0);
+              acc[j][i] += d * sc[i];
+            } else {
+              acc[j][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[j][i], 0, 0, 0, 0, 0, 0);
+            }
+          }
+        };
+        constexpr int NKK = FP8 ? 1 : 2;
         if (!SHORT) {
 #pragma unroll
-          for (int kk = 0; kk < 2; ++kk)
+          for (int kk = 0; kk < NKK; ++kk)
 #pragma unroll
             for (int j = 0; j < FN; ++j)
 #pragma unroll
-              for (int i = 0; i < FM; ++i)
-                acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[kk][j], xf[kk][i], acc[j][i], 0, 0, 0);
+              for (int i = 0; i < FM; ++i) mma(j, i, kk);
         } else {
 #pragma unroll
           for (int i = 0; i < FM; ++i) {
             if (i < nfm) {
 #pragma unroll
-              for (int kk = 0; kk < 2; ++kk)
+              for (int kk = 0; kk < NKK; ++kk)
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
-                  acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[kk][j], xf[kk][i], acc[j][i], 0, 0, 0);
+                for (int j = 0; j < FN; ++j) mma(j, i, kk);
             }
           }
         }
@@ -242,23 +317,33 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
 
       // Epilogue: lane holds y[m][n .. n+3] for m = (i * WM + wm) * 16 + lane % 16,
       // n = (wn * FN + j) * 16 + 4 * (lane / 16). Addresses are a per-fragment uniform base plus one
-      // 32-bit lane offset, so nothing has to stay in registers across the K loop.
-      // The lane indices pass through an empty asm so that the address arithmetic is redone here for
-      // every tile instead of being hoisted out of the tile loop, where it would occupy (and spill)
-      // registers during the K loop.
+      // 32-bit lane offset. The lane indices pass through an empty asm so that the address arithmetic
+      // is redone here for every tile instead of being hoisted out of the tile loop, where it would
+      // occupy (and spill) registers during the K loop.
       bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + (int64_t)t.g * p.col_block + n0;
       int er = fr, eq = fq;
       asm volatile("" : "+v"(er), "+v"(eq));
+      // Row-wise fp8 scales (groupgemm.py:374-384): y *= x_scale[m] * w_scale[g * N + n].
+      const float* xrow_scale = OP == OP_FP8_ROW ? p.x_scale + t.row0 + m0 : nullptr;
+      const float* wcol_scale = OP == OP_FP8_ROW ? p.w_scale + (int64_t)t.g * N + n0 : nullptr;
       if (p.vec_store && cols_valid == BN && p.ldy < (1 << 24)) {
         const uint32_t voff = (uint32_t)er * (uint32_t)p.ldy + (uint32_t)(wn * FN * 16 + eq * 4);
+        f32x4_t bs[FN];
+        if (OP == OP_FP8_ROW) {
+#pragma unroll
+          for (int j = 0; j < FN; ++j) bs[j] = *(const f32x4_t*)(wcol_scale + (wn * FN + j) * 16 + eq * 4);
+        }
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
           const int mrow = (i * WM + wm) * 16;
           bf16_t* ybase = yg + (int64_t)mrow * p.ldy;  // uniform
           if (mrow + er < rows_valid) {
+            float am = 1.f;
+            if (OP == OP_FP8_ROW) am = xrow_scale[mrow + er];
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
-              const f32x4_t v = acc[j][i];
+              f32x4_t v = acc[j][i];
+              if (OP == OP_FP8_ROW) v = v * am * bs[j];
               u32x2_t o;
               o[0] = pack_bf16x2(v[0], v[1]);
               o[1] = pack_bf16x2(v[2], v[3]);
@@ -272,13 +357,19 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
           const int m = (i * WM + wm) * 16 + er;
           if (m < rows_valid) {
             bf16_t* yrow = yg + (int64_t)m * p.ldy;
+            float am = 1.f;
+            if (OP == OP_FP8_ROW) am = xrow_scale[m];
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
               const int n = (wn * FN + j) * 16 + eq * 4;
               const f32x4_t v = acc[j][i];
 #pragma unroll
               for (int rr = 0; rr < 4; ++rr)
-                if (n + rr < cols_valid) yrow[n + rr] = (bf16_t)v[rr];
+                if (n + rr < cols_valid) {
+                  float o = v[rr];
+                  if (OP == OP_FP8_ROW) o = o * am * wcol_scale[n + rr];
+                  yrow[n + rr] = (bf16_t)o;
+                }
             }
           }
         }
@@ -291,12 +382,13 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   wait_vm<0>();                   // trailing (never read) slab loads must land before the LDS is released
 }
 
-__global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) {
-  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
+template <int OP>
+DEVINL void pingpong_body(const GgParams& p) {
+  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + (OP == OP_FP8_BLOCK ? 2 * SCALE_BYTES : 0)];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t tile_off[MOE_GG_MAX_GROUPS + 1];
 
-  build_group_tables(p.m_sizes, p.G, p.M, BM, moe_gg_cdiv(p.N, BN), row_off, tile_off);
+  build_group_tables(p.m_sizes, p.G, p.M, BM, moe_gg_cdiv(p.N, BN), row_off, tile_off, p.skip_rows);
   const int total = uni(tile_off[p.G]);
   const int nwg = gridDim.x;
   // Tiles of this workgroup: rounds 0 .. n_my - 1 (tile ids grow with the round).
@@ -306,13 +398,23 @@ __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) {
 
   Shared sh{row_off, tile_off, lds, n_my};
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
-  if (grp == 0) run_group<0>(p, sh);
-  else run_group<1>(p, sh);
+  if (grp == 0) run_group<0, OP>(p, sh);
+  else run_group<1, OP>(p, sh);
 }
+
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_body<OP_BF16>(p); }
+__global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise(GgParams p) { pingpong_body<OP_FP8_ROW>(p); }
+__global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpong_body<OP_FP8_BLOCK>(p); }
 
 }  // namespace
 
 hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream) {
   hipLaunchKernelGGL(gg_bf16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t gg_fp8_pingpong_launch(const GgParams& p, int scale_mode, int num_wg, hipStream_t stream) {
+  if (scale_mode == 0) hipLaunchKernelGGL(gg_fp8_pingpong_rowwise, dim3(num_wg), dim3(NT), 0, stream, p);
+  else hipLaunchKernelGGL(gg_fp8_pingpong_block, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }

@@ -24,8 +24,10 @@ struct GgParams {
 // block_m in {256, 128, 64}; the matching tile width is gg_bf16_tiled_block_n(block_m).
 hipError_t gg_bf16_tiled_launch(const GgParams& p, int block_m, int num_wg, hipStream_t stream);
 int gg_bf16_tiled_block_n(int block_m);
-// 256 x 256 tiles, ping-pong schedule.
+// 256 x 256 tiles, ping-pong schedule (gg_pingpong.hip); the fp8 form takes the scale modes of gg_fp8_launch
+// and honours p.skip_rows.
 hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream);
+hipError_t gg_fp8_pingpong_launch(const GgParams& p, int scale_mode, int num_wg, hipStream_t stream);
 hipError_t gg_bf16_generic_launch(const GgParams& p, hipStream_t stream);
 // Small-M split-K kernel; nf = 16-row weight fragments per wave (2 or 4), mf = 16-row activation
 // fragments per pass (1, 2 or 4). Needs K % 128 == 0 and 16-byte aligned x and w.

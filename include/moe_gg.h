@@ -150,6 +150,11 @@ int moe_gg_fp8_groupwise_quant(const void* in, int dtype, void* out, float* scal
 #define MOE_GG_GG_TILED_64 3     /* 64x128 tiles */
 #define MOE_GG_GG_GENERIC 4      /* one thread per output element, any shape / alignment */
 #define MOE_GG_GG_DECODE 5       /* small-M path: weights streamed once, split-K inside the workgroup */
+#define MOE_GG_OP_GG_FP8 1
+/* variants of MOE_GG_OP_GG_FP8 */
+#define MOE_GG_FP8_TILED_128 0       /* 128x128 tiles for every expert */
+#define MOE_GG_FP8_STREAM_PINGPONG 1 /* experts with <= 64 rows: streaming split-K kernel; others: 256x256 ping-pong */
+#define MOE_GG_FP8_STREAM_TILED 2    /* experts with <= 64 rows: streaming split-K kernel; others: 128x128 tiles */
 int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,
