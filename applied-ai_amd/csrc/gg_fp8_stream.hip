@@ -26,7 +26,9 @@ typedef __attribute__((__vector_size__(8 * sizeof(int)))) int i32x8_t;
 template <int MODE, int NF, int MF, int DEPTH>
 __global__ __launch_bounds__(256) void gg_fp8_stream(GgParams p, int max_rows) {
   constexpr int WAVES = 4;
-  __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MF][256];
+  constexpr int RP = MF >= 2 ? 2 : 1;          // the reduction runs in RP passes over MF / RP activation fragments,
+  constexpr int MFP = MF / RP;                 // which keeps the LDS footprint at 32 KB and three workgroups per CU
+  __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MFP][256];
   __shared__ int s_row0, s_rows;
 
   const int tid = threadIdx.x;
@@ -136,34 +138,39 @@ __global__ __launch_bounds__(256) void gg_fp8_stream(GgParams p, int max_rows) {
   // Split-K reduction through LDS, then scales (row-wise mode) and the store: lane holds y[m][n .. n+3],
   // m = i * 16 + lane % 16, n = n0 + j * 16 + 4 * (lane / 16).
 #pragma unroll
-  for (int j = 0; j < NF; ++j)
+  for (int rp = 0; rp < RP; ++rp) {
+    if (rp * MFP >= nmf) break;
+    if (rp) __syncthreads();
 #pragma unroll
-    for (int i = 0; i < MF; ++i) *(f32x4_t*)&red[wave][j * MF + i][lane * 4] = acc[j][i];
-  __syncthreads();
-  for (int f = wave; f < NF * MF; f += WAVES) {
-    const int j = f / MF, i = f % MF;
-    const int m = i * 16 + fr;
-    if (m >= rows) continue;
-    f32x4_t v = *(const f32x4_t*)&red[0][f][lane * 4];
+    for (int j = 0; j < NF; ++j)
 #pragma unroll
-    for (int w2 = 1; w2 < WAVES; ++w2) v += *(const f32x4_t*)&red[w2][f][lane * 4];
-    const int n = n0 + j * 16 + fq * 4;
-    if (MODE == 0) {
-      const float am = p.x_scale[row0 + m];
-      const float* bs = p.w_scale + (int64_t)g * N;
+      for (int i = 0; i < MFP; ++i) *(f32x4_t*)&red[wave][j * MFP + i][lane * 4] = acc[j][rp * MFP + i];
+    __syncthreads();
+    for (int f = wave; f < NF * MFP; f += WAVES) {
+      const int j = f / MFP, i = rp * MFP + f % MFP;
+      const int m = i * 16 + fr;
+      if (m >= rows) continue;
+      f32x4_t v = *(const f32x4_t*)&red[0][f][lane * 4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) v[r] = v[r] * am * bs[min(n + r, N - 1)];
-    }
-    bf16_t* yrow = (bf16_t*)p.y + (int64_t)(row0 + m) * p.ldy + (int64_t)g * p.col_block;
-    if (p.vec_store && n + 3 < N) {
-      u32x2_t o;
-      o[0] = pack_bf16x2(v[0], v[1]);
-      o[1] = pack_bf16x2(v[2], v[3]);
-      *(u32x2_t*)(yrow + n) = o;
-    } else {
+      for (int w2 = 1; w2 < WAVES; ++w2) v += *(const f32x4_t*)&red[w2][f][lane * 4];
+      const int n = n0 + j * 16 + fq * 4;
+      if (MODE == 0) {
+        const float am = p.x_scale[row0 + m];
+        const float* bs = p.w_scale + (int64_t)g * N;
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (n + r < N) yrow[n + r] = (bf16_t)v[r];
+        for (int r = 0; r < 4; ++r) v[r] = v[r] * am * bs[min(n + r, N - 1)];
+      }
+      bf16_t* yrow = (bf16_t*)p.y + (int64_t)(row0 + m) * p.ldy + (int64_t)g * p.col_block;
+      if (p.vec_store && n + 3 < N) {
+        u32x2_t o;
+        o[0] = pack_bf16x2(v[0], v[1]);
+        o[1] = pack_bf16x2(v[2], v[3]);
+        *(u32x2_t*)(yrow + n) = o;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N) yrow[n + r] = (bf16_t)v[r];
+      }
     }
   }
 }
@@ -179,7 +186,9 @@ hipError_t launch(const GgParams& p, hipStream_t stream) {
 
 int gg_fp8_stream_max_rows() { return 64; }
 
+// One K step of loads in flight per wave and three workgroups per CU measured best (more steps in flight
+// cost registers, hence resident waves, and were slower).
 hipError_t gg_fp8_stream_launch(const GgParams& p, int scale_mode, hipStream_t stream) {
-  if (scale_mode == 0) return launch<0, 4, 4, 2>(p, stream);
-  return launch<1, 4, 4, 2>(p, stream);
+  if (scale_mode == 0) return launch<0, 4, 4, 1>(p, stream);
+  return launch<1, 4, 4, 1>(p, stream);
 }
