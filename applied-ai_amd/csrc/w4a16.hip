@@ -183,14 +183,19 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
 }
 
 // group_size == 128 (four K steps per group). Every load - qweight, activations, scales, zeros - is
-// issued two groups (eight K steps) ahead of its use and consumed in issue order, because vector
-// memory loads return in order: a late-issued small load would otherwise wait for all the weight
-// loads queued before it.
-template <bool FP16, int MF, int GA>  // GA = groups kept in flight
-__global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_g128(W4Params p) {
+// issued GA groups ahead of its use and consumed in issue order, because vector memory loads return in
+// order: a late-issued small load would otherwise wait for all the weight loads queued before it.
+//
+// Operand roles are the other way round than in the kernel above: the activation fragment is the MFMA
+// "A" operand and the unpacked weights the "B" operand, so a lane ends up with output rows
+// 4 * (lane / 16) + r of the four adjacent columns n0 + 4 * (lane % 16) + j of its own qweight words. It
+// then needs just four scales and four zero points per group (one 8-byte and one 4-byte load), and the
+// fold costs a quarter of the vector instructions of the 16-columns-per-lane layout.
+template <bool FP16, int MF, int GA, int NWAVES>  // GA = groups kept in flight
+__global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
   using E = Elem<FP16>;
   constexpr int SPG = 4, D = SPG * GA;
-  __shared__ __attribute__((aligned(16))) float red[WAVES][MF][64 * 16];
+  __shared__ __attribute__((aligned(16))) float red[NWAVES][MF][16 * 64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -199,28 +204,29 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_g128(W4Params p) {
   const int N = p.N, K = p.K, M = p.M;
   const int n0 = blockIdx.x * 64;
   const int ngroups = K / 128;
-  const int my_groups = ngroups > wave ? (ngroups - wave + WAVES - 1) / WAVES : 0;
+  const int my_groups = ngroups > wave ? (ngroups - wave + NWAVES - 1) / NWAVES : 0;
   const int steps = my_groups * SPG;
-  auto kstep = [&](int t) { return ((t / SPG) * WAVES + wave) * SPG + t % SPG; };
+  auto kstep = [&](int t) { return ((t / SPG) * NWAVES + wave) * SPG + t % SPG; };
 
-  const int32_t* qw = p.qweight + n0 + 4 * fr;
-  const int ocol = n0 + 16 * fq;
-  const uint16_t* sc = (const uint16_t*)p.scales + ocol;
-  const int32_t* zp = p.qzeros + ocol / 8;
+  const int32_t* qw = p.qweight + n0 + 4 * fr;          // k-word row 4 * step + fq, columns n0 + 4 fr .. + 3
+  const uint16_t* sc = (const uint16_t*)p.scales + n0 + 4 * fr;
+  const int32_t* zp = p.qzeros + (n0 + 4 * fr) / 8;
+  const int zshift = 16 * (fr & 1);                     // the lane's four zero nibbles inside the word
 
   for (int mb = 0; mb < M; mb += 16 * MF) {
     const uint16_t* arow[MF];
 #pragma unroll
     for (int i = 0; i < MF; ++i) arow[i] = (const uint16_t*)p.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
 
-    f32x4_t total[MF][4];
+    f32x4_t total[MF][4];  // [row fragment i][column j]: rows mb + 16 i + 4 fq + r
 #pragma unroll
     for (int i = 0; i < MF; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) total[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    u32x4_t wb[D], xr[D][MF], s0[GA], s1[GA];
-    u32x2_t zw[GA];
+    u32x4_t wb[D], xr[D][MF];
+    u32x2_t sg[GA];
+    uint32_t zg[GA];
     auto load_step = [&](int d, int t) {
       const int ks = kstep(t);
       wb[d] = *(const u32x4_t*)(qw + (int64_t)(ks * 4 + fq) * N);
@@ -228,10 +234,9 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_g128(W4Params p) {
       for (int i = 0; i < MF; ++i) xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
     };
     auto load_group = [&](int q, int gi) {  // gi = index among this wave's groups
-      const int64_t g = (int64_t)gi * WAVES + wave;
-      s0[q] = *(const u32x4_t*)(sc + g * N);
-      s1[q] = *(const u32x4_t*)(sc + g * N + 8);
-      zw[q] = *(const u32x2_t*)(zp + g * (N / 8));
+      const int64_t g = (int64_t)gi * NWAVES + wave;
+      sg[q] = *(const u32x2_t*)(sc + g * N);
+      zg[q] = (uint32_t)zp[g * (N / 8)];
     };
 #pragma unroll
     for (int q = 0; q < GA; ++q) {
@@ -241,79 +246,76 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_g128(W4Params p) {
       if (q < my_groups) load_group(q, q);
     }
 
-    f32x4_t accg[MF][4], accs[MF];
-    for (int t0 = 0; t0 < steps; t0 += D) {
+    for (int g0 = 0; g0 < my_groups; g0 += GA) {
 #pragma unroll
-      for (int d = 0; d < D; ++d) {
-        const int t = t0 + d;
-        if (t < steps) {
-          if (d % SPG == 0) {
-#pragma unroll
-            for (int i = 0; i < MF; ++i) {
-#pragma unroll
-              for (int j = 0; j < 4; ++j) accg[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-              accs[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            }
-          }
-          u32x4_t xb[MF];
+      for (int q = 0; q < GA; ++q) {
+        const int gi = g0 + q;  // index among this wave's groups; its loads sit in ring slots q * SPG .. + 3
+        if (gi < my_groups) {
+          const bool more = gi + GA < my_groups;
+          f32x4_t accg[MF][4], accs[MF];
 #pragma unroll
           for (int i = 0; i < MF; ++i) {
-            const u32x4_t v = xr[d][i];
-            xb[i][0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // k 0, 4
-            xb[i][1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // k 1, 5
-            xb[i][2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // k 2, 6
-            xb[i][3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // k 3, 7
+#pragma unroll
+            for (int j = 0; j < 4; ++j) accg[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            accs[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
           }
-          const u32x4_t w4 = wb[d];
-          if (t + D < steps) load_step(d, t + D);
+#pragma unroll
+          for (int e = 0; e < SPG; ++e) {
+            const int d = q * SPG + e;
+            u32x4_t xb[MF];
+#pragma unroll
+            for (int i = 0; i < MF; ++i) {
+              const u32x4_t v = xr[d][i];
+              xb[i][0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // k 0, 4
+              xb[i][1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // k 1, 5
+              xb[i][2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // k 2, 6
+              xb[i][3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // k 3, 7
+            }
+            const u32x4_t w4 = wb[d];
+            if (more) load_step(d, (gi + GA) * SPG + e);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              u32x4_t bf;
+#pragma unroll
+              for (int e2 = 0; e2 < 4; ++e2) bf[e2] = ((w4[j] >> (4 * e2)) & 0x000F000Fu) | E::MAGIC;
+#pragma unroll
+              for (int i = 0; i < MF; ++i) accg[i][j] = E::mfma(xb[i], bf, accg[i][j]);
+            }
+            const u32x4_t ones = {E::ONES, E::ONES, E::ONES, E::ONES};
+#pragma unroll
+            for (int i = 0; i < MF; ++i) accs[i] = E::mfma(xb[i], ones, accs[i]);
+          }
+          const u32x2_t sq = sg[q];
+          const uint32_t zq = zg[q] >> zshift;
+          if (more) load_group(q, gi + GA);
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            u32x4_t af;
+            const uint32_t sw = sq[j >> 1];
+            const float s = E::to_f32((uint16_t)((j & 1) ? (sw >> 16) : (sw & 0xFFFFu)));
+            const uint32_t z = (zq >> (4 * j)) & 0xFu;
+            const float zz = E::BIAS + (float)(int)(z + (uint32_t)p.zero_offset);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) af[e] = ((w4[j] >> (4 * e)) & 0x000F000Fu) | E::MAGIC;
-#pragma unroll
-            for (int i = 0; i < MF; ++i) accg[i][j] = E::mfma(af, xb[i], accg[i][j]);
-          }
-          const u32x4_t ones = {E::ONES, E::ONES, E::ONES, E::ONES};
-#pragma unroll
-          for (int i = 0; i < MF; ++i) accs[i] = E::mfma(ones, xb[i], accs[i]);
-
-          if (d % SPG == SPG - 1) {
-            const int q = d / SPG;
-            const u32x4_t sa = s0[q], sb = s1[q];
-            const u32x2_t zq = zw[q];
-            if (t / SPG + GA < my_groups) load_group(q, t / SPG + GA);
-#pragma unroll
-            for (int ii = 0; ii < 4; ++ii)
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                const int c = 4 * ii + j;
-                const uint32_t sw = c < 8 ? sa[c >> 1] : sb[(c - 8) >> 1];
-                const float s = E::to_f32((uint16_t)((c & 1) ? (sw >> 16) : (sw & 0xFFFFu)));
-                const uint32_t z = (zq[c >> 3] >> (4 * (c & 7))) & 0xFu;
-                const float zz = E::BIAS + (float)(int)(z + (uint32_t)p.zero_offset);
-#pragma unroll
-                for (int i = 0; i < MF; ++i) total[i][j][ii] += s * (accg[i][j][ii] - zz * accs[i][ii]);
-              }
+            for (int i = 0; i < MF; ++i) total[i][j] += s * (accg[i][j] - zz * accs[i]);
           }
         }
       }
     }
 
+    // Cross-wave (split-K) reduction in a fixed order: red[wave][i][m_local * 64 + col_local].
 #pragma unroll
     for (int i = 0; i < MF; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int ii = 0; ii < 4; ++ii) red[wave][i][fr * 64 + 16 * fq + 4 * ii + j] = total[i][j][ii];
+      for (int r = 0; r < 4; ++r)
+        *(f32x4_t*)&red[wave][i][(4 * fq + r) * 64 + 4 * fr] = f32x4_t{total[i][0][r], total[i][1][r], total[i][2][r], total[i][3][r]};
     __syncthreads();
-    for (int o = tid; o < MF * 16 * 64; o += 64 * WAVES) {
-      const int i = o / 1024, rem = o % 1024;
-      const int m = mb + i * 16 + rem / 64, n = n0 + rem % 64;
+    const int rows_here = min(M - mb, 16 * MF);
+    for (int o = tid; o < rows_here * 64; o += 64 * NWAVES) {
+      const int ml = o / 64, col = o % 64;
+      const int i = ml / 16, rem = (ml % 16) * 64 + col;
       float v = red[0][i][rem];
 #pragma unroll
-      for (int w2 = 1; w2 < WAVES; ++w2) v += red[w2][i][rem];
-      if (m < M && n < N) ((uint16_t*)p.c)[(int64_t)m * N + n] = E::from_f32(v);
+      for (int w2 = 1; w2 < NWAVES; ++w2) v += red[w2][i][rem];
+      if (n0 + col < N) ((uint16_t*)p.c)[(int64_t)(mb + ml) * N + n0 + col] = E::from_f32(v);
     }
     __syncthreads();
   }
@@ -322,9 +324,10 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_g128(W4Params p) {
 template <bool FP16>
 hipError_t launch(const W4Params& p, hipStream_t stream) {
   dim3 grid((p.N + 63) / 64), block(64 * WAVES);
-  // M <= 16: one activation fragment, everything prefetched (group size 128 only). Larger M keeps up
-  // to four activation fragments per pass so that the weights are unpacked once per four fragments.
-  if (p.M <= 16 && p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 2>), grid, block, 0, stream, p);
+  // M <= 16 and group size 128: one activation fragment, all loads issued one group ahead (deeper queues
+  // and more waves measured slower). Larger M keeps up to four activation fragments per pass so that the
+  // weights are unpacked once per four fragments.
+  if (p.M <= 16 && p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES>), grid, block, 0, stream, p);
   else if (p.M <= 16) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 1>), grid, block, 0, stream, p);
   else if (p.M <= 32) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 2>), grid, block, 0, stream, p);
   else hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 4>), grid, block, 0, stream, p);
