@@ -39,6 +39,9 @@ SIGNATURES = {
     "moe_gg_route_topk": (_c_int, [_c_void_p, _c_i64, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "moe_gg_route_group": (_c_int, [_c_void_p, _c_i64, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "moe_gg_gather_rows": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_i64, _c_i64, _c_void_p]),
+    "moe_gg_silu_and_mul": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
+    "moe_gg_invert_perm": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_void_p, _c_void_p]),
+    "moe_gg_combine_topk": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_i64, _c_int, _c_int, _c_i64, _c_void_p]),
     "moe_gg_fp8_groupwise_quant": (_c_int, [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_i64, _c_void_p]),
     "moe_gg_host_enumerate_tiles": (
         _c_int,

@@ -217,6 +217,37 @@ int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int
   return (int)gather_rows_launch(x, perm, k, out, (int)n, row_bytes, (hipStream_t)stream);
 }
 
+int moe_gg_silu_and_mul(const void* in, void* out, int64_t rows, int n, void* stream) {
+  if (rows < 0 || n < 0) return MOE_GG_EINVAL;
+  if (rows == 0 || n == 0) return MOE_GG_OK;
+  if (!in || !out) return MOE_GG_EINVAL;
+  if (n % 8 != 0) return MOE_GG_ESHAPE;
+  if (!aligned(in, 16) || !aligned(out, 16)) return MOE_GG_EALIGN;
+  return (int)silu_and_mul_launch(in, out, rows, n, (hipStream_t)stream);
+}
+
+int moe_gg_invert_perm(const int32_t* perm, int32_t* inv, int64_t n, const int32_t* n_valid, void* stream) {
+  if (n < 0) return MOE_GG_EINVAL;
+  if (n == 0) return MOE_GG_OK;
+  if (!perm || !inv) return MOE_GG_EINVAL;
+  if (n > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  return (int)invert_perm_launch(perm, inv, (int)n, n_valid, (hipStream_t)stream);
+}
+
+int moe_gg_combine_topk(const void* y, const int32_t* inv, const void* weights, int weights_dtype, void* out,
+                        int64_t T, int k, int d, int64_t n_rows, void* stream) {
+  if (T < 0 || k <= 0 || d < 0 || n_rows < 0) return MOE_GG_EINVAL;
+  if (weights_dtype != MOE_GG_DTYPE_FP32 && weights_dtype != MOE_GG_DTYPE_BF16) return MOE_GG_EINVAL;
+  if (T == 0 || d == 0) return MOE_GG_OK;
+  if (!y || !inv || !weights || !out) return MOE_GG_EINVAL;
+  if (d % 8 != 0) return MOE_GG_ESHAPE;
+  if (T > INT32_MAX || n_rows > INT32_MAX || T * k > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (!aligned(y, 16) || !aligned(out, 16) || !aligned(weights, weights_dtype == MOE_GG_DTYPE_FP32 ? 4 : 2))
+    return MOE_GG_EALIGN;
+  return (int)combine_topk_launch(y, inv, weights, weights_dtype == MOE_GG_DTYPE_BF16, out, (int)T, k, d, (int)n_rows,
+                                  (hipStream_t)stream);
+}
+
 int moe_gg_fp8_groupwise_quant(const void* in, int dtype, void* out, float* scales, int64_t numel, void* stream) {
   if (numel < 0) return MOE_GG_EINVAL;
   if (dtype != MOE_GG_DTYPE_BF16 && dtype != MOE_GG_DTYPE_FP32) return MOE_GG_EINVAL;

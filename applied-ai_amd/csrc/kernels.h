@@ -63,3 +63,9 @@ hipError_t gather_rows_launch(const void* x, const int32_t* perm, int k, void* o
 // 1 x 128 fp8 quantiser (quant.hip); `groups` groups of 128 consecutive elements.
 hipError_t fp8_groupwise_quant_launch(const void* in, bool bf16_in, void* out, float* scales, int64_t groups,
                                       hipStream_t stream);
+
+// MoE layer glue (moe_layer.hip). bf16 data; n and d multiples of 8; 16-byte aligned pointers.
+hipError_t silu_and_mul_launch(const void* in, void* out, int64_t rows, int n, hipStream_t stream);
+hipError_t invert_perm_launch(const int32_t* perm, int32_t* inv, int n, const int32_t* n_valid, hipStream_t stream);
+hipError_t combine_topk_launch(const void* y, const int32_t* inv, const void* weights, bool weights_bf16, void* out,
+                               int T, int k, int d, int n_rows, hipStream_t stream);

@@ -1,0 +1,91 @@
+"""A whole MoE layer on top of the grouped GEMM, with the reference's fused_moe signature
+(kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:222-296).
+
+The reference pads every expert's token list to a block multiple (moe_align_block_size) and runs a gather-style
+GEMM twice; here the rows are gathered once into expert-sorted order and the two products are plain grouped GEMMs
+over m_sizes, so no padding rows are computed:
+
+    perm, m_sizes, offsets = group topk_ids by expert (stable)            moe_gg_route_group
+    xs  = hidden_states[perm // k]                                        moe_gg_gather_rows
+    h1  = grouped_gemm(xs, w1, m_sizes)            [R, 2n]                moe_gg_grouped_gemm_bf16
+    h2  = silu(h1[:, :n]) * h1[:, n:]              [R, n]                 moe_gg_silu_and_mul
+    y2  = grouped_gemm(h2, w2, m_sizes)            [R, d]                 moe_gg_grouped_gemm_bf16
+    out[t] = sum_j topk_weights[t, j] * y2[inv[t * k + j]]                moe_gg_invert_perm, moe_gg_combine_topk
+
+Everything runs in the HIP kernels behind include/moe_gg.h; torch only provides the buffers."""
+import torch
+
+from . import _lib
+from .ops import _require_cuda, _stream_ptr, grouped_gemm
+from .routing import gather_sorted, route_group
+
+
+def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """out = silu(x[:, :n]) * x[:, n:] for bf16 x [rows, 2n] (ops.silu_and_mul, v0_moe_fused.py:284)."""
+    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % 2:
+        raise ValueError("x must be bf16 [rows, 2n]")
+    dev = _require_cuda(x)
+    x = x.contiguous()
+    rows, n = x.shape[0], x.shape[1] // 2
+    out = torch.empty((rows, n), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_silu_and_mul(x.data_ptr(), out.data_ptr(), rows, n, _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_silu_and_mul")
+    return out
+
+
+def combine_topk(y: torch.Tensor, perm: torch.Tensor, offsets: torch.Tensor, topk_weights: torch.Tensor,
+                 out: torch.Tensor = None) -> torch.Tensor:
+    """out[t] = sum_j topk_weights[t, j] * y[row of (t, j)], y in expert-sorted row order (perm as from
+    route_group / route_topk, offsets its [E + 1] prefix table); fp32 accumulation, bf16 result."""
+    if y.dim() != 2 or y.dtype != torch.bfloat16:
+        raise ValueError("y must be bf16 [rows, d]")
+    if topk_weights.dim() != 2 or topk_weights.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("topk_weights must be fp32 or bf16 [T, k]")
+    dev = _require_cuda(y, perm, offsets, topk_weights)
+    y = y.contiguous()
+    topk_weights = topk_weights.contiguous()
+    T, k = topk_weights.shape
+    if perm.shape[0] != T * k:
+        raise ValueError("perm must have T * k entries")
+    inv = torch.full((T * k,), -1, dtype=torch.int32, device=dev)
+    if out is None:
+        out = torch.empty((T, y.shape[1]), dtype=torch.bfloat16, device=dev)
+    elif out.shape != (T, y.shape[1]) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError("out must be a contiguous bf16 [T, d] tensor")
+    wdt = 2 if topk_weights.dtype == torch.float32 else 0  # MOE_GG_DTYPE_FP32 / MOE_GG_DTYPE_BF16
+    with torch.cuda.device(dev):
+        L = _lib.lib()
+        rc = L.moe_gg_invert_perm(perm.data_ptr(), inv.data_ptr(), T * k, offsets[-1:].data_ptr(), _stream_ptr(dev))
+        _lib.check(rc, "moe_gg_invert_perm")
+        rc = L.moe_gg_combine_topk(y.data_ptr(), inv.data_ptr(), topk_weights.data_ptr(), wdt, out.data_ptr(), T, k,
+                                   y.shape[1], y.shape[0], _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_combine_topk")
+    return out
+
+
+def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk_weights: torch.Tensor,
+              topk_ids: torch.Tensor, inplace: bool = False) -> torch.Tensor:
+    """Mixture-of-experts layer with top-k gating; arguments as the reference's fused_moe
+    (v0_moe_fused.py:222-227): hidden_states [M, K], w1 [E, 2n, K], w2 [E, d, n], topk_weights / topk_ids [M, k].
+    bf16 only (the reference also takes fp16). With inplace=True the result is written into hidden_states
+    (d must equal K), as the reference does (:291-294)."""
+    assert hidden_states.shape[1] == w1.shape[2], "Incompatible dimensions"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert hidden_states.dtype == torch.bfloat16 and w1.dtype == torch.bfloat16 and w2.dtype == torch.bfloat16, \
+        "bf16 only"
+    _require_cuda(hidden_states, w1, w2, topk_weights, topk_ids)
+    E, two_n, K = w1.shape
+    assert two_n % 2 == 0 and w2.shape[0] == E and w2.shape[2] == two_n // 2, "Incompatible expert weights"
+    k = topk_ids.shape[1]
+    ids = topk_ids if topk_ids.dtype == torch.int32 else topk_ids.to(torch.int32)
+    tw = topk_weights if topk_weights.dtype in (torch.float32, torch.bfloat16) else topk_weights.float()
+
+    perm, m_sizes, offsets = route_group(ids, E)
+    xs = gather_sorted(hidden_states, perm, k)
+    h1 = grouped_gemm(xs, w1.view(E * two_n, K), m_sizes)
+    h2 = silu_and_mul(h1)
+    y2 = grouped_gemm(h2, w2.view(E * w2.shape[1], w2.shape[2]), m_sizes)
+    return combine_topk(y2, perm, offsets, tw, out=hidden_states if inplace else None)

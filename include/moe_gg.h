@@ -126,6 +126,26 @@ int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int
                        void* stream);
 
 /*
+ * Glue between the two grouped GEMMs of a whole MoE layer, as in the reference's fused_moe
+ * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:222-296; oracle torch_moe,
+ * kernels/triton/inference/col_major_moe_gemm/test_moe_gemm.py:16-30). All data bf16.
+ *
+ * moe_gg_silu_and_mul replaces ops.silu_and_mul (v0_moe_fused.py:284):
+ *   out[r, c] = silu(in[r, c]) * in[r, n + c];  in device [rows, 2n], out device [rows, n], n % 8 == 0.
+ * moe_gg_invert_perm: inv[perm[i]] = i for i < *n_valid (device int32, e.g. offsets + E of moe_gg_route_*;
+ *   NULL = all n). inv is not written elsewhere: fill it with -1 first if expert ids may have been dropped.
+ * moe_gg_combine_topk replaces the routed-weight multiply (MUL_ROUTED_WEIGHT, v0_moe_fused.py:122-126) and
+ *   the sum over the k rows of a token (:291-296):
+ *   out[t, :] = sum_j weights[t, j] * y[inv[t*k + j], :]   (fp32 accumulation, j ascending; inv entries
+ *   outside [0, n_rows) contribute nothing). y device [n_rows, d], out device [T, d], d % 8 == 0;
+ *   weights device [T, k], fp32 or bf16 (weights_dtype = MOE_GG_DTYPE_FP32 / MOE_GG_DTYPE_BF16).
+ */
+int moe_gg_silu_and_mul(const void* in, void* out, int64_t rows, int n, void* stream);
+int moe_gg_invert_perm(const int32_t* perm, int32_t* inv, int64_t n, const int32_t* n_valid, void* stream);
+int moe_gg_combine_topk(const void* y, const int32_t* inv, const void* weights, int weights_dtype, void* out,
+                        int64_t T, int k, int d, int64_t n_rows, void* stream);
+
+/*
  * 1 x 128 group-wise fp8 e4m3fn quantiser. Replaces float8_groupwise_quantize
  * (kernels/triton/inference/fp8/float8_groupwise_quant.py:53-91): per 128 consecutive elements
  * s = max(amax|x|, 1e-12) / 448, q = clamp(x / s, -448, 448) -> e4m3fn (RNE).

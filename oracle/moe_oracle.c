@@ -11,7 +11,8 @@
  *
  * Parity status:
  *   orc_offsets, orc_grouped_gemm, orc_route, orc_moe_align_block_size, orc_topk,
- *   orc_w4_dequant, orc_e4m3_*, orc_fp8_groupwise_quant, orc_grouped_gemm_fp8 (rowwise): pinned.
+ *   orc_w4_dequant, orc_e4m3_*, orc_fp8_groupwise_quant, orc_grouped_gemm_fp8 (rowwise),
+ *   orc_silu_and_mul, orc_fused_moe: pinned.
  *   orc_fp8_block_quant_weight (128x128 weight quantiser): PARITY UNPINNED - the reference calls an
  *   un-vendored FBGEMM routine for it (kernels/needs_perf_help/fp8_gemm_bench.py:16-21); this file
  *   defines it by analogy with the 1x128 quantiser and only its GEMM consumer is checked.
@@ -20,6 +21,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+
+float orc_round_bf16(float f);
 
 /* ---- offsets: exclusive prefix sum of m_sizes --------------------------------------------------
  * dev/triton_groupGEMM/groupgemm.py:159-165 (running M_start/M_end offsets) and the host form in
@@ -309,4 +312,61 @@ float orc_round_bf16(float f) {
   float r;
   memcpy(&r, &u, 4);
   return r;
+}
+
+/* ---- SiLU-and-mul ------------------------------------------------------------------------------
+ * ops.silu_and_mul as used by kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:284 and
+ * SiluAndMul in test_moe_gemm.py:29: out[r, c] = silu(in[r, c]) * in[r, n + c], silu(v) = v / (1 + e^-v).
+ * Pinned by: torch.nn.functional.silu on the CPU and the closed-form values silu(0) = 0,
+ * silu(v) - silu(-v) = v. */
+void orc_silu_and_mul(const float* in, int64_t rows, int n, float* out) {
+  for (int64_t r = 0; r < rows; ++r)
+    for (int c = 0; c < n; ++c) {
+      double g = in[r * 2 * n + c], u = in[r * 2 * n + n + c];
+      out[r * n + c] = (float)(g / (1.0 + exp(-g)) * u);
+    }
+}
+
+/* ---- whole MoE layer ----------------------------------------------------------------------------
+ * torch_moe of kernels/triton/inference/col_major_moe_gemm/test_moe_gemm.py:16-30:
+ *   out[t] = sum_j topk_weight[t, j] * ( silu_and_mul(a[t] @ w1[e]^T) @ w2[e]^T ),  e = topk_ids[t, j].
+ * a [T, K], w1 [E, 2n, K], w2 [E, d, n], out [T, d]; double accumulation. With round_intermediate != 0
+ * the two intermediate activations and the second product are rounded to bf16 where the layer stores
+ * them (the reference stores them in the activation dtype: intermediate_cache1..3, v0_moe_fused.py:266-274).
+ * Ids outside [0, E) contribute nothing.
+ * Pinned by: a torch float64 restatement with library matmuls on random inputs, and the special cases
+ * k = 1 with weight 1 (one expert's MLP) and w2 = 0 (zero output). */
+void orc_fused_moe(const float* a, const float* w1, const float* w2, const float* topk_weight,
+                   const int32_t* topk_ids, int64_t T, int K, int E, int n, int d, int k, int round_intermediate,
+                   float* out) {
+  float* h1 = (float*)malloc(sizeof(float) * 2 * (size_t)n);
+  float* h2 = (float*)malloc(sizeof(float) * (size_t)n);
+  for (int64_t t = 0; t < T; ++t) {
+    for (int c = 0; c < d; ++c) out[t * d + c] = 0.f;
+    double* accum = (double*)calloc((size_t)d, sizeof(double));
+    for (int j = 0; j < k; ++j) {
+      int e = topk_ids[t * k + j];
+      if (e < 0 || e >= E) continue;
+      const float* w1e = w1 + (size_t)e * 2 * n * K;
+      const float* w2e = w2 + (size_t)e * d * n;
+      for (int c = 0; c < 2 * n; ++c) {
+        double s = 0.0;
+        for (int q = 0; q < K; ++q) s += (double)a[t * K + q] * (double)w1e[(size_t)c * K + q];
+        h1[c] = round_intermediate ? orc_round_bf16((float)s) : (float)s;
+      }
+      orc_silu_and_mul(h1, 1, n, h2);
+      if (round_intermediate)
+        for (int c = 0; c < n; ++c) h2[c] = orc_round_bf16(h2[c]);
+      for (int c = 0; c < d; ++c) {
+        double s = 0.0;
+        for (int q = 0; q < n; ++q) s += (double)h2[q] * (double)w2e[(size_t)c * n + q];
+        float y = round_intermediate ? orc_round_bf16((float)s) : (float)s;
+        accum[c] += (double)topk_weight[t * k + j] * (double)y;
+      }
+    }
+    for (int c = 0; c < d; ++c) out[t * d + c] = (float)accum[c];
+    free(accum);
+  }
+  free(h1);
+  free(h2);
 }

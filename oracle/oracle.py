@@ -213,3 +213,47 @@ def grouped_gemm_torch_loop(x, w, m_sizes):
             y[start:start + m] = x[start:start + m] @ w[g * N:(g + 1) * N].T
         start += m
     return y
+
+
+def silu_and_mul(x):
+    """out = silu(x[:, :n]) * x[:, n:] (ops.silu_and_mul, v0_moe_fused.py:284)."""
+    x = _f32(x)
+    rows, n = x.shape[0], x.shape[1] // 2
+    out = np.empty((rows, n), dtype=np.float32)
+    _l().orc_silu_and_mul(_p(x), ctypes.c_int64(rows), ctypes.c_int(n), _p(out))
+    return out
+
+
+def fused_moe(a, w1, w2, topk_weight, topk_ids, round_intermediate=True):
+    """torch_moe of test_moe_gemm.py:16-30 in double precision: a [T, K], w1 [E, 2n, K], w2 [E, d, n],
+    topk_weight / topk_ids [T, k] -> out [T, d]. round_intermediate rounds the stored intermediates to bf16."""
+    a, w1, w2, tw, ids = _f32(a), _f32(w1), _f32(w2), _f32(topk_weight), _i32(topk_ids)
+    T, K = a.shape
+    E, two_n, _ = w1.shape
+    d = w2.shape[1]
+    k = ids.shape[1]
+    out = np.empty((T, d), dtype=np.float32)
+    _l().orc_fused_moe(_p(a), _p(w1), _p(w2), _p(tw), _p(ids), ctypes.c_int64(T), ctypes.c_int(K), ctypes.c_int(E),
+                       ctypes.c_int(two_n // 2), ctypes.c_int(d), ctypes.c_int(k), ctypes.c_int(1 if round_intermediate else 0),
+                       _p(out))
+    return out
+
+
+def fused_moe_torch(a, w1, w2, topk_weight, topk_ids):
+    """The same layer as a per-expert loop of fp32 torch matmuls on the CPU (the shape of the reference's
+    torch_moe, test_moe_gemm.py:16-30), for sizes the scalar C loop would take minutes on. Tensors in, tensor out."""
+    import torch
+
+    a, w1, w2 = a.float(), w1.float(), w2.float()
+    T, k = topk_ids.shape
+    n = w1.shape[1] // 2
+    rep = a.repeat_interleave(k, dim=0)
+    out = torch.zeros(T * k, w2.shape[1])
+    flat = topk_ids.reshape(-1)
+    for e in range(w1.shape[0]):
+        mask = flat == e
+        if mask.any():
+            h = rep[mask] @ w1[e].t()
+            h = torch.nn.functional.silu(h[:, :n]) * h[:, n:]
+            out[mask] = h @ w2[e].t()
+    return (out.view(T, k, -1) * topk_weight.float().view(T, k, 1)).sum(dim=1)

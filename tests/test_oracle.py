@@ -283,3 +283,51 @@ def test_round_bf16_vs_torch():
     x = np.concatenate([x, np.float32([1.00390625, 1.01171875, 0.0, -0.0])])  # ties
     t = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
     assert np.array_equal(O.round_bf16(x), t)
+
+
+def test_silu_and_mul_vs_torch_and_closed_forms():
+    rng = np.random.default_rng(16)
+    x = (rng.standard_normal((7, 24)) * 3).astype(np.float32)
+    t = torch.from_numpy(x).double()
+    e = torch.nn.functional.silu(t[:, :12]) * t[:, 12:]
+    np.testing.assert_allclose(O.silu_and_mul(x), e.numpy(), rtol=1e-6, atol=1e-7)
+    v = np.float32([[0.0, 2.5, -2.5, 1.0, 1.0, -1.0]])  # silu(0) = 0, silu(v) - silu(-v) = v
+    o = O.silu_and_mul(v)[0]
+    assert o[0] == 0.0 and abs(o[1] + o[2] - 2.5) < 1e-6
+
+
+def test_fused_moe_vs_torch_float64_and_special_cases():
+    """Pins orc_fused_moe: a float64 restatement with library matmuls (the structure of torch_moe,
+    test_moe_gemm.py:16-30), one expert with weight 1 = that expert's MLP, and w2 = 0."""
+    gen = torch.Generator().manual_seed(17)
+    T, K, E, n, d, k = 9, 32, 4, 16, 24, 2
+    a = torch.randn(T, K, generator=gen) / 3
+    w1 = torch.randn(E, 2 * n, K, generator=gen) / 3
+    w2 = torch.randn(E, d, n, generator=gen) / 3
+    score = torch.softmax(torch.randn(T, E, generator=gen), dim=-1)
+    tw, ids = torch.topk(score, k)
+    exp = torch.zeros(T, d, dtype=torch.float64)
+    for t in range(T):
+        for j in range(k):
+            e = int(ids[t, j])
+            h = w1[e].double() @ a[t].double()
+            h = torch.nn.functional.silu(h[:n]) * h[n:]
+            exp[t] += tw[t, j].double() * (w2[e].double() @ h)
+    got = O.fused_moe(a.numpy(), w1.numpy(), w2.numpy(), tw.numpy(), ids.numpy(), round_intermediate=False)
+    np.testing.assert_allclose(got, exp.numpy(), rtol=1e-5, atol=1e-6)
+    # the library-matmul form used for large sizes agrees too
+    np.testing.assert_allclose(O.fused_moe_torch(a, w1, w2, tw, ids).numpy(), exp.numpy(), rtol=1e-4, atol=1e-5)
+    # rounding the stored intermediates to bf16 moves the result by bf16-size errors only
+    got_r = O.fused_moe(a.numpy(), w1.numpy(), w2.numpy(), tw.numpy(), ids.numpy(), round_intermediate=True)
+    assert np.abs(got_r - exp.numpy()).max() < 2e-2
+    # k = 1, weight 1: one expert's MLP
+    one = O.fused_moe(a.numpy(), w1.numpy(), w2.numpy(), np.ones((T, 1), np.float32), np.full((T, 1), 2, np.int32), False)
+    h = a.double() @ w1[2].double().T
+    e1 = (torch.nn.functional.silu(h[:, :n]) * h[:, n:]) @ w2[2].double().T
+    np.testing.assert_allclose(one, e1.numpy(), rtol=1e-5, atol=1e-6)
+    assert np.all(O.fused_moe(a.numpy(), w1.numpy(), np.zeros_like(w2.numpy()), tw.numpy(), ids.numpy()) == 0)
+    # ids outside [0, E) contribute nothing
+    bad = ids.numpy().copy(); bad[:, 1] = E + 3
+    only0 = O.fused_moe(a.numpy(), w1.numpy(), w2.numpy(), tw.numpy(), bad, False)
+    first = O.fused_moe(a.numpy(), w1.numpy(), w2.numpy(), tw.numpy()[:, :1].copy(), ids.numpy()[:, :1].copy(), False)
+    np.testing.assert_allclose(only0, first, rtol=1e-6)
