@@ -166,6 +166,27 @@ def secondary_workloads(torch, A, dev):
                 "roofline": {"bound": "hbm", "kernel": "gg_fp8_stream (experts with <= 64 rows) + gg_fp8_pingpong_block", "achieved": round(byt / ms / 1e6, 1),
                              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
                              "traffic": None}})
+    del xq, wq, xs, ws, y
+
+    # ---- whole MoE layer (fused_moe): Mixtral 8x7B, T=4096 top-2, bf16 ----
+    T, K, n, E, topk = 4096, 4096, 14336, 8, 2
+    gen = torch.Generator(device=dev).manual_seed(1002)
+    h = (torch.randn(T, K, device=dev, generator=gen) / 10).to(torch.bfloat16)
+    w1 = torch.empty(E, 2 * n, K, device=dev, dtype=torch.bfloat16)
+    w2 = torch.empty(E, K, n, device=dev, dtype=torch.bfloat16)
+    for e in range(E):
+        w1[e] = (torch.randn(2 * n, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        w2[e] = (torch.randn(K, n, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    score = torch.softmax(torch.randn(T, E, device=dev, generator=gen), dim=-1)
+    tw, ids = torch.topk(score, topk)
+    ids = ids.to(torch.int32)
+    ms = event_time_ms(torch, lambda: A.fused_moe(h, w1, w2, tw, ids), 10, 3)
+    flop = 2.0 * T * topk * (2 * n * K + K * n)
+    out.append({"workload": "Mixtral 8x7B MoE layer (fused_moe: group, gather, w1 GEMM, SiLU-and-mul, w2 GEMM, top-2 combine), T=4096, bf16",
+                "ms_per_launch": round(ms, 3), "value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
+                "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong (two launches) + glue kernels", "achieved": round(flop / ms / 1e9, 1),
+                             "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                             "traffic": None}})
     return out
 
 
