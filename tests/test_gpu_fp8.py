@@ -132,3 +132,32 @@ def test_config5_shape_sampled_experts():
     g0 = slice(off[0], off[0] + 32)
     exact = x[g0].double() @ w[1024:1280].double().T
     assert rel_fro(to_np(y[g0, 1024:1280]), exact.numpy()) <= 6e-2
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])  # MOE_GG_FP8_TILED_128, _STREAM_PINGPONG, _STREAM_TILED
+@pytest.mark.parametrize("mode", [0, 1])
+def test_every_kernel_variant_against_oracle(variant, mode):
+    """Experts of 0, 1, 64 (streaming kernel's largest), 65 (tiled kernels' smallest), 300 and 17 rows through each
+    of the three kernel combinations of moe_gg_set_variant(MOE_GG_OP_GG_FP8, ...)."""
+    import applied_ai_amd as A
+
+    G, N, K = 6, 256, 512
+    m_sizes = [0, 1, 64, 65, 300, 17]
+    rng = np.random.default_rng(77)
+    M = sum(m_sizes)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((G * N, K)) * 0.05).astype(np.float32)
+    if mode == 1:
+        xq, xs = O.fp8_groupwise_quant(x); wq, ws = O.fp8_block_quant_weight(w)
+    else:
+        xs = np.abs(x).max(axis=1) / 448.0; ws = np.abs(w).max(axis=1) / 448.0
+        xq = torch.from_numpy(np.clip(x / xs[:, None], -448, 448)).to(F8).view(torch.uint8).numpy()
+        wq = torch.from_numpy(np.clip(w / ws[:, None], -448, 448)).to(F8).view(torch.uint8).numpy()
+    lib = A._lib.lib()
+    assert lib.moe_gg_set_variant(1, variant) == 0
+    try:
+        y = run(xq, wq, xs, ws, m_sizes, mode)
+    finally:
+        lib.moe_gg_set_variant(1, -1)
+    ref = O.grouped_gemm_fp8(xq, wq, xs, ws, m_sizes, mode)
+    assert rel_fro(to_np(y), ref) <= TOL
