@@ -43,6 +43,10 @@ struct W4Params {
   int M, N, K;
   int group_size;
   int zero_offset;
+  // Grouped (MoE) call: m_sizes != nullptr, G experts; a / c are [M, K] / [M, N] with rows sorted by expert,
+  // qweight [G, K/8, N], scales [G, K/group_size, N], qzeros [G, K/group_size, N/8]; M is the total row count.
+  const int32_t* m_sizes;
+  int G;
 };
 hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream);
 

@@ -53,6 +53,51 @@ struct Elem<true> {  // fp16
   static DEVINL uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
 };
 
+// What one workgroup works on: the whole problem (dense call), or expert blockIdx.y of a grouped call
+// (rows row0 .. row0 + M - 1 of a and c, and that expert's slice of the stacked weights).
+struct W4View {
+  const uint16_t* a;
+  const int32_t* qweight;
+  const uint16_t* scales;
+  const int32_t* qzeros;
+  uint16_t* c;
+  int M;
+};
+
+// Must be called by every thread of the workgroup (it contains a barrier in grouped mode).
+DEVINL W4View w4_view(const W4Params& p) {
+  W4View v{(const uint16_t*)p.a, p.qweight, (const uint16_t*)p.scales, p.qzeros, (uint16_t*)p.c, p.M};
+  if (p.m_sizes == nullptr) return v;
+  __shared__ int s_row0, s_rows;
+  const int g = blockIdx.y;
+  if (threadIdx.x < 64) {
+    long long s = 0;
+    for (int i = threadIdx.x; i < g; i += 64) {
+      const int m = p.m_sizes[i];
+      s += m < 0 ? 0 : (m > p.M ? p.M : m);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
+    if (threadIdx.x == 0) {
+      const long long r0 = s > p.M ? p.M : s;
+      int m = p.m_sizes[g];
+      m = m < 0 ? 0 : m;
+      s_row0 = (int)r0;
+      s_rows = (long long)m > p.M - r0 ? (int)(p.M - r0) : m;
+    }
+  }
+  __syncthreads();
+  const int row0 = s_row0;
+  const int ngroups = p.K / p.group_size;
+  v.M = s_rows;
+  v.a += (int64_t)row0 * p.K;
+  v.c += (int64_t)row0 * p.N;
+  v.qweight += (int64_t)g * (p.K / 8) * p.N;
+  v.scales += (int64_t)g * ngroups * p.N;
+  v.qzeros += (int64_t)g * ngroups * (p.N / 8);
+  return v;
+}
+
 constexpr int WAVES = 8;
 constexpr int DEPTH = 8;  // K steps of qweight loads in flight per wave
 
@@ -66,7 +111,8 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
-  const int N = p.N, K = p.K, M = p.M;
+  const W4View v = w4_view(p);
+  const int N = p.N, K = p.K, M = v.M;
   const int n0 = blockIdx.x * 64;
   const int spg = p.group_size / 32;               // K steps per quantisation group
   const int ngroups = K / p.group_size;
@@ -78,7 +124,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
 
   // qweight: lane reads words of columns n0 + 4*fr .. + 3 (clamped at the right edge), k-word row 4*step + fq
   const int wcol = min(n0 + 4 * fr, N - 4);
-  const int32_t* qw = p.qweight + wcol;
+  const int32_t* qw = v.qweight + wcol;
   // output / scale columns of this lane: n0 + 16*fq + 0..15
   const int ocol = n0 + 16 * fq;
   const int ocol_c = min(ocol, N - 16 >= 0 ? N - 16 : 0);
@@ -86,7 +132,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
   for (int mb = 0; mb < M; mb += 16 * MF) {
     const uint16_t* arow[MF];
 #pragma unroll
-    for (int i = 0; i < MF; ++i) arow[i] = (const uint16_t*)p.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
+    for (int i = 0; i < MF; ++i) arow[i] = v.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
 
     f32x4_t total[MF][4];  // [m fragment][j]: rows n-local 4*ii + j ... see epilogue
 #pragma unroll
@@ -119,11 +165,11 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
           u32x4_t xb[MF];
 #pragma unroll
           for (int i = 0; i < MF; ++i) {
-            const u32x4_t v = *(const u32x4_t*)(arow[i] + ks * 32);
-            xb[i][0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // k 0, 4
-            xb[i][1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // k 1, 5
-            xb[i][2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // k 2, 6
-            xb[i][3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // k 3, 7
+            const u32x4_t xv = *(const u32x4_t*)(arow[i] + ks * 32);
+            xb[i][0] = __builtin_amdgcn_perm(xv[2], xv[0], 0x05040100u);  // k 0, 4
+            xb[i][1] = __builtin_amdgcn_perm(xv[2], xv[0], 0x07060302u);  // k 1, 5
+            xb[i][2] = __builtin_amdgcn_perm(xv[3], xv[1], 0x05040100u);  // k 2, 6
+            xb[i][3] = __builtin_amdgcn_perm(xv[3], xv[1], 0x07060302u);  // k 3, 7
           }
           const u32x4_t w4 = wb[d];
           if (t + DEPTH < steps) loadw(d, t + DEPTH);
@@ -142,9 +188,9 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
           if (t % spg == spg - 1) {
             // fold scale and zero point of this group: lane's columns are ocol + 4*ii + j
             const int g = ks / spg;
-            const u32x4_t s0 = *(const u32x4_t*)((const uint16_t*)p.scales + (int64_t)g * N + ocol_c);
-            const u32x4_t s1 = *(const u32x4_t*)((const uint16_t*)p.scales + (int64_t)g * N + ocol_c + 8);
-            const u32x2_t zw = *(const u32x2_t*)(p.qzeros + (int64_t)g * (N / 8) + ocol_c / 8);
+            const u32x4_t s0 = *(const u32x4_t*)(v.scales + (int64_t)g * N + ocol_c);
+            const u32x4_t s1 = *(const u32x4_t*)(v.scales + (int64_t)g * N + ocol_c + 8);
+            const u32x2_t zw = *(const u32x2_t*)(v.qzeros + (int64_t)g * (N / 8) + ocol_c / 8);
 #pragma unroll
             for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
@@ -173,10 +219,10 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
     for (int o = tid; o < MF * 16 * 64; o += 64 * WAVES) {
       const int i = o / 1024, rem = o % 1024;
       const int m = mb + i * 16 + rem / 64, n = n0 + rem % 64;
-      float v = red[0][i][rem];
+      float sum = red[0][i][rem];
 #pragma unroll
-      for (int w2 = 1; w2 < WAVES; ++w2) v += red[w2][i][rem];
-      if (m < M && n < N) ((uint16_t*)p.c)[(int64_t)m * N + n] = E::from_f32(v);
+      for (int w2 = 1; w2 < WAVES; ++w2) sum += red[w2][i][rem];
+      if (m < M && n < N) v.c[(int64_t)m * N + n] = E::from_f32(sum);
     }
     __syncthreads();
   }
@@ -201,22 +247,23 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
-  const int N = p.N, K = p.K, M = p.M;
+  const W4View v = w4_view(p);
+  const int N = p.N, K = p.K, M = v.M;
   const int n0 = blockIdx.x * 64;
   const int ngroups = K / 128;
   const int my_groups = ngroups > wave ? (ngroups - wave + NWAVES - 1) / NWAVES : 0;
   const int steps = my_groups * SPG;
   auto kstep = [&](int t) { return ((t / SPG) * NWAVES + wave) * SPG + t % SPG; };
 
-  const int32_t* qw = p.qweight + n0 + 4 * fr;          // k-word row 4 * step + fq, columns n0 + 4 fr .. + 3
-  const uint16_t* sc = (const uint16_t*)p.scales + n0 + 4 * fr;
-  const int32_t* zp = p.qzeros + (n0 + 4 * fr) / 8;
+  const int32_t* qw = v.qweight + n0 + 4 * fr;          // k-word row 4 * step + fq, columns n0 + 4 fr .. + 3
+  const uint16_t* sc = v.scales + n0 + 4 * fr;
+  const int32_t* zp = v.qzeros + (n0 + 4 * fr) / 8;
   const int zshift = 16 * (fr & 1);                     // the lane's four zero nibbles inside the word
 
   for (int mb = 0; mb < M; mb += 16 * MF) {
     const uint16_t* arow[MF];
 #pragma unroll
-    for (int i = 0; i < MF; ++i) arow[i] = (const uint16_t*)p.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
+    for (int i = 0; i < MF; ++i) arow[i] = v.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
 
     f32x4_t total[MF][4];  // [row fragment i][column j]: rows mb + 16 i + 4 fq + r
 #pragma unroll
@@ -265,11 +312,11 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
             u32x4_t xb[MF];
 #pragma unroll
             for (int i = 0; i < MF; ++i) {
-              const u32x4_t v = xr[d][i];
-              xb[i][0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);  // k 0, 4
-              xb[i][1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);  // k 1, 5
-              xb[i][2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);  // k 2, 6
-              xb[i][3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);  // k 3, 7
+              const u32x4_t xv = xr[d][i];
+              xb[i][0] = __builtin_amdgcn_perm(xv[2], xv[0], 0x05040100u);  // k 0, 4
+              xb[i][1] = __builtin_amdgcn_perm(xv[2], xv[0], 0x07060302u);  // k 1, 5
+              xb[i][2] = __builtin_amdgcn_perm(xv[3], xv[1], 0x05040100u);  // k 2, 6
+              xb[i][3] = __builtin_amdgcn_perm(xv[3], xv[1], 0x07060302u);  // k 3, 7
             }
             const u32x4_t w4 = wb[d];
             if (more) load_step(d, (gi + GA) * SPG + e);
@@ -312,10 +359,10 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
     for (int o = tid; o < rows_here * 64; o += 64 * NWAVES) {
       const int ml = o / 64, col = o % 64;
       const int i = ml / 16, rem = (ml % 16) * 64 + col;
-      float v = red[0][i][rem];
+      float sum = red[0][i][rem];
 #pragma unroll
-      for (int w2 = 1; w2 < NWAVES; ++w2) v += red[w2][i][rem];
-      if (n0 + col < N) ((uint16_t*)p.c)[(int64_t)(mb + ml) * N + n0 + col] = E::from_f32(v);
+      for (int w2 = 1; w2 < NWAVES; ++w2) sum += red[w2][i][rem];
+      if (n0 + col < N) v.c[(int64_t)(mb + ml) * N + n0 + col] = E::from_f32(sum);
     }
     __syncthreads();
   }
@@ -323,13 +370,16 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
 
 template <bool FP16>
 hipError_t launch(const W4Params& p, hipStream_t stream) {
-  dim3 grid((p.N + 63) / 64), block(64 * WAVES);
+  // Grouped call: one grid row per expert; the kernel variant follows the average rows per expert (an
+  // expert with more rows than one pass covers is done in several passes over its weights).
+  dim3 grid((p.N + 63) / 64, p.m_sizes ? p.G : 1), block(64 * WAVES);
+  const int M = p.m_sizes ? (p.M + p.G - 1) / p.G : p.M;
   // M <= 16 and group size 128: one activation fragment, all loads issued one group ahead (deeper queues
   // and more waves measured slower). Larger M keeps up to four activation fragments per pass so that the
   // weights are unpacked once per four fragments.
-  if (p.M <= 16 && p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES>), grid, block, 0, stream, p);
-  else if (p.M <= 16) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 1>), grid, block, 0, stream, p);
-  else if (p.M <= 32) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 2>), grid, block, 0, stream, p);
+  if (M <= 16 && p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES>), grid, block, 0, stream, p);
+  else if (M <= 16) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 1>), grid, block, 0, stream, p);
+  else if (M <= 32) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 2>), grid, block, 0, stream, p);
   else hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 4>), grid, block, 0, stream, p);
   return hipGetLastError();
 }

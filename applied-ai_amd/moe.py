@@ -16,7 +16,7 @@ Everything runs in the HIP kernels behind include/moe_gg.h; torch only provides 
 import torch
 
 from . import _lib
-from .ops import _require_cuda, _stream_ptr, grouped_gemm
+from .ops import _require_cuda, _stream_ptr, grouped_gemm, matmul_split_k_grouped
 from .routing import gather_sorted, route_group
 
 
@@ -89,3 +89,35 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, t
     h2 = silu_and_mul(h1)
     y2 = grouped_gemm(h2, w2.view(E * w2.shape[1], w2.shape[2]), m_sizes)
     return combine_topk(y2, perm, offsets, tw, out=hidden_states if inplace else None)
+
+
+def dequant_gemm_moe(hidden_states: torch.Tensor, qw1: torch.Tensor, qw2: torch.Tensor, scales_qw1: torch.Tensor,
+                     scales_qw2: torch.Tensor, zeros_qw1: torch.Tensor, zeros_qw2: torch.Tensor, topk_ids: torch.Tensor,
+                     topk_weights: torch.Tensor = None, zero_offset: int = 1) -> torch.Tensor:
+    """MoE layer with int4 (GPTQ) expert weights; arguments as the reference's dequant_gemm_moe
+    (kernels/triton/inference/gptq/mixtral/w4a16_fused_dequant_gemm.py:255-318): hidden_states [M, K] bf16,
+    qw1 [E, K/8, 2n] / qw2 [E, n/8, d] int32, scales [E, K/g, 2n] / [E, n/g, d] bf16, zeros [E, K/g, 2n/8] /
+    [E, n/g, d/8] int32, topk_ids [M, k]. Like the reference, the k rows of a token are summed without routed
+    weights (:316-317) unless topk_weights is given. Same pipeline as fused_moe with the two products done by
+    the grouped W4A16 kernel (moe_gg_w4a16_grouped)."""
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert qw1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert qw2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert hidden_states.dtype == torch.bfloat16, "bf16 only"
+    _require_cuda(hidden_states, qw1, qw2, scales_qw1, scales_qw2, zeros_qw1, zeros_qw2, topk_ids)
+    E = qw1.shape[0]
+    assert hidden_states.shape[1] == qw1.shape[1] * 8, "Incompatible dimensions"
+    assert qw2.shape[0] == E and qw2.shape[1] * 8 * 2 == qw1.shape[2], "Incompatible expert weights"
+    T, k = topk_ids.shape
+    ids = topk_ids if topk_ids.dtype == torch.int32 else topk_ids.to(torch.int32)
+    if topk_weights is None:
+        tw = torch.ones((T, k), dtype=torch.float32, device=hidden_states.device)
+    else:
+        tw = topk_weights if topk_weights.dtype in (torch.float32, torch.bfloat16) else topk_weights.float()
+
+    perm, m_sizes, offsets = route_group(ids, E)
+    xs = gather_sorted(hidden_states, perm, k)
+    h1 = matmul_split_k_grouped(xs, qw1, scales_qw1, zeros_qw1, m_sizes, zero_offset=zero_offset)
+    h2 = silu_and_mul(h1)
+    y2 = matmul_split_k_grouped(h2, qw2, scales_qw2, zeros_qw2, m_sizes, zero_offset=zero_offset)
+    return combine_topk(y2, perm, offsets, tw)

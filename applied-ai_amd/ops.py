@@ -113,6 +113,39 @@ def matmul_split_k(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros
     return c
 
 
+def matmul_split_k_grouped(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
+                           m_sizes: torch.Tensor, zero_offset: int = 1, groupsize: Optional[int] = None) -> torch.Tensor:
+    """W4A16 grouped GEMM over expert-sorted rows: c[rows of expert g] = a[rows of g] @ dequant(b[g], scales[g], zeros[g]).
+
+    The GEMM of the reference's W4A16 fused MoE kernel
+    (kernels/triton/inference/gptq/mixtral/w4a16_fused_dequant_gemm.py:49-149) without its padded token lists:
+    a [M, K] fp16 or bf16, rows sorted by expert; b [E, K/8, N] int32; scales [E, K/g, N]; zeros [E, K/g, N/8] int32;
+    m_sizes [E] int32 on the device. Packing and zero_offset as in matmul_split_k."""
+    if a.dim() != 2 or b.dim() != 3 or scales.dim() != 3 or zeros.dim() != 3 or m_sizes.dim() != 1:
+        raise ValueError("a must be 2-D, b / scales / zeros 3-D, m_sizes 1-D")
+    m, k = a.shape
+    e, kw, n = b.shape
+    if kw * 8 != k:
+        raise ValueError(f"b has {kw} packed rows per expert, expected K/8 = {k // 8}")
+    if b.dtype != torch.int32 or zeros.dtype != torch.int32 or m_sizes.dtype != torch.int32:
+        raise ValueError("b, zeros and m_sizes must be int32")
+    if a.dtype not in (torch.bfloat16, torch.float16) or scales.dtype != a.dtype:
+        raise ValueError("a and scales must both be bf16 or both fp16")
+    g = groupsize if groupsize is not None else k // scales.shape[1]
+    if scales.shape != (e, k // g, n) or zeros.shape != (e, k // g, n // 8) or m_sizes.shape[0] != e:
+        raise ValueError("scales must be [E, K/g, N], zeros [E, K/g, N/8], m_sizes [E]")
+    dev = _require_cuda(a, b, scales, zeros, m_sizes)
+    a, b, scales, zeros, m_sizes = a.contiguous(), b.contiguous(), scales.contiguous(), zeros.contiguous(), m_sizes.contiguous()
+    c = torch.empty((m, n), device=dev, dtype=a.dtype)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_w4a16_grouped(
+            a.data_ptr(), b.data_ptr(), scales.data_ptr(), zeros.data_ptr(), c.data_ptr(), m_sizes.data_ptr(), e, m, n,
+            k, g, zero_offset, 1 if a.dtype == torch.float16 else 0, _stream_ptr(dev),
+        )
+    _lib.check(rc, "moe_gg_w4a16_grouped")
+    return c
+
+
 SCALE_ROWWISE = 0
 SCALE_BLOCK128 = 1
 

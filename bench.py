@@ -132,6 +132,32 @@ def secondary_workloads(torch, A, dev):
                                  "traffic": None}})
     del qws
 
+    # ---- W4A16 grouped (int4 experts), Mixtral decode: config 3's 64 rows over 8 experts, config 4's weight format ----
+    E = 8
+    qwe = [torch.randint(-2**31, 2**31 - 1, (E, K // 8, N), dtype=torch.int32, device=dev) for _ in range(2)]
+    sce = (torch.rand(E, K // 128, N, device=dev) * 0.015 + 0.005).to(torch.bfloat16)
+    qze = torch.randint(-2**31, 2**31 - 1, (E, K // 128, N // 8), dtype=torch.int32, device=dev)
+    a = torch.randn(64, K, device=dev).to(torch.bfloat16)
+    c = torch.empty(64, N, device=dev, dtype=torch.bfloat16)
+    ms3 = c3["m_sizes"].to(dev)
+    state = {"i": 0}
+
+    def call():
+        q = qwe[state["i"] & 1]
+        state["i"] += 1
+        lib.moe_gg_w4a16_grouped(a.data_ptr(), q.data_ptr(), sce.data_ptr(), qze.data_ptr(), c.data_ptr(), ms3.data_ptr(),
+                                 E, 64, N, K, 128, 0, 0, stream)
+
+    ms = event_time_ms(torch, call, 40, 6)
+    act = sum(1 for m in c3["m_sizes"].tolist() if m > 0)
+    byt = act * (K * N // 2 + K // 128 * N * 2 + K // 128 * N // 2) + 64 * K * 2 + 64 * N * 2
+    out.append({"workload": f"W4A16 grouped GEMM (int4 experts), Mixtral decode: 64 rows over 8 experts, K={K} N={N} group 128",
+                "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
+                "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128 (grid.y = experts)", "achieved": round(byt / ms / 1e6, 1),
+                             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
+                             "traffic": None}})
+    del qwe
+
     # ---- config 5: DeepSeek-V3-style fp8 block-scaled, 256 experts top-8, Zipf(1.1) routing ----
     _, _, _, m5 = configs.cfg5_routing()
     G, N, K = 256, 4096, 7168

@@ -99,6 +99,22 @@ int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scale
                         void* c, int M, int N, int K, int group_size, int zero_offset, int dtype,
                         void* stream);
 
+/*
+ * W4A16 grouped (MoE) GEMM: every expert has its own int4 weights; rows of a and c are sorted by expert.
+ * Replaces the GEMM of the reference's W4A16 fused MoE kernel (w4a16_fused_moe_kernel / invoke_dequant_gemm_moe,
+ * kernels/triton/inference/gptq/mixtral/w4a16_fused_dequant_gemm.py:49-149, 153-208) on expert-sorted rows instead
+ * of its padded token lists:  c[off_g + i, :] = a[off_g + i, :] @ dequant(qweight[g], scales[g], qzeros[g]).
+ *   a device [M, K], c device [M, N] (bf16 or fp16, dtype); m_sizes device int32 [G] (consumed on the device);
+ *   qweight device int32 [G, K/8, N]; scales device [G, K/group_size, N]; qzeros device int32 [G, K/group_size, N/8];
+ *   nibble order, dequantisation formula, zero_offset and requirements as for moe_gg_w4a16_splitk
+ *   (the reference kernel uses zero_offset = 1: w4a16_fused_dequant_gemm.py:133-137).
+ * Rows >= sum(m_sizes) of c are not written. Built for a few rows per expert (decode): an expert with more
+ * than 64 rows is computed in several passes over its weights.
+ */
+int moe_gg_w4a16_grouped(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros, void* c,
+                         const int32_t* m_sizes, int G, int64_t M, int N, int K, int group_size, int zero_offset,
+                         int dtype, void* stream);
+
 #define MOE_GG_MAX_ROUTE_EXPERTS 768
 
 /*

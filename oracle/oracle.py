@@ -257,3 +257,33 @@ def fused_moe_torch(a, w1, w2, topk_weight, topk_ids):
             h = torch.nn.functional.silu(h[:, :n]) * h[:, n:]
             out[mask] = h @ w2[e].t()
     return (out.view(T, k, -1) * topk_weight.float().view(T, k, 1)).sum(dim=1)
+
+
+def w4a16_grouped(a, qweight, scales, qzeros, m_sizes, group_size=128, zero_offset=1, fill=np.nan):
+    """Per-expert W4A16 product over expert-sorted rows (the GEMM of w4a16_fused_moe_kernel,
+    gptq/mixtral/w4a16_fused_dequant_gemm.py:49-149): qweight [E, K/8, N], scales [E, K/g, N], qzeros [E, K/g, N/8].
+    Composition of w4a16_gemm (pinned on its own) over the offsets of m_sizes; unwritten rows hold `fill`."""
+    a = _f32(a)
+    E = len(m_sizes)
+    N = qweight.shape[2]
+    out = np.full((a.shape[0], N), fill, dtype=np.float32)
+    start = 0
+    for e in range(E):
+        m = int(m_sizes[e])
+        if m:
+            out[start:start + m] = w4a16_gemm(a[start:start + m], qweight[e], scales[e], qzeros[e], group_size, zero_offset)
+        start += m
+    return out
+
+
+def dequant_gemm_moe(a, qw1, qw2, s1, s2, z1, z2, topk_ids, topk_weight=None, group_size=128, zero_offset=1,
+                     round_intermediate=True):
+    """The W4A16 MoE layer (dequant_gemm_moe, gptq/mixtral/w4a16_fused_dequant_gemm.py:255-318): both expert weight
+    sets dequantised with w4_dequant, then fused_moe. The reference sums the top-k rows without routed weights
+    (:316-317), which is topk_weight = None here."""
+    E = qw1.shape[0]
+    w1 = np.stack([w4_dequant(qw1[e], s1[e], z1[e], group_size, zero_offset).T for e in range(E)])   # [E, 2n, K]
+    w2 = np.stack([w4_dequant(qw2[e], s2[e], z2[e], group_size, zero_offset).T for e in range(E)])   # [E, d, n]
+    ids = _i32(topk_ids)
+    tw = np.ones(ids.shape, dtype=np.float32) if topk_weight is None else _f32(topk_weight)
+    return fused_moe(a, w1, w2, tw, ids, round_intermediate)

@@ -331,3 +331,39 @@ def test_fused_moe_vs_torch_float64_and_special_cases():
     only0 = O.fused_moe(a.numpy(), w1.numpy(), w2.numpy(), tw.numpy(), bad, False)
     first = O.fused_moe(a.numpy(), w1.numpy(), w2.numpy(), tw.numpy()[:, :1].copy(), ids.numpy()[:, :1].copy(), False)
     np.testing.assert_allclose(only0, first, rtol=1e-6)
+
+
+def test_w4a16_grouped_and_int4_layer_compose_pinned_parts():
+    """w4a16_grouped is w4a16_gemm per expert slice; dequant_gemm_moe is w4_dequant + fused_moe: check both against a
+    direct numpy evaluation (dequantise, matmul in float64), including an empty expert and unweighted top-k sums."""
+    rng = np.random.default_rng(19)
+    E, K, N, gs = 3, 128, 16, 64
+    q = rng.integers(0, 16, size=(E, K, N)); zz = rng.integers(0, 16, size=(E, K // gs, N))
+    qw = np.stack([O.pack_int4_along_k(q[e]) for e in range(E)]); qz = np.stack([O.pack_int4_along_n(zz[e]) for e in range(E)])
+    sc = rng.uniform(0.01, 0.02, size=(E, K // gs, N)).astype(np.float32)
+    m_sizes = [2, 0, 3]
+    a = rng.standard_normal((5, K)).astype(np.float32)
+    got = O.w4a16_grouped(a, qw, sc, qz, m_sizes, gs, 1)
+    w = (q - (np.repeat(zz, gs, axis=1) + 1)) * np.repeat(sc, gs, axis=1).astype(np.float64)      # [E, K, N]
+    exp = np.concatenate([a[:2].astype(np.float64) @ w[0], a[2:].astype(np.float64) @ w[2]])
+    np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-6)
+    # layer: K -> 2n = N (n = 8), second weights n -> d
+    n, d = N // 2, 16
+    q2 = rng.integers(0, 16, size=(E, 64, d)); zz2 = rng.integers(0, 16, size=(E, 1, d))
+    # the second product's K dimension is n = 8 < a quantisation group, so use a layer whose n is one group
+    E2, K2, n2, d2, g2 = 2, 64, 64, 16, 64
+    qa = rng.integers(0, 16, size=(E2, K2, 2 * n2)); za = rng.integers(0, 16, size=(E2, 1, 2 * n2)); sa = rng.uniform(0.01, 0.02, size=(E2, 1, 2 * n2)).astype(np.float32)
+    qb = rng.integers(0, 16, size=(E2, n2, d2)); zb = rng.integers(0, 16, size=(E2, 1, d2)); sb = rng.uniform(0.01, 0.02, size=(E2, 1, d2)).astype(np.float32)
+    pk = lambda t: np.stack([O.pack_int4_along_k(t[e]) for e in range(t.shape[0])])
+    pn = lambda t: np.stack([O.pack_int4_along_n(t[e]) for e in range(t.shape[0])])
+    x = (rng.standard_normal((4, K2)) / 4).astype(np.float32)
+    ids = np.array([[0, 1], [1, 0], [0, 1], [1, 0]], dtype=np.int32)
+    got = O.dequant_gemm_moe(x, pk(qa), pk(qb), sa, sb, pn(za), pn(zb), ids, None, g2, 1, round_intermediate=False)
+    wa = (qa - (za + 1)) * sa.astype(np.float64); wb = (qb - (zb + 1)) * sb.astype(np.float64)
+    exp = np.zeros((4, d2))
+    for t in range(4):
+        for e in ids[t]:
+            h = x[t].astype(np.float64) @ wa[e]
+            h = h[:n2] / (1 + np.exp(-h[:n2])) * h[n2:]
+            exp[t] += h @ wb[e]
+    np.testing.assert_allclose(got, exp, rtol=1e-4, atol=1e-5)
