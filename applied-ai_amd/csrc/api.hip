@@ -38,6 +38,14 @@ int current_device_info(const DeviceInfo** out) {
 
 bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
+// The dedicated small-M kernels (weights streamed straight into MFMA operands, split-K inside the workgroup)
+// beat the ping-pong kernel only for a few rows per expert (measured: up to about 12) or when the launch has
+// too few 256 x 256 tiles to give every CU several (few experts, narrow N); never above 40 rows per expert.
+bool use_streaming_kernel(int64_t M, int G, int64_t ntn256, int num_wg) {
+  if (M > (int64_t)G * 40) return false;
+  return M <= (int64_t)G * 12 || (int64_t)G * ntn256 < 4 * (int64_t)num_wg;
+}
+
 }  // namespace
 
 extern "C" {
@@ -97,7 +105,8 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
   const bool decode_ok = K % 128 == 0;
-  if (variant < 0 && decode_ok && M <= (int64_t)G * 40) variant = MOE_GG_GG_DECODE;
+  const int64_t ntn256 = (N + 255) / 256;
+  if (variant < 0 && decode_ok && use_streaming_kernel(M, G, ntn256, num_wg)) variant = MOE_GG_GG_DECODE;
   if (variant == MOE_GG_GG_DECODE) {
     if (!decode_ok) return MOE_GG_EUNSUPPORTED;
     const int64_t avg = (M + G - 1) / G;
@@ -107,13 +116,14 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
     return (int)gg_bf16_decode_launch(p, nf, mf, s);
   }
   if (variant < 0) {
-    // m_sizes lives on the device and is never copied back, so the tile shape is picked from the
-    // average rows per expert and a rough tile count (each expert adds about half a partial tile).
-    const int64_t avg = M / G;
-    const int64_t t256 = (M / 256 + (G + 1) / 2) * ((N + 255) / 256);
-    const int64_t t128 = (M / 128 + (G + 1) / 2) * ((N + 127) / 128);
-    if (avg >= 160 && t256 * 4 >= (int64_t)num_wg * 3) variant = MOE_GG_GG_PINGPONG_256;
-    else if (avg >= 80 && t128 * 2 >= num_wg) variant = MOE_GG_GG_TILED_128;
+    // m_sizes lives on the device and is never copied back, so the tile shape is picked from a rough
+    // count of 256 x 256 tiles (each expert adds about half a partial row tile). Measured over expert
+    // counts 2 .. 256 and 128 .. 8192 rows: the ping-pong kernel wins whenever there are enough tiles
+    // to occupy the CUs, also for experts of 16 .. 128 rows (short tiles skip most of their work and
+    // the kernel then streams weights at 5 TB/s); smaller tiles only pay for small problems.
+    const int64_t t256 = (M / 256 + (G + 1) / 2) * ntn256;
+    if (t256 * 4 >= (int64_t)num_wg * 3) variant = MOE_GG_GG_PINGPONG_256;
+    else if (t256 * 4 >= num_wg) variant = MOE_GG_GG_TILED_128;
     else variant = MOE_GG_GG_TILED_64;
   }
   switch (variant) {
@@ -154,13 +164,16 @@ int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* 
   p.xcds = di->xcds;
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
-  // Experts with a few rows are weight-streaming problems: they go to the split-K streaming kernel, a
-  // tiled kernel takes the rest. m_sizes stays on the device, so both are always launched; a kernel whose
-  // share is empty exits after reading m_sizes.
+  // A few rows per expert (see use_streaming_kernel): the experts with up to 64 rows go to the streaming
+  // split-K kernel and the ping-pong kernel takes the rest; m_sizes stays on the device, so both are launched
+  // and a workgroup whose expert belongs to the other kernel exits after reading m_sizes. Otherwise the
+  // ping-pong kernel does everything.
   int variant = g_variant[MOE_GG_OP_GG_FP8].load();
-  if (variant < 0) variant = MOE_GG_FP8_STREAM_PINGPONG;
+  if (variant < 0)
+    variant = use_streaming_kernel(M, G, (N + 255) / 256, num_wg) ? MOE_GG_FP8_STREAM_PINGPONG : MOE_GG_FP8_PINGPONG;
   hipStream_t s = (hipStream_t)stream;
   if (variant == MOE_GG_FP8_TILED_128) return (int)gg_fp8_launch(p, scale_mode, num_wg, s);
+  if (variant == MOE_GG_FP8_PINGPONG) return (int)gg_fp8_pingpong_launch(p, scale_mode, num_wg, s);
   if (variant != MOE_GG_FP8_STREAM_PINGPONG && variant != MOE_GG_FP8_STREAM_TILED) return MOE_GG_EINVAL;
   hipError_t e = gg_fp8_stream_launch(p, scale_mode, s);
   if (e != hipSuccess) return (int)e;

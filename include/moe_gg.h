@@ -191,6 +191,7 @@ int moe_gg_fp8_groupwise_quant(const void* in, int dtype, void* out, float* scal
 #define MOE_GG_FP8_TILED_128 0       /* 128x128 tiles for every expert */
 #define MOE_GG_FP8_STREAM_PINGPONG 1 /* experts with <= 64 rows: streaming split-K kernel; others: 256x256 ping-pong */
 #define MOE_GG_FP8_STREAM_TILED 2    /* experts with <= 64 rows: streaming split-K kernel; others: 128x128 tiles */
+#define MOE_GG_FP8_PINGPONG 3        /* 256x256 ping-pong kernel for every expert */
 int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,

@@ -134,11 +134,11 @@ def test_config5_shape_sampled_experts():
     assert rel_fro(to_np(y[g0, 1024:1280]), exact.numpy()) <= 6e-2
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])  # MOE_GG_FP8_TILED_128, _STREAM_PINGPONG, _STREAM_TILED
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])  # MOE_GG_FP8_TILED_128, _STREAM_PINGPONG, _STREAM_TILED, _PINGPONG
 @pytest.mark.parametrize("mode", [0, 1])
 def test_every_kernel_variant_against_oracle(variant, mode):
     """Experts of 0, 1, 64 (streaming kernel's largest), 65 (tiled kernels' smallest), 300 and 17 rows through each
-    of the three kernel combinations of moe_gg_set_variant(MOE_GG_OP_GG_FP8, ...)."""
+    of the four kernel combinations of moe_gg_set_variant(MOE_GG_OP_GG_FP8, ...)."""
     import applied_ai_amd as A
 
     G, N, K = 6, 256, 512
