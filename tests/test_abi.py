@@ -49,6 +49,37 @@ def test_argument_errors_are_rejected_before_any_launch(lib):
     assert f(None, None, None, None, 2, 0, 8, 8, 8, 0, None) == 0    # M == 0: nothing to do
 
 
+def test_argument_errors_of_the_other_entry_points(lib):
+    """Every entry point validates sizes, enums and null pointers before it touches a device."""
+    f8 = lib.moe_gg_grouped_gemm_fp8
+    assert f8(None, None, None, None, None, 5, None, 2, 8, 128, 128, 128, 0, None) == -1   # bad scale mode
+    assert f8(None, None, None, None, None, 0, None, 2, 8, 128, 128, 64, 0, None) == -2    # ldy < N
+    assert f8(None, None, None, None, None, 0, None, 2, 8, 128, 128, 128, 0, None) == -1   # null pointers
+    assert f8(None, None, None, None, None, 0, None, 0, 8, 128, 128, 128, 0, None) == 0    # G == 0
+    w4 = lib.moe_gg_w4a16_splitk
+    assert w4(None, None, None, None, None, 1, 64, 128, 0, 1, 0, None) == -1      # group_size <= 0
+    assert w4(None, None, None, None, None, 1, 64, 128, 128, 2, 0, None) == -1    # zero_offset not 0 / 1
+    assert w4(None, None, None, None, None, 1, 64, 128, 128, 1, 2, None) == -1    # fp32 is not a W4A16 dtype
+    assert w4(None, None, None, None, None, 1, 64, 128, 128, 1, 0, None) == -1    # null pointers
+    assert w4(None, None, None, None, None, 0, 64, 128, 128, 1, 0, None) == 0     # M == 0
+    w4g = lib.moe_gg_w4a16_grouped
+    assert w4g(None, None, None, None, None, None, -1, 4, 64, 128, 128, 1, 0, None) == -1
+    assert w4g(None, None, None, None, None, None, 2, 4, 64, 128, 128, 1, 0, None) == -1    # null pointers
+    assert w4g(None, None, None, None, None, None, 2, 0, 64, 128, 128, 1, 0, None) == 0     # no rows
+    assert lib.moe_gg_route_topk(None, 4, 8, 9, None, None, None, None, None) == -1         # k > E
+    assert lib.moe_gg_route_topk(None, 4, 1000, 2, None, None, None, None, None) == -4      # E too large
+    assert lib.moe_gg_route_group(None, 4, 0, None, None, None, None) == -1
+    assert lib.moe_gg_gather_rows(None, None, 0, None, 4, 16, None) == -1                    # k <= 0
+    assert lib.moe_gg_silu_and_mul(None, None, 4, 12, None) == -1                            # null pointers
+    assert lib.moe_gg_silu_and_mul(None, None, 0, 12, None) == 0
+    assert lib.moe_gg_invert_perm(None, None, -1, None, None) == -1
+    assert lib.moe_gg_combine_topk(None, None, None, 1, None, 4, 2, 8, 8, None) == -1        # fp16 weights unsupported
+    assert lib.moe_gg_combine_topk(None, None, None, 2, None, 4, 0, 8, 8, None) == -1        # k <= 0
+    assert lib.moe_gg_fp8_groupwise_quant(None, 1, None, None, 128, None) == -1              # fp16 input unsupported
+    assert lib.moe_gg_set_variant(9, 0) == -1
+    assert lib.moe_gg_set_variant(0, -1) == 0
+
+
 def enumerate_tiles(lib, m_sizes, M, N, bm, bn, nwg, xcds):
     ms = np.ascontiguousarray(m_sizes, dtype=np.int32)
     cap = 1 << 16
