@@ -250,6 +250,84 @@ int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int
   return (int)gather_rows_launch(x, perm, k, out, (int)n, row_bytes, (hipStream_t)stream);
 }
 
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+// Leading dimension of the transposed operands: every expert padded to whole 64-row blocks.
+static int64_t backward_ldm(int G, int64_t M) { return (M / 64 + G) * 64; }
+
+size_t moe_gg_grouped_gemm_backward_workspace(int G, int64_t M, int N, int K, int grad_layout) {
+  if (G <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
+  const size_t ldm = (size_t)backward_ldm(G, M);
+  size_t b = align256((size_t)G * N * K * 2) + align256((size_t)N * ldm * 2) + align256((size_t)K * ldm * 2);
+  if (grad_layout == MOE_GG_OUT_BLOCK) b += align256((size_t)M * N * 2);
+  return b;
+}
+
+int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int grad_layout, const void* x, const void* w,
+                                      const int32_t* m_sizes, int G, int64_t M, int N, int K, void* grad_x, void* grad_w,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  if (G < 0 || M < 0 || N < 0 || K < 0) return MOE_GG_EINVAL;
+  if (grad_layout != MOE_GG_OUT_MN && grad_layout != MOE_GG_OUT_BLOCK) return MOE_GG_EINVAL;
+  const int64_t min_ld = grad_layout == MOE_GG_OUT_BLOCK ? (int64_t)N * G : (int64_t)N;
+  if (ld_go < min_ld) return MOE_GG_ESHAPE;
+  if (G == 0 || N == 0 || K == 0) return MOE_GG_OK;
+  if (!grad_w || !m_sizes) return MOE_GG_EINVAL;
+  if (M > 0 && (!grad_out || !x || !w || !grad_x)) return MOE_GG_EINVAL;
+  if (G > MOE_GG_MAX_GROUPS_ABI || M > INT32_MAX - 64 * (int64_t)G || (int64_t)G * N > INT32_MAX || ld_go > INT32_MAX)
+    return MOE_GG_EUNSUPPORTED;
+  if (N % 4 != 0 || K % 4 != 0 || ld_go % 4 != 0) return MOE_GG_EUNSUPPORTED;
+  // 32-bit byte offsets inside a 256-row operand tile of pitch 2 * ldm
+  if (backward_ldm(G, M > 0 ? M : 1) > (1 << 22)) return MOE_GG_EUNSUPPORTED;
+  if (grad_layout == MOE_GG_OUT_MN && ld_go != N) return MOE_GG_EUNSUPPORTED;
+  if (!workspace || workspace_bytes < moe_gg_grouped_gemm_backward_workspace(G, M > 0 ? M : 1, N, K, grad_layout))
+    return MOE_GG_EINVAL;
+  if (!aligned(grad_out, 16) || !aligned(x, 16) || !aligned(w, 16) || !aligned(grad_x, 16) || !aligned(grad_w, 16) ||
+      !aligned(workspace, 256) || !aligned(m_sizes, 4))
+    return MOE_GG_EALIGN;
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != MOE_GG_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t Mw = M > 0 ? M : 1;
+  const int64_t ldm = backward_ldm(G, Mw);
+  char* ws = (char*)workspace;
+  void* wt = ws;                      ws += align256((size_t)G * N * K * 2);
+  void* dyt = ws;                     ws += align256((size_t)N * ldm * 2);
+  void* xt = ws;                      ws += align256((size_t)K * ldm * 2);
+  void* dyc = ws;
+
+  hipError_t e;
+  if (M > 0) {
+    // grad_x: the forward kernels on (dY [M, N], w^T [G*K, N]).
+    e = transpose_batched_launch(w, wt, G, N, K, s);
+    if (e != hipSuccess) return (int)e;
+    const void* dy = grad_out;
+    if (grad_layout == MOE_GG_OUT_BLOCK) {
+      e = compact_block_launch(grad_out, dyc, m_sizes, G, (int)M, N, ld_go, N, s);
+      if (e != hipSuccess) return (int)e;
+      dy = dyc;
+    }
+    rc = moe_gg_grouped_gemm_bf16(dy, wt, grad_x, m_sizes, G, M, K, N, K, MOE_GG_OUT_MN, stream);
+    if (rc != MOE_GG_OK) return rc;
+    // grad_w: dY^T and x^T with every expert padded to whole 64-row blocks.
+    e = transpose_padded_launch(grad_out, dyt, m_sizes, G, (int)M, N, ld_go, grad_layout == MOE_GG_OUT_BLOCK ? N : 0, ldm, s);
+    if (e != hipSuccess) return (int)e;
+    e = transpose_padded_launch(x, xt, m_sizes, G, (int)M, K, K, 0, ldm, s);
+    if (e != hipSuccess) return (int)e;
+  }
+  GgParams p{};
+  p.x = dyt; p.w = xt; p.y = grad_w; p.m_sizes = m_sizes;
+  p.G = G; p.M = (int)ldm; p.N = N; p.K = K;
+  p.ldy = K;
+  p.col_block = 0;
+  p.vec_store = aligned(grad_w, 8) && K % 4 == 0;
+  p.xcds = di->xcds;
+  p.skip_rows = (int)M;
+  int num_wg = di->cus - di->cus % p.xcds;
+  if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
+  const int64_t t256 = (int64_t)G * ((N + 255) / 256) * ((K + 255) / 256);
+  return (int)gg_bf16_wgrad_launch(p, t256 >= num_wg ? 256 : 128, num_wg, s);
+}
+
 int moe_gg_silu_and_mul(const void* in, void* out, int64_t rows, int n, void* stream) {
   if (rows < 0 || n < 0) return MOE_GG_EINVAL;
   if (rows == 0 || n == 0) return MOE_GG_OK;

@@ -53,7 +53,14 @@ DEVINL void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <class C>
+// WGRAD = false: the forward product above. WGRAD = true: the weight gradient of the same layer,
+//   dW[g][n][k] = sum over the rows m of expert g of dY[m][n] * X[m][k]
+// (kernels/MoE/group_GEMM/triton/tgroup_gemm_backwards.py:202-375; eager form testing/pytorch_reference_backwards.py:165-197),
+// as the same tiled product on transposed operands: p.x = dY^T [N, ldm] and p.w = X^T [K, ldm], both with the rows of
+// expert g in columns pad_off[g] .. pad_off[g] + roundup(m_g, 64) - 1 (zero padded), so the reduction of expert g
+// is a whole number of 64-wide steps. Every expert has the same ceil(N / BM) * ceil(K / BN) tiles; an expert
+// without rows gets zeros. p.N = rows of dW per expert (N), p.K = columns (K), p.M = ldm, p.y = dW [G * N, K].
+template <class C, bool WGRAD>
 __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[2 * C::STAGE];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
@@ -66,11 +73,15 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
   const int wm = wave % C::WM;
   const int wn = wave / C::WM;
   const int K = p.K, N = p.N;
-  const int n_tiles_n = moe_gg_cdiv(N, C::BN);
+  const int n_tiles_n = moe_gg_cdiv(WGRAD ? K : N, C::BN);
+  const int tiles_per_group = moe_gg_cdiv(N, C::BM) * n_tiles_n;  // WGRAD only
 
-  build_group_tables(p.m_sizes, p.G, p.M, C::BM, n_tiles_n, row_off, tile_off);
-  const int total = tile_off[p.G];
-  const int KT = K / 64;
+  // WGRAD: tile_off counts 64-row blocks per expert, i.e. pad_off[g] = 64 * tile_off[g]; rows are bounded by
+  // the number of gradient rows (p.skip_rows carries it, p.M is the padded leading dimension).
+  if (WGRAD) build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off);
+  else build_group_tables(p.m_sizes, p.G, p.M, C::BM, n_tiles_n, row_off, tile_off);
+  const int total = WGRAD ? p.G * tiles_per_group : tile_off[p.G];
+  const uint32_t pitch = WGRAD ? (uint32_t)p.M * 2u : (uint32_t)K * 2u;  // bytes between operand rows
 
   // Slab-load geometry: instruction i of wave w fills rows (i * NW + w) * 8 + lane / 8; the lane's
   // physical 16-byte slot is lane % 8 and must hold logical chunk slot ^ ((row >> 1) & 7).
@@ -90,21 +101,38 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
   for (int round = 0; round * (int)gridDim.x < total; ++round) {
     const int L = moe_gg_tile_of(blockIdx.x, gridDim.x, p.xcds, round);
     if (L >= total) continue;
-    const MoeGgTile t = moe_gg_decode_tile(row_off, tile_off, p.G, L, C::BM);
+    MoeGgTile t;
+    int KT;
+    const char *xg, *wg;
+    if (WGRAD) {
+      t.g = L / tiles_per_group;
+      const int rem = L - t.g * tiles_per_group;
+      t.tm = rem % moe_gg_cdiv(N, C::BM);   // tile along the rows of dW (n)
+      t.tn = rem / moe_gg_cdiv(N, C::BM);   // tile along its columns (k)
+      t.row0 = 0;
+      t.rows = N;
+      KT = tile_off[t.g + 1] - tile_off[t.g];
+      const int64_t col0 = (int64_t)tile_off[t.g] * 128;  // byte offset of the expert's padded columns
+      xg = xp + (int64_t)(t.tm * C::BM) * pitch + col0;
+      wg = wp + (int64_t)(t.tn * C::BN) * pitch + col0;
+    } else {
+      t = moe_gg_decode_tile(row_off, tile_off, p.G, L, C::BM);
+      KT = K / 64;
+      xg = xp + (int64_t)(t.row0 + t.tm * C::BM) * pitch;
+      wg = wp + ((int64_t)t.g * N + t.tn * C::BN) * pitch;
+    }
     const int m0 = t.tm * C::BM;
     const int rows_valid = min(t.rows - m0, C::BM);
     const int n0 = t.tn * C::BN;
-    const int cols_valid = min(N - n0, C::BN);
+    const int cols_valid = min((WGRAD ? K : N) - n0, C::BN);
 
-    const char* xg = xp + (int64_t)(t.row0 + m0) * K * 2;
-    const char* wg = wp + ((int64_t)t.g * N + n0) * K * 2;
     uint32_t xoff[C::XI], woff[C::WI];
 #pragma unroll
     for (int i = 0; i < C::XI; ++i)
-      xoff[i] = (uint32_t)min((i * NW + wave) * 8 + d_r, rows_valid - 1) * (uint32_t)(K * 2) + d_c * 16;
+      xoff[i] = (uint32_t)min((i * NW + wave) * 8 + d_r, rows_valid - 1) * pitch + d_c * 16;
 #pragma unroll
     for (int i = 0; i < C::WI; ++i)
-      woff[i] = (uint32_t)min((i * NW + wave) * 8 + d_r, cols_valid - 1) * (uint32_t)(K * 2) + d_c * 16;
+      woff[i] = (uint32_t)min((i * NW + wave) * 8 + d_r, cols_valid - 1) * pitch + d_c * 16;
 
     auto dma = [&](int kt, int buf) {
       const char* xs = xg + kt * 128;
@@ -150,12 +178,12 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
       __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * NR > 0 ? NM - PER * NR : 0, 0);
     };
 
-    // Prologue: slabs 0 and 1 in flight, F0 <- (slab 0, half 0).
-    dma(0, 0);
+    // Prologue: slabs 0 and 1 in flight, F0 <- (slab 0, half 0). (KT = 0: an expert without rows, WGRAD only.)
+    if (KT > 0) dma(0, 0);
     if (KT > 1) dma(1, 1);
     if (KT > 1) wait_vmcnt<C::NLOAD>(); else wait_vmcnt<0>();
     __syncthreads();
-    read_frags(0, 0, wf0, xf0);
+    if (KT > 0) read_frags(0, 0, wf0, xf0);
 
     for (int kt = 0; kt < KT; ++kt) {
       const int cur = kt & 1;
@@ -179,7 +207,8 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
     __syncthreads();
 
     // Epilogue: lane holds y[m][n .. n+3] for m = frag_m * 16 + lane % 16, n = frag_n * 16 + 4 * (lane / 16).
-    bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + (int64_t)t.g * p.col_block + n0;
+    bf16_t* yg = WGRAD ? yp + ((int64_t)t.g * N + m0) * p.ldy + n0
+                       : yp + (int64_t)(t.row0 + m0) * p.ldy + (int64_t)t.g * p.col_block + n0;
     const bool vec_ok = p.vec_store;
 #pragma unroll
     for (int i = 0; i < C::FM; ++i) {
@@ -206,9 +235,9 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
   }
 }
 
-template <class C>
+template <class C, bool WGRAD = false>
 hipError_t launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  hipLaunchKernelGGL((gg_bf16_persistent<C>), dim3(num_wg), dim3(C::NT), 0, stream, p);
+  hipLaunchKernelGGL((gg_bf16_persistent<C, WGRAD>), dim3(num_wg), dim3(C::NT), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -224,3 +253,8 @@ hipError_t gg_bf16_tiled_launch(const GgParams& p, int block_m, int num_wg, hipS
 }
 
 int gg_bf16_tiled_block_n(int block_m) { return block_m == 256 ? 256 : 128; }
+
+hipError_t gg_bf16_wgrad_launch(const GgParams& p, int block, int num_wg, hipStream_t stream) {
+  if (block == 256) return launch<Cfg<256, 256, 2, 4>, true>(p, num_wg, stream);
+  return launch<Cfg<128, 128, 2, 2>, true>(p, num_wg, stream);
+}

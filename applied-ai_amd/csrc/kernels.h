@@ -73,3 +73,16 @@ hipError_t silu_and_mul_launch(const void* in, void* out, int64_t rows, int n, h
 hipError_t invert_perm_launch(const int32_t* perm, int32_t* inv, int n, const int32_t* n_valid, hipStream_t stream);
 hipError_t combine_topk_launch(const void* y, const int32_t* inv, const void* weights, bool weights_bf16, void* out,
                                int T, int k, int d, int n_rows, hipStream_t stream);
+
+// Backward pass (gg_backward.hip, gg_bf16_prefill.hip). bf16.
+// src [B, R, C] -> dst [B, C, R].
+hipError_t transpose_batched_launch(const void* src, void* dst, int B, int R, int C, hipStream_t stream);
+// dst[c][pad_off[g] + i] = src[row_off[g] + i][g * col_block + c], experts padded to multiples of 64 columns with zeros.
+hipError_t transpose_padded_launch(const void* src, void* dst, const int32_t* m_sizes, int G, int M, int C,
+                                   int64_t src_pitch, int col_block, int64_t ldm, hipStream_t stream);
+// dst [M, C] <- the expert's own C columns (at g * col_block) of src [M, src_pitch]. C % 4 == 0, 8-byte aligned rows.
+hipError_t compact_block_launch(const void* src, void* dst, const int32_t* m_sizes, int G, int M, int C, int64_t src_pitch,
+                                int col_block, hipStream_t stream);
+// dW = dY^T X per expert on the transposed, padded operands; p.x = dY^T [N, ldm], p.w = X^T [K, ldm], p.M = ldm,
+// p.skip_rows = number of gradient rows (bound for m_sizes), p.y = dW [G * N, K] with p.ldy = K. block in {256, 128}.
+hipError_t gg_bf16_wgrad_launch(const GgParams& p, int block, int num_wg, hipStream_t stream);

@@ -77,6 +77,49 @@ def grouped_gemm_forward(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor
     return _grouped_gemm_bf16(x, w, m_sizes, OUT_BLOCK)
 
 
+def grouped_gemm_backward(grad_output: torch.Tensor, x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor):
+    """Backward pass of the bf16 grouped GEMM: returns (grad_x [M, K], grad_w [G*N, K]).
+
+    Drop-in for grouped_gemm_backward (kernels/MoE/group_GEMM/triton/tgroup_gemm_backwards.py:382-590):
+    grad_output is the gradient of grouped_gemm_forward's [M, N*G] output, of which only the expert's own column
+    block of each row is read; the [M, N] gradient of grouped_gemm is accepted as well. As in the reference, a K
+    mismatch raises ValueError, inputs are made contiguous, grad_x rows at or beyond sum(m_sizes) are zero
+    (torch.zeros_like, :442-443) and an expert without rows gets a zero grad_w block."""
+    if grad_output.dim() != 2 or x.dim() != 2 or w.dim() != 2 or m_sizes.dim() != 1:
+        raise ValueError("grad_output must be [M, N*G] or [M, N], x [M, K], w [G*N, K], m_sizes [G]")
+    G = m_sizes.shape[0]
+    M, K = x.shape
+    if K != w.shape[1]:
+        raise ValueError("K dimensions must match for grouped GEMM backward")
+    if G == 0 or w.shape[0] % G != 0:
+        raise ValueError(f"w.shape[0]={w.shape[0]} is not a multiple of G={G}")
+    N = w.shape[0] // G
+    if grad_output.shape == (M, N * G) and G > 1:
+        layout = OUT_BLOCK
+    elif grad_output.shape == (M, N):
+        layout = OUT_MN
+    else:
+        raise ValueError(f"grad_output is {tuple(grad_output.shape)}, expected [{M}, {N * G}] or [{M}, {N}]")
+    if grad_output.dtype != torch.bfloat16 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ValueError("grouped_gemm_backward takes bf16 grad_output, x and w")
+    if m_sizes.dtype != torch.int32:
+        raise ValueError("m_sizes must be int32")
+    dev = _require_cuda(grad_output, x, w, m_sizes)
+    grad_output, x, w, m_sizes = grad_output.contiguous(), x.contiguous(), w.contiguous(), m_sizes.contiguous()
+    grad_x = torch.zeros_like(x)
+    grad_w = torch.empty_like(w)
+    with torch.cuda.device(dev):
+        L = _lib.lib()
+        nbytes = L.moe_gg_grouped_gemm_backward_workspace(G, max(M, 1), N, K, layout)
+        workspace = torch.empty(max(nbytes, 256), device=dev, dtype=torch.uint8)
+        rc = L.moe_gg_grouped_gemm_backward_bf16(
+            grad_output.data_ptr(), grad_output.shape[1], layout, x.data_ptr(), w.data_ptr(), m_sizes.data_ptr(),
+            G, M, N, K, grad_x.data_ptr(), grad_w.data_ptr(), workspace.data_ptr(), workspace.numel(), _stream_ptr(dev),
+        )
+    _lib.check(rc, "moe_gg_grouped_gemm_backward_bf16")
+    return grad_x, grad_w
+
+
 def matmul_split_k(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
                    zero_offset: int = 1, groupsize: Optional[int] = None) -> torch.Tensor:
     """W4A16 split-K dequant GEMM: c = a @ dequant(b, scales, zeros).

@@ -142,6 +142,26 @@ int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int
                        void* stream);
 
 /*
+ * Backward pass of the bf16 grouped GEMM. Replaces grouped_gemm_backward
+ * (kernels/MoE/group_GEMM/triton/tgroup_gemm_backwards.py:382-590; eager form
+ * kernels/MoE/group_GEMM/triton/testing/pytorch_reference_backwards.py:165-197):
+ *   grad_x[rows of g, :] = dY_g @ w[g]            grad_w[g*N : (g+1)*N, :] = dY_g^T @ x[rows of g, :]
+ * where dY_g = grad_out[rows of g, g*N : (g+1)*N] for grad_layout = MOE_GG_OUT_BLOCK (the reference: grad_out is
+ * [M, N*G]) and grad_out[rows of g, 0 : N] for MOE_GG_OUT_MN. fp32 accumulation, bf16 results.
+ *   grad_out device bf16, leading dimension ld_go; x device [M, K]; w device [G*N, K]; m_sizes device int32 [G];
+ *   grad_x device out [M, K]: rows >= sum(m_sizes) are not written; grad_w device out [G*N, K]: fully written
+ *   (zeros for an expert without rows).
+ *   workspace: device scratch of at least moe_gg_grouped_gemm_backward_workspace(...) bytes, 256-byte aligned,
+ *   owned by the caller (the library never allocates); it holds w^T and the transposed, zero-padded copies of
+ *   grad_out and x that make every operand contiguous along its reduction dimension.
+ * Requires N % 4 == 0 and K % 4 == 0; N % 64 == 0 for the fast grad_x kernels.
+ */
+size_t moe_gg_grouped_gemm_backward_workspace(int G, int64_t M, int N, int K, int grad_layout);
+int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int grad_layout, const void* x, const void* w,
+                                      const int32_t* m_sizes, int G, int64_t M, int N, int K, void* grad_x, void* grad_w,
+                                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Glue between the two grouped GEMMs of a whole MoE layer, as in the reference's fused_moe
  * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:222-296; oracle torch_moe,
  * kernels/triton/inference/col_major_moe_gemm/test_moe_gemm.py:16-30). All data bf16.

@@ -12,7 +12,7 @@
  * Parity status:
  *   orc_offsets, orc_grouped_gemm, orc_route, orc_moe_align_block_size, orc_topk,
  *   orc_w4_dequant, orc_e4m3_*, orc_fp8_groupwise_quant, orc_grouped_gemm_fp8 (rowwise),
- *   orc_silu_and_mul, orc_fused_moe: pinned.
+ *   orc_silu_and_mul, orc_fused_moe, orc_grouped_gemm_backward: pinned.
  *   orc_fp8_block_quant_weight (128x128 weight quantiser): PARITY UNPINNED - the reference calls an
  *   un-vendored FBGEMM routine for it (kernels/needs_perf_help/fp8_gemm_bench.py:16-21); this file
  *   defines it by analogy with the 1x128 quantiser and only its GEMM consumer is checked.
@@ -66,6 +66,41 @@ void orc_grouped_gemm(const float* x, const float* w, const int32_t* m_sizes, in
     }
   }
   (void)M;
+}
+
+/* ---- backward of the grouped GEMM ---------------------------------------------------------------
+ * kernels/MoE/group_GEMM/triton/testing/pytorch_reference_backwards.py:165-197 (per expert
+ * grad_x[rows] = dY_g @ w[g], grad_w[g] = dY_g^T @ x[rows]; outputs start from zeros) which is what
+ * grouped_gemm_backward (tgroup_gemm_backwards.py:382-590) computes. dY_g = go[rows of g, g*col_block .. + N).
+ * Pinned by: torch.autograd through the per-expert forward loop of fast_verification.py:83-99,
+ * G = 1 equals the dense dY @ w and dY^T @ x (numpy float64), and the adjoint identity
+ * <dY, forward(x, w)> = <grad_x, x> = <grad_w, w>. */
+void orc_grouped_gemm_backward(const float* go, int64_t ld_go, int col_block, const float* x, const float* w,
+                               const int32_t* m_sizes, int G, int64_t M, int N, int K, float* grad_x,
+                               float* grad_w) {
+  memset(grad_x, 0, sizeof(float) * (size_t)M * K);
+  memset(grad_w, 0, sizeof(float) * (size_t)G * N * K);
+  int64_t off = 0;
+  for (int g = 0; g < G; ++g) {
+    int64_t m = m_sizes[g];
+    if (m <= 0) continue;
+    const float* dy = go + off * ld_go + (int64_t)g * col_block;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < m; ++i)
+      for (int k = 0; k < K; ++k) {
+        double acc = 0.0;
+        for (int n = 0; n < N; ++n) acc += (double)dy[i * ld_go + n] * (double)w[((int64_t)g * N + n) * K + k];
+        grad_x[(off + i) * K + k] = (float)acc;
+      }
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; ++n)
+      for (int k = 0; k < K; ++k) {
+        double acc = 0.0;
+        for (int64_t i = 0; i < m; ++i) acc += (double)dy[i * ld_go + n] * (double)x[(off + i) * K + k];
+        grad_w[((int64_t)g * N + n) * K + k] = (float)acc;
+      }
+    off += m;
+  }
 }
 
 /* ---- top-k routing ------------------------------------------------------------------------------

@@ -69,6 +69,22 @@ def grouped_gemm(x, w, m_sizes, block_layout=False, fill=np.nan):
     return y
 
 
+def grouped_gemm_backward(grad_output, x, w, m_sizes):
+    """fp32 (grad_x [M, K], grad_w [G*N, K]) of the grouped GEMM (pytorch_reference_backwards.py:165-197).
+    grad_output is [M, N*G] (each expert reads its own column block) or [M, N]."""
+    go, x, w, m = _f32(grad_output), _f32(x), _f32(w), _i32(m_sizes)
+    G = m.shape[0]
+    M, K = x.shape
+    N = w.shape[0] // G
+    block = go.shape[1] == N * G and G > 1
+    gx = np.empty((M, K), dtype=np.float32)
+    gw = np.empty((G * N, K), dtype=np.float32)
+    _l().orc_grouped_gemm_backward(_p(go), ctypes.c_int64(go.shape[1]), ctypes.c_int(N if block else 0), _p(x), _p(w),
+                                   _p(m), ctypes.c_int(G), ctypes.c_int64(M), ctypes.c_int(N), ctypes.c_int(K),
+                                   _p(gx), _p(gw))
+    return gx, gw
+
+
 def topk(logits, k):
     """Top-k expert ids per token, descending score, ties to the lower index (test_moe_gemm.py:54-57)."""
     lg = _f32(logits)

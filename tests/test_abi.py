@@ -76,6 +76,16 @@ def test_argument_errors_of_the_other_entry_points(lib):
     assert lib.moe_gg_combine_topk(None, None, None, 1, None, 4, 2, 8, 8, None) == -1        # fp16 weights unsupported
     assert lib.moe_gg_combine_topk(None, None, None, 2, None, 4, 0, 8, 8, None) == -1        # k <= 0
     assert lib.moe_gg_fp8_groupwise_quant(None, 1, None, None, 128, None) == -1              # fp16 input unsupported
+    bw = lib.moe_gg_grouped_gemm_backward_bf16
+    ws = lib.moe_gg_grouped_gemm_backward_workspace
+    assert bw(None, 128, 7, None, None, None, 2, 8, 64, 64, None, None, None, 0, None) == -1     # bad layout
+    assert bw(None, 64, 1, None, None, None, 2, 8, 64, 64, None, None, None, 0, None) == -2      # ld_go < N * G
+    assert bw(None, 128, 1, None, None, None, 2, 8, 64, 64, None, None, None, 0, None) == -1     # null pointers
+    assert bw(None, 128, 1, None, None, None, 0, 8, 64, 64, None, None, None, 0, None) == 0      # G == 0
+    assert ws(0, 8, 64, 64, 1) == 0
+    # w^T + dY^T and x^T at ldm = (M / 64 + G) * 64 columns + the compacted dY; each part 256-byte aligned
+    assert ws(2, 100, 64, 128, 1) == 2 * 64 * 128 * 2 + 64 * 192 * 2 + 128 * 192 * 2 + 100 * 64 * 2 + 0
+    assert ws(2, 100, 64, 128, 0) == 2 * 64 * 128 * 2 + 64 * 192 * 2 + 128 * 192 * 2
     assert lib.moe_gg_set_variant(9, 0) == -1
     assert lib.moe_gg_set_variant(0, -1) == 0
 

@@ -1,0 +1,111 @@
+"""GPU parity of the grouped-GEMM backward pass against the double-precision oracle.
+Bar: |g - ref| <= 1e-2 + 1e-2 |ref| on both gradients, the tolerance of the reference's own check
+(kernels/MoE/group_GEMM/triton/testing/fast_verification.py:110-122, rtol = atol = 1e-2 on bf16)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.gpu_util import to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def bf(t):
+    return t.to(torch.bfloat16)
+
+
+def even_split(M, G):
+    # fast_verification.py:42-47
+    return [M // G + (1 if i < M % G else 0) for i in range(G)]
+
+
+def run_case(sizes, M, N, K, seed, block_layout=True, scale=1.0):
+    import applied_ai_amd as A
+
+    G = len(sizes)
+    gen = torch.Generator().manual_seed(seed)
+    x = bf(torch.randn(M, K, generator=gen) * scale)
+    w = bf(torch.randn(G * N, K, generator=gen) * scale)
+    go = bf(torch.randn(M, N * G if block_layout else N, generator=gen) * scale)
+    m = torch.tensor(sizes, dtype=torch.int32)
+    gx, gw = A.grouped_gemm_backward(go.cuda(), x.cuda(), w.cuda(), m.cuda())
+    assert gx.shape == x.shape and gw.shape == w.shape and gx.dtype == torch.bfloat16 and gw.dtype == torch.bfloat16
+    rx, rw = O.grouped_gemm_backward(go.float().numpy(), x.float().numpy(), w.float().numpy(), sizes)
+    for name, got, ref in (("grad_x", to_np(gx), rx), ("grad_w", to_np(gw), rw)):
+        d = np.abs(got - ref)
+        assert np.all(d <= 1e-2 + 1e-2 * np.abs(ref)), (name, sizes[:8], M, N, K, float(d.max()))
+    return to_np(gx), to_np(gw)
+
+
+def test_fast_verification_case():
+    # G = 20, M = 1024, N = 512, K = 256, randn data (fast_verification.py:31-40)
+    run_case(even_split(1024, 20), 1024, 512, 256, seed=1)
+
+
+@pytest.mark.parametrize("sizes,M,N,K", [
+    ([64, 64], 128, 128, 128),
+    ([100, 0, 27, 1], 128, 64, 192),            # ragged, an empty expert, a single row
+    ([0, 0, 0], 64, 64, 64),                    # nothing routed: grad_w all zeros
+    ([37, 90, 200, 3, 0, 70], 448, 256, 320),   # rows beyond sum(m_sizes) stay zero in grad_x
+    ([513, 255], 768, 320, 448),                # N and K not multiples of the tile
+    ([300] * 8, 2400, 512, 512),                # enough tiles for the 256 x 256 weight-gradient kernel
+    ([17, 5], 24, 72, 40),                      # reduction dimension of grad_x not a multiple of 64
+])
+def test_ragged_shapes(sizes, M, N, K):
+    gx, gw = run_case(sizes, M, N, K, seed=7, scale=0.5)
+    assert not gx[sum(sizes):].any()
+    for g, m in enumerate(sizes):
+        if m == 0:
+            assert not gw[g * N:(g + 1) * N].any()
+
+
+def test_mn_gradient_layout_and_single_group():
+    run_case([40, 88], 128, 128, 64, seed=9, block_layout=False)
+    run_case([96], 96, 128, 128, seed=10)
+
+
+def test_adjoint_identity_at_training_size():
+    """<dY, forward(x, w)> = <grad_x, x> = <grad_w, w> at a size the oracle does not reach in seconds:
+    16 experts, 8192 rows, N = K = 2048. dY = forward(x, w) itself, so the pairing is a sum of squares and a
+    dropped or doubled block shows as a relative change."""
+    import applied_ai_amd as A
+
+    G, M, N, K = 16, 8192, 2048, 2048
+    gen = torch.Generator().manual_seed(12)
+    sizes = torch.randint(300, 700, (G,), generator=gen)
+    sizes[3] = 0
+    sizes = (sizes.float() / sizes.sum() * (M - 100)).to(torch.int32)
+    x = bf(torch.randn(M, K, generator=gen) / 8).cuda()
+    w = bf(torch.randn(G * N, K, generator=gen) / 8).cuda()
+    m = sizes.cuda()
+    y = A.grouped_gemm_forward(x, w, m)
+    go = torch.where(torch.isfinite(y), y, torch.zeros_like(y))   # unwritten parts of y are uninitialised
+    gx, gw = A.grouped_gemm_backward(go, x, w, m)
+    off = 0
+    lhs = 0.0
+    for g in range(G):
+        n = int(sizes[g])
+        lhs += float((go[off:off + n, g * N:(g + 1) * N].double() * y[off:off + n, g * N:(g + 1) * N].double()).sum())
+        off += n
+    ax = float((gx.double() * x.double()).sum())
+    aw = float((gw.double() * w.double()).sum())
+    # every term carries one bf16 rounding (2^-9 relative, random sign): the sums agree far below 1e-3
+    assert lhs > 0 and abs(lhs - ax) <= 1e-3 * lhs and abs(lhs - aw) <= 1e-3 * lhs, (lhs, ax, aw)
+    assert not gx[off:].any() and not gw[3 * N:4 * N].any()
+
+
+def test_errors():
+    import applied_ai_amd as A
+
+    x = torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(2 * 64, 128, dtype=torch.bfloat16, device="cuda")
+    go = torch.zeros(8, 128, dtype=torch.bfloat16, device="cuda")
+    m = torch.tensor([4, 4], dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError, match="K dimensions must match"):   # tgroup_gemm_backwards.py:430-433
+        A.grouped_gemm_backward(go, x, w, m)
+    w = torch.zeros(2 * 64, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        A.grouped_gemm_backward(go[:, :100], x, w, m)
+    with pytest.raises(RuntimeError):
+        A.grouped_gemm_backward(go.cpu(), x, w, m)

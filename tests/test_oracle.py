@@ -367,3 +367,52 @@ def test_w4a16_grouped_and_int4_layer_compose_pinned_parts():
             h = h[:n2] / (1 + np.exp(-h[:n2])) * h[n2:]
             exp[t] += h @ wb[e]
     np.testing.assert_allclose(got, exp, rtol=1e-4, atol=1e-5)
+
+
+def test_grouped_gemm_backward_vs_autograd_and_closed_forms():
+    # torch.autograd through the per-expert forward loop (fast_verification.py:83-99), float64.
+    rng = np.random.default_rng(31)
+    for G, sizes, N, K, pad in [(3, [5, 0, 9], 8, 12, 2), (4, [7, 7, 7, 7], 16, 8, 0), (1, [11], 4, 20, 0)]:
+        M = sum(sizes) + pad
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        w = rng.standard_normal((G * N, K)).astype(np.float32)
+        go = rng.standard_normal((M, N * G)).astype(np.float32)
+        gx, gw = O.grouped_gemm_backward(go, x, w, sizes)
+        xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+        wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+        y = torch.zeros((M, N * G), dtype=torch.float64)
+        s = 0
+        for g, m in enumerate(sizes):
+            if m > 0:
+                y[s:s + m, g * N:(g + 1) * N] = xt[s:s + m] @ wt[g * N:(g + 1) * N].T
+            s += m
+        y.backward(torch.tensor(go, dtype=torch.float64))
+        np.testing.assert_allclose(gx, xt.grad.numpy(), rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(gw, wt.grad.numpy(), rtol=1e-5, atol=1e-5)
+        # rows beyond sum(m_sizes) and experts without rows get zeros
+        assert not gx[sum(sizes):].any()
+        for g, m in enumerate(sizes):
+            if m == 0:
+                assert not gw[g * N:(g + 1) * N].any()
+        # adjoint identity with the pinned forward: <dY, y> = <grad_x, x> = <grad_w, w>
+        yf = O.grouped_gemm(x, w, sizes, block_layout=True, fill=0.0).astype(np.float64)
+        lhs = float((go.astype(np.float64) * yf).sum())
+        assert abs(lhs - float((gx.astype(np.float64) * x).sum())) < 1e-3 * max(1.0, abs(lhs))
+        assert abs(lhs - float((gw.astype(np.float64) * w).sum())) < 1e-3 * max(1.0, abs(lhs))
+        # the [M, N] gradient layout reads the same numbers
+        go_mn = np.zeros((M, N), dtype=np.float32)
+        s = 0
+        for g, m in enumerate(sizes):
+            go_mn[s:s + m] = go[s:s + m, g * N:(g + 1) * N]
+            s += m
+        if G > 1:
+            gx2, gw2 = O.grouped_gemm_backward(go_mn, x, w, sizes)
+            np.testing.assert_array_equal(gx, gx2)
+            np.testing.assert_array_equal(gw, gw2)
+    # G = 1: dense products
+    x = rng.standard_normal((6, 5)).astype(np.float32)
+    w = rng.standard_normal((4, 5)).astype(np.float32)
+    go = rng.standard_normal((6, 4)).astype(np.float32)
+    gx, gw = O.grouped_gemm_backward(go, x, w, [6])
+    np.testing.assert_allclose(gx, go.astype(np.float64) @ w, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(gw, go.astype(np.float64).T @ x, rtol=1e-6, atol=1e-6)
