@@ -325,7 +325,11 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
   const int64_t t256 = (int64_t)G * ((N + 255) / 256) * ((K + 255) / 256);
-  return (int)gg_bf16_wgrad_launch(p, t256 >= num_wg ? 256 : 128, num_wg, s);
+  const int v = g_variant[MOE_GG_OP_GG_BF16].load();
+  if (v == MOE_GG_GG_TILED_256) return (int)gg_bf16_wgrad_launch(p, 256, num_wg, s);
+  if (v == MOE_GG_GG_TILED_128) return (int)gg_bf16_wgrad_launch(p, 128, num_wg, s);
+  if (v == MOE_GG_GG_PINGPONG_256 || (v < 0 && t256 * 4 >= (int64_t)num_wg * 3)) return (int)gg_bf16_pingpong_wgrad_launch(p, num_wg, s);
+  return (int)gg_bf16_wgrad_launch(p, 128, num_wg, s);
 }
 
 int moe_gg_silu_and_mul(const void* in, void* out, int64_t rows, int n, void* stream) {

@@ -15,6 +15,7 @@ namespace {
 
 constexpr int TT = 64;  // tile edge
 
+
 // Reads tile[r][c] = src[(r0 + r) * src_pitch + c0 + c] for r < rvalid, c < cvalid (zeros elsewhere) and writes
 // dst[(dst_row0 + c0 + c) * dst_pitch + q0 + r] for c < cvalid and r < rstore. 256 threads; 16-byte global accesses
 // where the addresses allow, 2-byte accesses elsewhere. tile: 64 rows of 33 dwords (64 values + padding).
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(256) void transpose_batched_kernel(const uint16_t* 
 
 // Per-expert padded transpose: src rows are expert-sorted; expert g owns rows row_off[g] .. + m_g - 1 and, in src,
 // columns g * col_block .. + C - 1 (col_block = 0: the same C columns for every expert). dst [C, ldm]:
-// dst[c][pad_off[g] + i] = src[row_off[g] + i][g * col_block + c] for i < m_g, zero for m_g <= i < roundup(m_g, 64).
+// dst[c][pad_off[g] + i] = src[row_off[g] + i][g * col_block + c] for i < m_g, zero for m_g <= i < max(64, roundup(m_g, 64)).
 // Grid (upper bound on the number of 64-row blocks, ceil(C / 64)); blocks beyond the real count exit.
 __global__ __launch_bounds__(256) void transpose_padded_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
                                                                const int32_t* __restrict__ m_sizes, int G, int M, int C,
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(256) void transpose_padded_kernel(const uint16_t* _
   __shared__ uint32_t tile[TT][TT / 2 + 1];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t blk_off[MOE_GG_MAX_GROUPS + 1];
-  build_group_tables(m_sizes, G, M, TT, 1, row_off, blk_off);
+  build_group_tables(m_sizes, G, M, TT, 1, row_off, blk_off, 0, 1);  // an expert without rows owns one block of zeros
   const int L = blockIdx.x;
   if (L >= blk_off[G]) return;
   const int g = moe_gg_find_group(blk_off, G, L);

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
 
   // WGRAD: tile_off counts 64-row blocks per expert, i.e. pad_off[g] = 64 * tile_off[g]; rows are bounded by
   // the number of gradient rows (p.skip_rows carries it, p.M is the padded leading dimension).
-  if (WGRAD) build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off);
+  if (WGRAD) build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
   else build_group_tables(p.m_sizes, p.G, p.M, C::BM, n_tiles_n, row_off, tile_off);
   const int total = WGRAD ? p.G * tiles_per_group : tile_off[p.G];
   const uint32_t pitch = WGRAD ? (uint32_t)p.M * 2u : (uint32_t)K * 2u;  // bytes between operand rows
@@ -178,12 +178,12 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
       __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * NR > 0 ? NM - PER * NR : 0, 0);
     };
 
-    // Prologue: slabs 0 and 1 in flight, F0 <- (slab 0, half 0). (KT = 0: an expert without rows, WGRAD only.)
-    if (KT > 0) dma(0, 0);
+    // Prologue: slabs 0 and 1 in flight, F0 <- (slab 0, half 0).
+    dma(0, 0);
     if (KT > 1) dma(1, 1);
     if (KT > 1) wait_vmcnt<C::NLOAD>(); else wait_vmcnt<0>();
     __syncthreads();
-    if (KT > 0) read_frags(0, 0, wf0, xf0);
+    read_frags(0, 0, wf0, xf0);
 
     for (int kt = 0; kt < KT; ++kt) {
       const int cur = kt & 1;

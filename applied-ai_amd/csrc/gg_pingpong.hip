@@ -56,7 +56,13 @@ constexpr int STAGE = (BM + BN) * 128;
 constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x 256 B of weight-block scales
 
 // Operand kinds.
-constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2;
+// OP_BF16_WGRAD: the weight gradient of the bf16 layer, dW[g][n][k] = sum over the rows m of expert g of
+// dY[m][n] * X[m][k] (kernels/MoE/group_GEMM/triton/tgroup_gemm_backwards.py:202-375), as the same product on
+// transposed operands: p.x = dY^T [N, ldm], p.w = X^T [K, ldm], the rows of expert g zero-padded to whole
+// 64-column blocks (at least one), so the reduction of a tile is a whole number of K steps that depends on
+// its expert. Every expert has the same ceil(N / 256) * ceil(K / 256) tiles. p.M = ldm, p.skip_rows = number
+// of gradient rows, p.y = dW [G * N, K].
+constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3;
 
 // 64 lanes x 16 B (or 4 B) from global memory straight into LDS: lane l's bytes land at lds_addr + 16 l
 // (4 l). Issued from inline assembly so that the compiler does not serialise the in-flight slab against
@@ -106,13 +112,15 @@ struct Cursor {
   int x_last;       // last valid activation row of the tile (rows beyond it re-read this one)
   int w_last;       // last valid weight row of the tile
   int ws_second;    // block mode: byte offset of the second column block's scales (0 if there is none)
+  int KT;           // K steps of the cursor's tile
   int round, kt, step;
 };
 
 template <int GRP, int OP>
 DEVINL void run_group(const GgParams& p, const Shared& sh) {
-  constexpr bool FP8 = OP != OP_BF16;
+  constexpr bool FP8 = OP == OP_FP8_ROW || OP == OP_FP8_BLOCK;
   constexpr bool BLOCK = OP == OP_FP8_BLOCK;
+  constexpr bool WGRAD = OP == OP_BF16_WGRAD;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -120,9 +128,35 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   const int wn = wave >> 1;
   const int gw = wave & 3;  // wave index inside its group
   const int N = p.N;
-  const uint32_t KROW = (uint32_t)p.K * (FP8 ? 1u : 2u);  // bytes per operand row
-  const int KT = (int)(KROW / 128u);
+  const uint32_t KROW = WGRAD ? (uint32_t)p.M * 2u : (uint32_t)p.K * (FP8 ? 1u : 2u);  // bytes per operand row
+  const int KT_fwd = (int)((uint32_t)p.K * (FP8 ? 1u : 2u) / 128u);  // K steps of every forward tile
+  const int NCOLS = WGRAD ? p.K : N;                                 // output columns of a group
+  const int wg_ntm = moe_gg_cdiv(N, BM);                             // WGRAD: tiles along the rows of dW
+  const int wg_tpg = wg_ntm * moe_gg_cdiv(p.K, BN);                  // WGRAD: tiles per expert
   const int nwg = gridDim.x;
+  // Tile of a round. Forward: rows of x / rows of w[g]. WGRAD: rows of dY^T (n) / rows of X^T (k), both at the
+  // column offset of the expert's padded block; t.row0 = first row of the expert's block of dW, t.rows = N.
+  struct TileRef { MoeGgTile t; int KT; int64_t xoff, woff; };
+  auto tile_ref = [&](int round) {
+    TileRef r;
+    const int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, round);
+    if (WGRAD) {
+      const int g = uni(L / wg_tpg);
+      const int rem = L - g * wg_tpg;
+      r.t.g = g; r.t.tn = uni(rem / wg_ntm); r.t.tm = rem - r.t.tn * wg_ntm;
+      r.t.row0 = g * N; r.t.rows = N;
+      const int b0 = uni(sh.tile_off[g]);
+      r.KT = uni(sh.tile_off[g + 1]) - b0;
+      r.xoff = (int64_t)(r.t.tm * BM) * KROW + (int64_t)b0 * 128;
+      r.woff = (int64_t)(r.t.tn * BN) * KROW + (int64_t)b0 * 128;
+    } else {
+      r.t = uni_tile(moe_gg_decode_tile(sh.row_off, sh.tile_off, p.G, L, BM));
+      r.KT = KT_fwd;
+      r.xoff = (int64_t)(r.t.row0 + r.t.tm * BM) * KROW;
+      r.woff = ((int64_t)r.t.g * N + r.t.tn * BN) * KROW;
+    }
+    return r;
+  };
 
   // Slab-load geometry: an instruction fills 8 rows (1 KB of LDS); lane -> row lane / 8, physical
   // 16-byte slot lane % 8, which must hold logical chunk slot ^ ((row >> 1) & 7). Inside a group the
@@ -144,21 +178,23 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   auto cursor_tile = [&](int round) {
     c.round = round;
     if (round >= sh.n_my) return;  // past the last tile: keep re-loading the last tile (never read)
-    const MoeGgTile t = uni_tile(moe_gg_decode_tile(sh.row_off, sh.tile_off, p.G, moe_gg_tile_of(blockIdx.x, nwg, p.xcds, round), BM));
+    const TileRef tr = tile_ref(round);
+    const MoeGgTile& t = tr.t;
     const int m0 = t.tm * BM, n0 = t.tn * BN;
+    c.KT = tr.KT;
     c.x_last = min(t.rows - m0, BM) - 1;
-    c.w_last = min(N - n0, BN) - 1;
-    c.xg = uni_ptr(xp + (int64_t)(t.row0 + m0) * KROW);
-    c.wg = uni_ptr(wp + ((int64_t)t.g * N + n0) * KROW);
+    c.w_last = min(NCOLS - n0, BN) - 1;
+    c.xg = uni_ptr(xp + tr.xoff);
+    c.wg = uni_ptr(wp + tr.woff);
     if (BLOCK) {
-      c.xsg = uni_ptr((const char*)(p.x_scale + (int64_t)(t.row0 + m0) * KT));
-      c.wsg = uni_ptr((const char*)(p.w_scale + (((int64_t)t.g * N + n0) / 128) * KT));
-      c.ws_second = n0 + 128 < N ? KT * 4 : 0;
+      c.xsg = uni_ptr((const char*)(p.x_scale + (int64_t)(t.row0 + m0) * KT_fwd));
+      c.wsg = uni_ptr((const char*)(p.w_scale + (((int64_t)t.g * N + n0) / 128) * KT_fwd));
+      c.ws_second = n0 + 128 < N ? KT_fwd * 4 : 0;
     }
   };
   auto cursor_next = [&]() {
     ++c.step;
-    if (++c.kt == KT) {
+    if (++c.kt == c.KT) {
       c.kt = 0;
       cursor_tile(c.round + 1);
     }
@@ -177,7 +213,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   // 64 gw .. 64 gw + 63 (one per lane) and a private copy of the two weight-block scales (lanes 0-31 the
   // first column block, lanes 32-63 the second).
   auto dma_xscale = [&]() {
-    const uint32_t off = (uint32_t)min(gw * 64 + lane, c.x_last) * (uint32_t)(KT * 4);
+    const uint32_t off = (uint32_t)min(gw * 64 + lane, c.x_last) * (uint32_t)(KT_fwd * 4);
     dma4(c.xsg + c.kt * 4, off, lds_scale + (c.step & 1) * SCALE_BYTES + gw * 256);
   };
   auto dma_wscale = [&]() {
@@ -216,10 +252,12 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
 
   int step = 0;
   for (int r = 0; r < sh.n_my; ++r) {
-    const MoeGgTile t = uni_tile(moe_gg_decode_tile(sh.row_off, sh.tile_off, p.G, moe_gg_tile_of(blockIdx.x, nwg, p.xcds, r), BM));
+    const TileRef tr = tile_ref(r);
+    const MoeGgTile& t = tr.t;
+    const int KT = tr.KT;
     const int m0 = t.tm * BM, n0 = t.tn * BN;
     const int rows_valid = min(t.rows - m0, BM);
-    const int cols_valid = min(N - n0, BN);
+    const int cols_valid = min(NCOLS - n0, BN);
     // Activation fragments of this wave that hold at least one valid row (fragments are dealt
     // alternately to wm = 0 / 1, so a short tile shortens every wave's C phase alike).
     const int nfm = min(FM, max(0, ((rows_valid + 15) / 16 - wm + WM - 1) / WM));
@@ -320,7 +358,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       // 32-bit lane offset. The lane indices pass through an empty asm so that the address arithmetic
       // is redone here for every tile instead of being hoisted out of the tile loop, where it would
       // occupy (and spill) registers during the K loop.
-      bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + (int64_t)t.g * p.col_block + n0;
+      bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + (WGRAD ? 0 : (int64_t)t.g * p.col_block) + n0;
       int er = fr, eq = fq;
       asm volatile("" : "+v"(er), "+v"(eq));
       // Row-wise fp8 scales (groupgemm.py:374-384): y *= x_scale[m] * w_scale[g * N + n].
@@ -388,8 +426,10 @@ DEVINL void pingpong_body(const GgParams& p) {
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t tile_off[MOE_GG_MAX_GROUPS + 1];
 
-  build_group_tables(p.m_sizes, p.G, p.M, BM, moe_gg_cdiv(p.N, BN), row_off, tile_off, p.skip_rows);
-  const int total = uni(tile_off[p.G]);
+  // WGRAD: tile_off counts the 64-column blocks of the padded operands (at least one per expert).
+  if (OP == OP_BF16_WGRAD) build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
+  else build_group_tables(p.m_sizes, p.G, p.M, BM, moe_gg_cdiv(p.N, BN), row_off, tile_off, p.skip_rows);
+  const int total = OP == OP_BF16_WGRAD ? p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN) : uni(tile_off[p.G]);
   const int nwg = gridDim.x;
   // Tiles of this workgroup: rounds 0 .. n_my - 1 (tile ids grow with the round).
   int n_my = 0;
@@ -403,6 +443,7 @@ DEVINL void pingpong_body(const GgParams& p) {
 }
 
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_body<OP_BF16>(p); }
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise(GgParams p) { pingpong_body<OP_FP8_ROW>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpong_body<OP_FP8_BLOCK>(p); }
 
@@ -410,6 +451,11 @@ __global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpo
 
 hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream) {
   hipLaunchKernelGGL(gg_bf16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t gg_bf16_pingpong_wgrad_launch(const GgParams& p, int num_wg, hipStream_t stream) {
+  hipLaunchKernelGGL(gg_bf16_pingpong_wgrad, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -18,10 +18,10 @@ DEVINL long long wave_incl_scan_i64(long long x) {
 // Must be called by every thread of the workgroup (it contains barriers).
 // row_off / tile_off: LDS arrays of G + 1 entries, G <= MOE_GG_MAX_GROUPS.
 // Groups with at most skip_rows rows keep their rows in row_off but get no tiles (another kernel
-// of the same call computes them).
+// of the same call computes them). min_tiles: lower bound of every group's tile count (also of an empty group).
 DEVINL void build_group_tables(const int32_t* __restrict__ m_sizes, int G, int M, int BM, int n_tiles_n,
-                               int32_t* row_off, int32_t* tile_off, int skip_rows = 0) {
-  auto tiles_of = [&](int rows) { return rows > skip_rows ? moe_gg_cdiv(rows, BM) * n_tiles_n : 0; };
+                               int32_t* row_off, int32_t* tile_off, int skip_rows = 0, int min_tiles = 0) {
+  auto tiles_of = [&](int rows) { return max(min_tiles, rows > skip_rows ? moe_gg_cdiv(rows, BM) * n_tiles_n : 0); };
   const int per = (G + 63) >> 6;
   if (wave_id() == 0) {
     const int g0 = lane_id() * per;

@@ -213,6 +213,32 @@ def secondary_workloads(torch, A, dev):
                 "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong (two launches) + glue kernels", "achieved": round(flop / ms / 1e9, 1),
                              "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
                              "traffic": None}})
+    del h, w1, w2
+
+    # ---- backward of the grouped GEMM (training), Mixtral w1 shape, [M, N] gradient ----
+    G, M, N, K = 8, 8192, 14336, 4096
+    ms_dev = torch.tensor([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], dtype=torch.int32, device=dev)  # config 2's routing
+    x = (torch.randn(M, K, device=dev, generator=gen) / 8).to(torch.bfloat16)
+    w = torch.empty(G * N, K, device=dev, dtype=torch.bfloat16)
+    for g in range(G):
+        w[g * N:(g + 1) * N] = (torch.randn(N, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    go = (torch.randn(M, N, device=dev, generator=gen) / 8).to(torch.bfloat16)
+    gx = torch.zeros_like(x)
+    gw = torch.empty_like(w)
+    nbytes = lib.moe_gg_grouped_gemm_backward_workspace(G, M, N, K, 0)
+    wsp = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+    def call():
+        lib.moe_gg_grouped_gemm_backward_bf16(go.data_ptr(), N, 0, x.data_ptr(), w.data_ptr(), ms_dev.data_ptr(), G, M, N, K,
+                                              gx.data_ptr(), gw.data_ptr(), wsp.data_ptr(), nbytes, stream)
+
+    ms = event_time_ms(torch, call, 5, 2)
+    flop = 4.0 * M * N * K
+    out.append({"workload": "grouped GEMM backward (grad_x and grad_w), Mixtral 8x7B w1 shape: 8192 rows, K=4096, N=14336, 8 experts, bf16",
+                "ms_per_launch": round(ms, 3), "value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
+                "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong + gg_bf16_pingpong_wgrad + three transposes",
+                             "achieved": round(flop / ms / 1e9, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                             "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None}})
     return out
 
 
