@@ -250,6 +250,29 @@ int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int
   return (int)gather_rows_launch(x, perm, k, out, (int)n, row_bytes, (hipStream_t)stream);
 }
 
+int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M,
+                                    int n, int K, int64_t ldy, void* stream) {
+  if (G < 0 || M < 0 || n < 0 || K < 0) return MOE_GG_EINVAL;
+  if (ldy < n) return MOE_GG_ESHAPE;
+  if (G == 0 || M == 0 || n == 0) return MOE_GG_OK;
+  if (!x || !w || !y || !m_sizes) return MOE_GG_EINVAL;
+  if (G > MOE_GG_MAX_GROUPS_ABI || M > INT32_MAX || ldy > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (K == 0 || K % 64 != 0 || n % 4 != 0 || (int64_t)2 * n * K >= INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (!aligned(x, 16) || !aligned(w, 16) || !aligned(y, 2) || !aligned(m_sizes, 4)) return MOE_GG_EALIGN;
+  const DeviceInfo* di = nullptr;
+  int rc = current_device_info(&di);
+  if (rc != MOE_GG_OK) return rc;
+  GgParams p{};
+  p.x = x; p.w = w; p.y = y; p.m_sizes = m_sizes;
+  p.G = G; p.M = (int)M; p.N = 2 * n; p.K = K;
+  p.ldy = (int)ldy;
+  p.vec_store = aligned(y, 8) && ldy % 4 == 0;
+  p.xcds = di->xcds;
+  int num_wg = di->cus - di->cus % p.xcds;
+  if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
+  return (int)gg_bf16_pingpong_swiglu_launch(p, num_wg, (hipStream_t)stream);
+}
+
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 // Leading dimension of the transposed operands: every expert padded to whole 64-row blocks.
 static int64_t backward_ldm(int G, int64_t M) { return (M / 64 + G) * 64; }

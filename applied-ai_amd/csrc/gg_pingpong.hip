@@ -62,7 +62,15 @@ constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x
 // 64-column blocks (at least one), so the reduction of a tile is a whole number of K steps that depends on
 // its expert. Every expert has the same ceil(N / 256) * ceil(K / 256) tiles. p.M = ldm, p.skip_rows = number
 // of gradient rows, p.y = dW [G * N, K].
-constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3;
+// OP_BF16_SWIGLU: the first GEMM of a gated MoE layer with SiLU-and-mul in the epilogue
+// (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:271-284: GEMM with w1 [E, 2n, K], then
+// ops.silu_and_mul): y[m][c] = silu(x[m] . w[g][c]) * (x[m] . w[g][n + c]), y is [M, n]. The layout of w is the
+// reference's (gate rows 0 .. n-1, up rows n .. 2n-1 of every expert); a tile takes 128 gate rows and the 128 up
+// rows of the same output columns, placed in LDS so that every wave holds the gate and the up value of its own
+// 32 output columns: weight-tile row 64 wn + 32 h + c (h = 0 gate, 1 up) is output column 32 wn + c.
+// Both products are rounded to bf16 before the activation, as they are when the GEMM output is stored first.
+// p.N = 2n.
+constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4;
 
 // 64 lanes x 16 B (or 4 B) from global memory straight into LDS: lane l's bytes land at lds_addr + 16 l
 // (4 l). Issued from inline assembly so that the compiler does not serialise the in-flight slab against
@@ -121,6 +129,8 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   constexpr bool FP8 = OP == OP_FP8_ROW || OP == OP_FP8_BLOCK;
   constexpr bool BLOCK = OP == OP_FP8_BLOCK;
   constexpr bool WGRAD = OP == OP_BF16_WGRAD;
+  constexpr bool SWIGLU = OP == OP_BF16_SWIGLU;
+  constexpr int TILE_COLS = SWIGLU ? BN / 2 : BN;  // output columns of a tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -130,7 +140,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   const int N = p.N;
   const uint32_t KROW = WGRAD ? (uint32_t)p.M * 2u : (uint32_t)p.K * (FP8 ? 1u : 2u);  // bytes per operand row
   const int KT_fwd = (int)((uint32_t)p.K * (FP8 ? 1u : 2u) / 128u);  // K steps of every forward tile
-  const int NCOLS = WGRAD ? p.K : N;                                 // output columns of a group
+  const int NCOLS = WGRAD ? p.K : (SWIGLU ? N / 2 : N);               // output columns of a group
   const int wg_ntm = moe_gg_cdiv(N, BM);                             // WGRAD: tiles along the rows of dW
   const int wg_tpg = wg_ntm * moe_gg_cdiv(p.K, BN);                  // WGRAD: tiles per expert
   const int nwg = gridDim.x;
@@ -153,7 +163,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       r.t = uni_tile(moe_gg_decode_tile(sh.row_off, sh.tile_off, p.G, L, BM));
       r.KT = KT_fwd;
       r.xoff = (int64_t)(r.t.row0 + r.t.tm * BM) * KROW;
-      r.woff = ((int64_t)r.t.g * N + r.t.tn * BN) * KROW;
+      r.woff = ((int64_t)r.t.g * N + r.t.tn * TILE_COLS) * KROW;
     }
     return r;
   };
@@ -180,10 +190,10 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     if (round >= sh.n_my) return;  // past the last tile: keep re-loading the last tile (never read)
     const TileRef tr = tile_ref(round);
     const MoeGgTile& t = tr.t;
-    const int m0 = t.tm * BM, n0 = t.tn * BN;
+    const int m0 = t.tm * BM, n0 = t.tn * TILE_COLS;
     c.KT = tr.KT;
     c.x_last = min(t.rows - m0, BM) - 1;
-    c.w_last = min(NCOLS - n0, BN) - 1;
+    c.w_last = min(NCOLS - n0, TILE_COLS) - 1;  // SWIGLU: last valid output column of the tile
     c.xg = uni_ptr(xp + tr.xoff);
     c.wg = uni_ptr(wp + tr.woff);
     if (BLOCK) {
@@ -206,7 +216,10 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     dma16(c.xg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + b * 1024);
   };
   auto dma_w = [&](int b) {
-    const uint32_t off = (uint32_t)min(b * 8 + d_r, c.w_last) * KROW + d_c16;
+    uint32_t row;
+    if (SWIGLU) row = (uint32_t)min((b >> 3) * 32 + (b & 3) * 8 + d_r, c.w_last) + (((b >> 2) & 1) ? (uint32_t)NCOLS : 0u);
+    else row = (uint32_t)min(b * 8 + d_r, c.w_last);
+    const uint32_t off = row * KROW + d_c16;
     dma16(c.wg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + X_BYTES + b * 1024);
   };
   // Block scales of the cursor slab: wave gw of group 0 fetches the activation scales of rows
@@ -255,9 +268,9 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const TileRef tr = tile_ref(r);
     const MoeGgTile& t = tr.t;
     const int KT = tr.KT;
-    const int m0 = t.tm * BM, n0 = t.tn * BN;
+    const int m0 = t.tm * BM, n0 = t.tn * TILE_COLS;
     const int rows_valid = min(t.rows - m0, BM);
-    const int cols_valid = min(NCOLS - n0, BN);
+    const int cols_valid = min(NCOLS - n0, TILE_COLS);
     // Activation fragments of this wave that hold at least one valid row (fragments are dealt
     // alternately to wm = 0 / 1, so a short tile shortens every wave's C phase alike).
     const int nfm = min(FM, max(0, ((rows_valid + 15) / 16 - wm + WM - 1) / WM));
@@ -364,7 +377,40 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       // Row-wise fp8 scales (groupgemm.py:374-384): y *= x_scale[m] * w_scale[g * N + n].
       const float* xrow_scale = OP == OP_FP8_ROW ? p.x_scale + t.row0 + m0 : nullptr;
       const float* wcol_scale = OP == OP_FP8_ROW ? p.w_scale + (int64_t)t.g * N + n0 : nullptr;
-      if (p.vec_store && cols_valid == BN && p.ldy < (1 << 24)) {
+      if (SWIGLU) {
+        // acc[j][i], j = 0, 1: gate of output columns 32 wn + 16 j + 4 eq .. + 3; acc[j + 2][i]: up of the same columns.
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          const int m = (i * WM + wm) * 16 + er;
+          if (m < rows_valid) {
+            bf16_t* yrow = yg + (int64_t)m * p.ldy;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const int n = wn * 32 + j * 16 + eq * 4;
+              const f32x4_t gv = acc[j][i], uv = acc[j + 2][i];
+              const uint32_t g01 = pack_bf16x2(gv[0], gv[1]), g23 = pack_bf16x2(gv[2], gv[3]);
+              const uint32_t u01 = pack_bf16x2(uv[0], uv[1]), u23 = pack_bf16x2(uv[2], uv[3]);
+              const float g[4] = {__builtin_bit_cast(float, g01 << 16), __builtin_bit_cast(float, g01 & 0xFFFF0000u),
+                                  __builtin_bit_cast(float, g23 << 16), __builtin_bit_cast(float, g23 & 0xFFFF0000u)};
+              const float u[4] = {__builtin_bit_cast(float, u01 << 16), __builtin_bit_cast(float, u01 & 0xFFFF0000u),
+                                  __builtin_bit_cast(float, u23 << 16), __builtin_bit_cast(float, u23 & 0xFFFF0000u)};
+              float o[4];
+#pragma unroll
+              for (int rr = 0; rr < 4; ++rr) o[rr] = g[rr] / (1.f + __expf(-g[rr])) * u[rr];
+              if (p.vec_store && n + 3 < cols_valid) {
+                u32x2_t q;
+                q[0] = pack_bf16x2(o[0], o[1]);
+                q[1] = pack_bf16x2(o[2], o[3]);
+                *(u32x2_t*)(yrow + n) = q;
+              } else {
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr)
+                  if (n + rr < cols_valid) yrow[n + rr] = (bf16_t)o[rr];
+              }
+            }
+          }
+        }
+      } else if (p.vec_store && cols_valid == BN && p.ldy < (1 << 24)) {
         const uint32_t voff = (uint32_t)er * (uint32_t)p.ldy + (uint32_t)(wn * FN * 16 + eq * 4);
         f32x4_t bs[FN];
         if (OP == OP_FP8_ROW) {
@@ -428,6 +474,7 @@ DEVINL void pingpong_body(const GgParams& p) {
 
   // WGRAD: tile_off counts the 64-column blocks of the padded operands (at least one per expert).
   if (OP == OP_BF16_WGRAD) build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
+  else if (OP == OP_BF16_SWIGLU) build_group_tables(p.m_sizes, p.G, p.M, BM, moe_gg_cdiv(p.N / 2, BN / 2), row_off, tile_off);
   else build_group_tables(p.m_sizes, p.G, p.M, BM, moe_gg_cdiv(p.N, BN), row_off, tile_off, p.skip_rows);
   const int total = OP == OP_BF16_WGRAD ? p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN) : uni(tile_off[p.G]);
   const int nwg = gridDim.x;
@@ -444,6 +491,7 @@ DEVINL void pingpong_body(const GgParams& p) {
 
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_body<OP_BF16>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise(GgParams p) { pingpong_body<OP_FP8_ROW>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpong_body<OP_FP8_BLOCK>(p); }
 
@@ -456,6 +504,11 @@ hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t st
 
 hipError_t gg_bf16_pingpong_wgrad_launch(const GgParams& p, int num_wg, hipStream_t stream) {
   hipLaunchKernelGGL(gg_bf16_pingpong_wgrad, dim3(num_wg), dim3(NT), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream) {
+  hipLaunchKernelGGL(gg_bf16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -83,6 +83,8 @@ hipError_t transpose_padded_launch(const void* src, void* dst, const int32_t* m_
 // dst [M, C] <- the expert's own C columns (at g * col_block) of src [M, src_pitch]. C % 4 == 0, 8-byte aligned rows.
 hipError_t compact_block_launch(const void* src, void* dst, const int32_t* m_sizes, int G, int M, int C, int64_t src_pitch,
                                 int col_block, hipStream_t stream);
+// y [M, n] = silu(x w_gate^T) * (x w_up^T) with w [G * 2n, K] (gate rows first); p.N = 2n, p.ldy >= n, p.col_block unused.
+hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream);
 hipError_t gg_bf16_pingpong_wgrad_launch(const GgParams& p, int num_wg, hipStream_t stream);
 // dW = dY^T X per expert on the transposed, padded operands; p.x = dY^T [N, ldm], p.w = X^T [K, ldm], p.M = ldm,
 // p.skip_rows = number of gradient rows (bound for m_sizes), p.y = dW [G * N, K] with p.ldy = K. block in {256, 128}.

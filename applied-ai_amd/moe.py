@@ -9,6 +9,7 @@ over m_sizes, so no padding rows are computed:
     xs  = hidden_states[perm // k]                                        moe_gg_gather_rows
     h1  = grouped_gemm(xs, w1, m_sizes)            [R, 2n]                moe_gg_grouped_gemm_bf16
     h2  = silu(h1[:, :n]) * h1[:, n:]              [R, n]                 moe_gg_silu_and_mul
+          (both in one kernel without h1 when there are many rows: moe_gg_grouped_gemm_swiglu_bf16, same bits)
     y2  = grouped_gemm(h2, w2, m_sizes)            [R, d]                 moe_gg_grouped_gemm_bf16
     out[t] = sum_j topk_weights[t, j] * y2[inv[t * k + j]]                moe_gg_invert_perm, moe_gg_combine_topk
 
@@ -16,8 +17,12 @@ Everything runs in the HIP kernels behind include/moe_gg.h; torch only provides 
 import torch
 
 from . import _lib
-from .ops import _require_cuda, _stream_ptr, grouped_gemm, matmul_split_k_grouped
+from .ops import _require_cuda, _stream_ptr, grouped_gemm, grouped_gemm_swiglu, matmul_split_k_grouped
 from .routing import gather_sorted, route_group
+
+# fused_moe folds SiLU-and-mul into the first GEMM from this many expert-sorted rows on (the fused kernel is the
+# 256 x 256 ping-pong kernel; below, the small-M kernels of grouped_gemm are faster than it).
+FUSED_SWIGLU_MIN_ROWS = 1024
 
 
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
@@ -85,8 +90,10 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, t
 
     perm, m_sizes, offsets = route_group(ids, E)
     xs = gather_sorted(hidden_states, perm, k)
-    h1 = grouped_gemm(xs, w1.view(E * two_n, K), m_sizes)
-    h2 = silu_and_mul(h1)
+    if xs.shape[0] >= FUSED_SWIGLU_MIN_ROWS and K % 64 == 0 and two_n % 8 == 0 and two_n * K < 2 ** 31:
+        h2 = grouped_gemm_swiglu(xs, w1.view(E * two_n, K), m_sizes)
+    else:
+        h2 = silu_and_mul(grouped_gemm(xs, w1.view(E * two_n, K), m_sizes))
     y2 = grouped_gemm(h2, w2.view(E * w2.shape[1], w2.shape[2]), m_sizes)
     return combine_topk(y2, perm, offsets, tw, out=hidden_states if inplace else None)
 

@@ -77,6 +77,37 @@ def grouped_gemm_forward(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor
     return _grouped_gemm_bf16(x, w, m_sizes, OUT_BLOCK)
 
 
+def grouped_gemm_swiglu(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor) -> torch.Tensor:
+    """silu(x @ w_gate.T) * (x @ w_up.T) per expert in one kernel: x [M, K] expert-sorted, w [G*2n, K] with the
+    reference's w1 layout (per expert n gate rows, then n up rows), result [M, n] bf16.
+
+    The first GEMM of fused_moe with ops.silu_and_mul folded into its epilogue
+    (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:271-284); bit-identical to
+    silu_and_mul(grouped_gemm(x, w, m_sizes))."""
+    assert x.is_contiguous()
+    assert w.is_contiguous()
+    assert m_sizes.is_contiguous()
+    if x.dim() != 2 or w.dim() != 2 or m_sizes.dim() != 1:
+        raise ValueError("x must be [M, K], w must be [G*2n, K], m_sizes must be [G]")
+    G = m_sizes.shape[0]
+    M, K = x.shape
+    if G == 0 or w.shape[0] % (2 * G) != 0:
+        raise ValueError(f"w.shape[0]={w.shape[0]} is not a multiple of 2*G={2 * G}")
+    n = w.shape[0] // (2 * G)
+    assert K == w.shape[1], f"K mismatch: x has {K}, w has {w.shape[1]}"
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ValueError("grouped_gemm_swiglu takes bf16 x and w")
+    if m_sizes.dtype != torch.int32:
+        raise ValueError("m_sizes must be int32")
+    dev = _require_cuda(x, w, m_sizes)
+    y = torch.empty((M, n), device=dev, dtype=torch.bfloat16)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_grouped_gemm_swiglu_bf16(
+            x.data_ptr(), w.data_ptr(), y.data_ptr(), m_sizes.data_ptr(), G, M, n, K, n, _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_grouped_gemm_swiglu_bf16")
+    return y
+
+
 def grouped_gemm_backward(grad_output: torch.Tensor, x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor):
     """Backward pass of the bf16 grouped GEMM: returns (grad_x [M, K], grad_w [G*N, K]).
 

@@ -162,6 +162,19 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
                                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * First GEMM of a gated MoE layer with the activation fused into its epilogue. Replaces the pair
+ * invoke_fused_moe_kernel(hidden_states, w1, ...) + ops.silu_and_mul
+ * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:271-284):
+ *   y[off_g + i, c] = silu(x[off_g + i] . w[g*2n + c]) * (x[off_g + i] . w[g*2n + n + c]),   c < n
+ * x device [M, K] bf16 expert-sorted; w device [G*2n, K] bf16 (per expert n gate rows, then n up rows: the
+ * reference's w1 layout); y device out [M, n] bf16 with leading dimension ldy. Both products are rounded to bf16
+ * before the activation, so the result equals moe_gg_grouped_gemm_bf16 followed by moe_gg_silu_and_mul bit for
+ * bit, without the [M, 2n] intermediate. Requires K % 64 == 0, n % 4 == 0, 2n*K < 2^31, 16-byte aligned x and w.
+ */
+int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M,
+                                    int n, int K, int64_t ldy, void* stream);
+
+/*
  * Glue between the two grouped GEMMs of a whole MoE layer, as in the reference's fused_moe
  * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:222-296; oracle torch_moe,
  * kernels/triton/inference/col_major_moe_gemm/test_moe_gemm.py:16-30). All data bf16.

@@ -76,6 +76,10 @@ def test_argument_errors_of_the_other_entry_points(lib):
     assert lib.moe_gg_combine_topk(None, None, None, 1, None, 4, 2, 8, 8, None) == -1        # fp16 weights unsupported
     assert lib.moe_gg_combine_topk(None, None, None, 2, None, 4, 0, 8, 8, None) == -1        # k <= 0
     assert lib.moe_gg_fp8_groupwise_quant(None, 1, None, None, 128, None) == -1              # fp16 input unsupported
+    sw = lib.moe_gg_grouped_gemm_swiglu_bf16
+    assert sw(None, None, None, None, 2, 8, 64, 64, 32, None) == -2      # ldy < n
+    assert sw(None, None, None, None, 2, 8, 64, 64, 64, None) == -1      # null pointers
+    assert sw(None, None, None, None, 2, 0, 64, 64, 64, None) == 0       # no rows
     bw = lib.moe_gg_grouped_gemm_backward_bf16
     ws = lib.moe_gg_grouped_gemm_backward_workspace
     assert bw(None, 128, 7, None, None, None, 2, 8, 64, 64, None, None, None, 0, None) == -1     # bad layout

@@ -113,6 +113,28 @@ def test_fused_moe_reference_test_shape():
     assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 1e-2
 
 
+def test_fused_moe_prefill_rows_take_the_fused_activation_path():
+    """768 tokens, top-2 -> 1536 expert-sorted rows: the first GEMM runs with SiLU-and-mul in its epilogue.
+    Same oracle, same bar; and the result equals the layer built from the separate kernels bit for bit."""
+    import applied_ai_amd as A
+    from applied_ai_amd import moe
+
+    assert 768 * 2 >= moe.FUSED_SWIGLU_MIN_ROWS
+    a, w1, w2, tw, ids = make(768, 192, 256, 8, 2, seed=21)
+    args = (a.cuda(), w1.cuda(), w2.cuda(), tw.cuda(), ids.cuda())
+    y = A.fused_moe(*args)
+    ref = O.fused_moe(a.float().numpy(), w1.float().numpy(), w2.float().numpy(), tw.numpy(), ids.numpy())
+    ok, worst = close(to_np(y), ref)
+    assert ok, worst
+    saved = moe.FUSED_SWIGLU_MIN_ROWS
+    try:
+        moe.FUSED_SWIGLU_MIN_ROWS = 1 << 40
+        y2 = A.fused_moe(*args)
+    finally:
+        moe.FUSED_SWIGLU_MIN_ROWS = saved
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+
+
 def test_fused_moe_rejects_bad_arguments():
     import applied_ai_amd as A
 
@@ -123,3 +145,42 @@ def test_fused_moe_rejects_bad_arguments():
         A.fused_moe(a.cuda().half(), w1.cuda(), w2.cuda(), tw.cuda(), ids.cuda())
     with pytest.raises(RuntimeError):
         A.fused_moe(a, w1, w2, tw, ids)
+
+
+@pytest.mark.parametrize("sizes,n,K", [
+    ([300, 0, 41, 700], 256, 128),        # ragged, an empty expert
+    ([256, 256], 128, 64),                # one K step
+    ([100, 37], 200, 192),                # n not a multiple of the 128-column tile
+    ([513, 64, 1], 1032, 256),            # several column tiles and a partial one
+])
+def test_swiglu_gemm_equals_gemm_then_silu_and_mul(sizes, n, K):
+    """The fused kernel rounds both products to bf16 before the activation: bit-identical to the two-kernel path,
+    and within the GEMM bar of the double-precision oracle."""
+    import applied_ai_amd as A
+
+    G, M = len(sizes), sum(sizes) + 5
+    gen = torch.Generator().manual_seed(77)
+    x = bf(torch.randn(M, K, generator=gen))
+    w = bf(torch.randn(G * 2 * n, K, generator=gen) / 8)
+    m = torch.tensor(sizes, dtype=torch.int32)
+    fused = A.grouped_gemm_swiglu(x.cuda(), w.cuda(), m.cuda())
+    two = A.silu_and_mul(A.grouped_gemm(x.cuda(), w.cuda(), m.cuda()))
+    R = sum(sizes)
+    assert fused.shape == (M, n)
+    assert torch.equal(fused[:R].view(torch.int16), two[:R].view(torch.int16))
+    h1 = O.round_bf16(O.grouped_gemm(x.float().numpy(), w.float().numpy(), sizes, fill=0.0))
+    ref = O.silu_and_mul(h1)[:R]
+    ok, worst = close(to_np(fused)[:R], ref)
+    assert ok, worst
+
+
+def test_swiglu_errors(lib=None):
+    import applied_ai_amd as A
+
+    x = torch.zeros(8, 96, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(2 * 2 * 64, 96, dtype=torch.bfloat16, device="cuda")
+    m = torch.tensor([4, 4], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError):      # K % 64 != 0: unsupported
+        A.grouped_gemm_swiglu(x, w, m)
+    with pytest.raises(AssertionError):    # K mismatch
+        A.grouped_gemm_swiglu(x[:, :64].contiguous(), w, m)
