@@ -60,6 +60,10 @@ SIGNATURES = {
         _c_int,
         [_i32_p, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _i32_p, _c_int],
     ),
+    "moe_gg_host_enumerate_tiles_two_lists": (
+        _c_int,
+        [_i32_p, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _i32_p, _c_int],
+    ),
 }
 
 _lib = None

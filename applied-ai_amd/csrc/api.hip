@@ -420,4 +420,57 @@ int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, i
   return written;
 }
 
+int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
+                                          int block_n, int num_workgroups, int xcds, int32_t* out,
+                                          int max_tiles) {
+  if (!m_sizes_host || !out || G <= 0 || G > MOE_GG_MAX_GROUPS_ABI || block_m <= 0 || block_n <= 0 ||
+      num_workgroups <= 0 || xcds <= 0 || num_workgroups % xcds != 0 || M < 0 || N <= 0)
+    return MOE_GG_EINVAL;
+  static thread_local int32_t row_off[MOE_GG_MAX_GROUPS_ABI + 1], long_off[MOE_GG_MAX_GROUPS_ABI + 1],
+      low_off[MOE_GG_MAX_GROUPS_ABI + 1];
+  const int ntn = moe_gg_cdiv(N, block_n);
+  int64_t r = 0;
+  int nl = 0, ns = 0;
+  for (int g = 0; g < G; ++g) {
+    row_off[g] = (int32_t)r; long_off[g] = nl; low_off[g] = ns;
+    const int m = moe_gg_clamp_rows(m_sizes_host[g], r, M);
+    r += m;
+    nl += moe_gg_long_row_tiles(m, block_m) * ntn;
+    ns += moe_gg_low_row_tiles(m, block_m) * ntn;
+  }
+  row_off[G] = (int32_t)r; long_off[G] = nl; low_off[G] = ns;
+  const int total = nl + ns;
+  int written = 0;
+  for (int wg = 0; wg < num_workgroups; ++wg) {
+    int n_long = 0, n_low = 0;
+    while (n_long * num_workgroups < nl && moe_gg_tile_of(wg, num_workgroups, xcds, n_long) < nl) ++n_long;
+    while ((n_long + n_low) * num_workgroups < total && moe_gg_tile_of(wg, num_workgroups, xcds, n_long + n_low) < total) ++n_low;
+    const int n_my = n_long + n_low, phase = moe_gg_low_phase(wg, xcds);
+    for (int seq = 0; seq < n_my; ++seq) {
+      const int lb = moe_gg_low_before(seq, n_my, n_low, phase);
+      const bool low = moe_gg_low_before(seq + 1, n_my, n_low, phase) > lb;
+      const int L = moe_gg_tile_of(wg, num_workgroups, xcds, low ? n_long + lb : seq - lb);
+      if (written >= max_tiles) return written;
+      int g, tm, tn;
+      if (!low) {
+        if (L >= nl) return MOE_GG_EINVAL;  // cannot happen: a long position maps to a long tile id
+        g = moe_gg_find_group(long_off, G, L);
+        const int idx = L - long_off[g];
+        const int nf = moe_gg_long_row_tiles(row_off[g + 1] - row_off[g], block_m);
+        tn = idx / nf; tm = idx - tn * nf;
+      } else {
+        const int Lp = L - nl;
+        if (Lp < 0 || Lp >= ns) return MOE_GG_EINVAL;
+        g = moe_gg_find_group(low_off, G, Lp);
+        tn = Lp - low_off[g];
+        tm = (row_off[g + 1] - row_off[g]) / block_m;
+      }
+      int32_t* o = out + (size_t)written * 5;
+      o[0] = wg; o[1] = g; o[2] = tm; o[3] = tn; o[4] = row_off[g];
+      ++written;
+    }
+  }
+  return written;
+}
+
 }  // extern "C"

@@ -106,9 +106,12 @@ DEVINL MoeGgTile uni_tile(MoeGgTile t) {
 
 struct Shared {
   const int32_t* row_off;
-  const int32_t* tile_off;
+  const int32_t* tile_off;   // forward: prefix of the long tiles; WGRAD: prefix of the padded 64-column blocks
+  const int32_t* part_off;   // forward: prefix of the low tiles (one row of tiles per group at most)
   char* lds;
-  int n_my;
+  int n_my;      // tiles of this workgroup
+  int n_low_my;  // of which low tiles (forward only)
+  int phase;     // 0 .. 255: where in the workgroup's sequence its low tiles sit (the same for all workgroups of an XCD)
 };
 
 // Slab-load cursor of one wave: which slab (tile round, K step) its next load instructions fetch.
@@ -147,9 +150,20 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   // Tile of a round. Forward: rows of x / rows of w[g]. WGRAD: rows of dY^T (n) / rows of X^T (k), both at the
   // column offset of the expert's padded block; t.row0 = first row of the expert's block of dW, t.rows = N.
   struct TileRef { MoeGgTile t; int KT; int64_t xoff, woff; };
-  auto tile_ref = [&](int round) {
+  // The workgroup's own sequence: its long tiles in round order with its low tiles spread evenly between
+  // them. low_before(i) = number of low tiles among the first i sequence positions; low tile j sits at
+  // position floor((j + phase / 256) * n_my / n_low_my). The phase differs between XCDs, so the low tiles
+  // (which stream a whole weight tile from memory for a few rows) are spread over the launch instead of
+  // running all at once, while the workgroups of one XCD still take theirs together and stay in step.
+  // (The block-scaled kernel has no registers left for this arithmetic: it keeps all tiles in the first list.)
+  auto low_before = [&](int i) { return BLOCK ? 0 : moe_gg_low_before(i, sh.n_my, sh.n_low_my, sh.phase); };
+  auto tile_ref = [&](int seq) {
     TileRef r;
-    const int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, round);
+    const int lb = uni(low_before(seq));
+    const bool low = uni(low_before(seq + 1)) > lb;
+    // Tile ids: long tiles 0 .. n_long - 1, then the low tiles; ids are dealt round-robin, so this workgroup's
+    // low tiles are its last rounds.
+    const int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, low ? (sh.n_my - sh.n_low_my) + lb : seq - lb);
     if (WGRAD) {
       const int g = uni(L / wg_tpg);
       const int rem = L - g * wg_tpg;
@@ -160,7 +174,28 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       r.xoff = (int64_t)(r.t.tm * BM) * KROW + (int64_t)b0 * 128;
       r.woff = (int64_t)(r.t.tn * BN) * KROW + (int64_t)b0 * 128;
     } else {
-      r.t = uni_tile(moe_gg_decode_tile(sh.row_off, sh.tile_off, p.G, L, BM));
+      // Tile list: the long tiles of all groups (group, then column tile, then row tile), then the low tiles
+      // (group, column tile; see moe_gg_long_row_tiles), dealt to the workgroups round-robin:
+      // every workgroup gets the same number (+- 1) of long tiles, and the low tiles go on where the long
+      // ones stopped.
+      MoeGgTile t;
+      if (BLOCK || !low) {
+        t.g = moe_gg_find_group(sh.tile_off, p.G, L);
+        t.row0 = sh.row_off[t.g];
+        t.rows = sh.row_off[t.g + 1] - t.row0;
+        const int idx = L - sh.tile_off[t.g];
+        const int nf = BLOCK ? moe_gg_cdiv(t.rows, BM) : moe_gg_long_row_tiles(t.rows, BM);
+        t.tn = idx / nf;
+        t.tm = idx - t.tn * nf;
+      } else {
+        const int Lp = L - uni(sh.tile_off[p.G]);
+        t.g = moe_gg_find_group(sh.part_off, p.G, Lp);
+        t.row0 = sh.row_off[t.g];
+        t.rows = sh.row_off[t.g + 1] - t.row0;
+        t.tn = Lp - sh.part_off[t.g];
+        t.tm = t.rows / BM;
+      }
+      r.t = uni_tile(t);
       r.KT = KT_fwd;
       r.xoff = (int64_t)(r.t.row0 + r.t.tm * BM) * KROW;
       r.woff = ((int64_t)r.t.g * N + r.t.tn * TILE_COLS) * KROW;
@@ -471,19 +506,35 @@ DEVINL void pingpong_body(const GgParams& p) {
   __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + (OP == OP_FP8_BLOCK ? 2 * SCALE_BYTES : 0)];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t tile_off[MOE_GG_MAX_GROUPS + 1];
+  __shared__ int32_t part_off[MOE_GG_MAX_GROUPS + 1];
 
-  // WGRAD: tile_off counts the 64-column blocks of the padded operands (at least one per expert).
-  if (OP == OP_BF16_WGRAD) build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
-  else if (OP == OP_BF16_SWIGLU) build_group_tables(p.m_sizes, p.G, p.M, BM, moe_gg_cdiv(p.N / 2, BN / 2), row_off, tile_off);
-  else build_group_tables(p.m_sizes, p.G, p.M, BM, moe_gg_cdiv(p.N, BN), row_off, tile_off, p.skip_rows);
-  const int total = OP == OP_BF16_WGRAD ? p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN) : uni(tile_off[p.G]);
+  int total, total_low = 0;
+  if (OP == OP_BF16_WGRAD) {
+    // tile_off counts the 64-column blocks of the padded operands (at least one per expert).
+    build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
+    total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
+  } else {
+    const int ntn = OP == OP_BF16_SWIGLU ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
+    const int skip = p.skip_rows;
+    build_row_offsets(p.m_sizes, p.G, p.M, row_off);
+    if (OP == OP_FP8_BLOCK) {
+      build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_cdiv(rows, BM) * ntn : 0; });
+    } else {
+      build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
+      build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
+      total_low = uni(part_off[p.G]);
+    }
+    total = uni(tile_off[p.G]);
+  }
   const int nwg = gridDim.x;
-  // Tiles of this workgroup: rounds 0 .. n_my - 1 (tile ids grow with the round).
-  int n_my = 0;
-  while (n_my * nwg < total && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_my) < total) ++n_my;
-  if (n_my == 0) return;
+  // Tiles of this workgroup in each list: rounds 0 .. n - 1 (tile ids grow with the round).
+  int n_long = 0, n_low = 0;
+  while (n_long * nwg < total && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < total) ++n_long;
+  while ((n_long + n_low) * nwg < total + total_low && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < total + total_low)
+    ++n_low;
+  if (n_long + n_low == 0) return;
 
-  Shared sh{row_off, tile_off, lds, n_my};
+  Shared sh{row_off, tile_off, part_off, lds, n_long + n_low, n_low, moe_gg_low_phase(blockIdx.x, p.xcds)};
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
   if (grp == 0) run_group<0, OP>(p, sh);
   else run_group<1, OP>(p, sh);

@@ -15,13 +15,9 @@ DEVINL long long wave_incl_scan_i64(long long x) {
   return x;
 }
 
-// Must be called by every thread of the workgroup (it contains barriers).
-// row_off / tile_off: LDS arrays of G + 1 entries, G <= MOE_GG_MAX_GROUPS.
-// Groups with at most skip_rows rows keep their rows in row_off but get no tiles (another kernel
-// of the same call computes them). min_tiles: lower bound of every group's tile count (also of an empty group).
-DEVINL void build_group_tables(const int32_t* __restrict__ m_sizes, int G, int M, int BM, int n_tiles_n,
-                               int32_t* row_off, int32_t* tile_off, int skip_rows = 0, int min_tiles = 0) {
-  auto tiles_of = [&](int rows) { return max(min_tiles, rows > skip_rows ? moe_gg_cdiv(rows, BM) * n_tiles_n : 0); };
+// Must be called by every thread of the workgroup (it ends with a barrier).
+// row_off: LDS array of G + 1 entries, G <= MOE_GG_MAX_GROUPS: row_off[g] = min(sum of the clamped sizes before g, M).
+DEVINL void build_row_offsets(const int32_t* __restrict__ m_sizes, int G, int M, int32_t* row_off) {
   const int per = (G + 63) >> 6;
   if (wave_id() == 0) {
     const int g0 = lane_id() * per;
@@ -47,6 +43,13 @@ DEVINL void build_group_tables(const int32_t* __restrict__ m_sizes, int G, int M
     if (lane_id() == 63) row_off[G] = (int32_t)(run > M ? M : run);
   }
   __syncthreads();
+}
+
+// tile_off[g] = sum over the groups before g of tiles_of(rows of the group); G + 1 entries. Needs row_off
+// complete (build_row_offsets); every thread of the workgroup must call it (it ends with a barrier).
+template <class F>
+DEVINL void build_tile_prefix(const int32_t* row_off, int G, int32_t* tile_off, F tiles_of) {
+  const int per = (G + 63) >> 6;
   if (wave_id() == 0) {
     const int g0 = lane_id() * per;
     long long s = 0;
@@ -65,4 +68,14 @@ DEVINL void build_group_tables(const int32_t* __restrict__ m_sizes, int G, int M
     if (lane_id() == 63) tile_off[G] = (int32_t)run;
   }
   __syncthreads();
+}
+
+// Groups with at most skip_rows rows keep their rows in row_off but get no tiles (another kernel
+// of the same call computes them). min_tiles: lower bound of every group's tile count (also of an empty group).
+DEVINL void build_group_tables(const int32_t* __restrict__ m_sizes, int G, int M, int BM, int n_tiles_n,
+                               int32_t* row_off, int32_t* tile_off, int skip_rows = 0, int min_tiles = 0) {
+  build_row_offsets(m_sizes, G, M, row_off);
+  build_tile_prefix(row_off, G, tile_off, [&](int rows) {
+    return max(min_tiles, rows > skip_rows ? moe_gg_cdiv(rows, BM) * n_tiles_n : 0);
+  });
 }

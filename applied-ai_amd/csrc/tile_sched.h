@@ -86,3 +86,29 @@ MOE_GG_HD int moe_gg_tile_of(int wg, int nwg, int xcds, int round) {
   int per = nwg / xcds;
   return round * nwg + (wg % xcds) * per + wg / xcds;
 }
+
+// ---- Two-list order of the ping-pong kernel ---------------------------------------------------------
+// Row tiles of a group that go into the list of long tiles: all of them, except a last tile of fewer than
+// BM / 2 rows when the group has at least two full tiles before it. Such a low tile goes into the list of low
+// tiles. (A low tile streams its whole weight tile for a few rows; next to its full neighbours it finds their
+// weight slabs in the L2, away from them it reads them again, which only pays for tall groups, where the
+// better balance is worth more than one more pass over the group's weights.)
+MOE_GG_HD int moe_gg_long_row_tiles(int rows, int BM) {
+  const int full = rows / BM, rem = rows - full * BM;
+  return full + ((rem >= BM / 2 || (rem > 0 && full < 2)) ? 1 : 0);
+}
+MOE_GG_HD int moe_gg_low_row_tiles(int rows, int BM) { return moe_gg_cdiv(rows, BM) - moe_gg_long_row_tiles(rows, BM); }
+
+// A workgroup's own sequence of n_my tiles, n_low_my of them low: its long tiles in round order with its low
+// tiles spread evenly between them. Returns the number of low tiles among the first i sequence positions;
+// low tile j sits at position floor((j + phase / 256) * n_my / n_low_my), 0 <= phase < 256.
+MOE_GG_HD int moe_gg_low_before(int i, int n_my, int n_low_my, int phase) {
+  if (n_low_my == 0) return 0;
+  const int den = 256 * n_my;
+  const int num = i * n_low_my * 256 - phase * n_my;
+  const int c = num <= 0 ? 0 : (num + den - 1) / den;
+  return c < n_low_my ? c : n_low_my;
+}
+// Phase of a workgroup: the same for all workgroups of an XCD (they take their low tiles together and stay in
+// step), different between XCDs (the low tiles, which are memory-bound, are spread over the launch).
+MOE_GG_HD int moe_gg_low_phase(int wg, int xcds) { return ((wg % xcds) * 256 + 128) / xcds; }

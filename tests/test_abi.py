@@ -146,3 +146,50 @@ def test_scheduler_rejects_bad_arguments(lib):
     args = (ms.ctypes.data_as(I32P), 2, 3, 64, 16, 64)
     assert lib.moe_gg_host_enumerate_tiles(*args, 6, 4, out.ctypes.data_as(I32P), 8) == -1  # 6 % 4 != 0
     assert lib.moe_gg_host_enumerate_tiles(*args, 0, 1, out.ctypes.data_as(I32P), 8) == -1
+
+
+@pytest.mark.parametrize("m_sizes,N,nwg", [
+    ([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], 14336, 256),   # Mixtral prefill: 4 experts end in a low tile
+    ([25, 50, 25], 512, 8),                                          # short experts: nothing is split off
+    ([600, 0, 513, 255, 1, 2048 + 17], 1000, 16),
+    ([700] * 40, 2048, 256),
+    ([530], 256, 8),                                                 # fewer tiles than workgroups
+])
+def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
+    """The ping-pong kernels' order: every (group, row tile, column tile) exactly once; a low tile is the last row
+    tile of a group with at least two full tiles and fewer than 128 rows left; every workgroup gets the same
+    number of tiles (+- 1), its low tiles spread through its sequence."""
+    ms = np.ascontiguousarray(m_sizes, dtype=np.int32)
+    M = int(ms.sum())
+    cap = 1 << 16
+    out = np.zeros((cap, 5), dtype=np.int32)
+    n = lib.moe_gg_host_enumerate_tiles_two_lists(ms.ctypes.data_as(I32P), len(ms), M, N, 256, 256, nwg, 8,
+                                                  out.ctypes.data_as(I32P), cap)
+    assert n >= 0
+    tiles = out[:n].tolist()
+    off = O.offsets(m_sizes)
+    expect = {(g, tm, tn) for g, m in enumerate(m_sizes) for tm in range(-(-m // 256)) for tn in range(-(-N // 256))}
+    got = [tuple(t[1:4]) for t in tiles]
+    assert len(got) == len(set(got)) == len(expect) and set(got) == expect
+    assert all(t[4] == off[t[1]] for t in tiles)
+
+    def is_low(g, tm):
+        m = m_sizes[g]
+        return tm == m // 256 and m // 256 >= 2 and 0 < m % 256 < 128
+
+    per_wg = {}
+    for wg, g, tm, tn, _ in tiles:
+        per_wg.setdefault(wg, []).append(is_low(g, tm))
+    counts = [len(v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
+    assert max(counts) - min(counts) <= 1
+    lows = [sum(v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
+    assert max(lows) - min(lows) <= 1
+    if m_sizes[0] == 1012:
+        # 7 long tiles and at most one low tile per workgroup: the XCDs (wg % 8) take their low tile at 8 different
+        # positions of the sequence, the workgroups of one XCD at the same one
+        pos = {}
+        for wg, v in per_wg.items():
+            if any(v):
+                pos.setdefault(wg % 8, set()).add(v.index(True))
+        assert all(len(p) == 1 for p in pos.values())
+        assert len(pos) == 7 and len({next(iter(p)) for p in pos.values()}) == 7   # 224 low tiles: 7 XCDs of 32
