@@ -30,11 +30,12 @@
 //
 // Which stage regions are free when decides who loads what:
 //   X(s) is read in phases 2s and 2s+1, W0(s) only in 2s (group 0), W1(s) only in 2s+1 (group 1).
-//   group 0 in L(s)  [phase 2s]   issues X(s+1) and W1(s+1) -> stage (s+1)&1, free since phase 2s-1;
-//   group 1 in L(s)  [phase 2s+1] issues W0(s+2)            -> stage s&1, free since phase 2s.
-// Group 0 waits for its loads at the end of C(s); group 1 waits for W0(s+1) at the end of L(s), with
-// the W0(s+2) instructions it has just issued still in flight. The slab sequence runs straight
-// through tile boundaries, so the next tile's first slabs are in flight during the epilogue.
+//   group 0 in L(s)  [phase 2s]   issues X(s+1)  -> stage (s+1)&1, free since phase 2s-1 (32 KB);
+//   group 1 in L(s)  [phase 2s+1] issues W1(s+1) -> stage (s+1)&1, free since phase 2s-1,
+//                                    and W0(s+2) -> stage s&1, free since phase 2s (32 KB together).
+// Both load phases so put the same 32 KB through the CU's vector-memory path. Each group waits for its own
+// loads at the end of the compute phase that follows. The slab sequence runs straight through tile
+// boundaries, so the next tile's first slabs are in flight during the epilogue.
 // Block scales of step s+1 (256 activation scales, the tile's two weight-block scales) travel with
 // group 0's loads into a small per-stage LDS area.
 #include <type_traits>
@@ -250,13 +251,19 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const uint32_t off = (uint32_t)min(b * 8 + d_r, c.x_last) * KROW + d_c16;
     dma16(c.xg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + b * 1024);
   };
-  auto dma_w = [&](int b) {
+  // Weight rows: of the cursor slab, or (prev) of the slab before it, whose state group 1 keeps in wp_*.
+  const char* wp_wg = nullptr;
+  int wp_last = 0, wp_kt = 0, wp_step = 0;
+  auto dma_w = [&](int b, bool prev) {
+    const int w_last = prev ? wp_last : c.w_last;
     uint32_t row;
-    if (SWIGLU) row = (uint32_t)min((b >> 3) * 32 + (b & 3) * 8 + d_r, c.w_last) + (((b >> 2) & 1) ? (uint32_t)NCOLS : 0u);
-    else row = (uint32_t)min(b * 8 + d_r, c.w_last);
+    if (SWIGLU) row = (uint32_t)min((b >> 3) * 32 + (b & 3) * 8 + d_r, w_last) + (((b >> 2) & 1) ? (uint32_t)NCOLS : 0u);
+    else row = (uint32_t)min(b * 8 + d_r, w_last);
     const uint32_t off = row * KROW + d_c16;
-    dma16(c.wg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + X_BYTES + b * 1024);
+    dma16((prev ? wp_wg : c.wg) + (prev ? wp_kt : c.kt) * 128, off,
+          lds_base + ((prev ? wp_step : c.step) & 1) * STAGE + X_BYTES + b * 1024);
   };
+  auto keep_prev = [&]() { wp_wg = c.wg; wp_last = c.w_last; wp_kt = c.kt; wp_step = c.step; };
   // Block scales of the cursor slab: wave gw of group 0 fetches the activation scales of rows
   // 64 gw .. 64 gw + 63 (one per lane) and a private copy of the two weight-block scales (lanes 0-31 the
   // first column block, lanes 32-63 the second).
@@ -268,33 +275,46 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const uint32_t off = lane < 32 ? 0u : (uint32_t)c.ws_second;
     dma4(c.wsg + c.kt * 4, off, lds_scale + (c.step & 1) * SCALE_BYTES + 1024 + gw * 256);
   };
-  // Load instruction idx of this wave for the cursor slab; the last one advances the cursor.
-  // Group 0: 8 activation blocks (idx 0-7), 4 blocks of W1 (idx 8-11), block mode: the scales (12, 13).
-  // Group 1: 4 blocks of W0.
-  constexpr int NDMA = GRP == 0 ? (BLOCK ? 14 : 12) : 4;
+  // Load instruction idx of this wave in a load phase; the last one advances the cursor. Both groups issue
+  // 8 slab instructions per wave and phase:
+  // Group 0 (cursor = slab s + 1): 8 activation blocks (idx 0-7); block mode: the scales (8, 9).
+  // Group 1 (cursor = slab s + 2): 4 blocks of W1 of the slab before the cursor (idx 0-3), 4 blocks of W0 of the
+  // cursor slab (idx 4-7).
+  constexpr int NDMA = GRP == 0 ? (BLOCK ? 10 : 8) : 8;
   auto dma_one = [&](int idx) {
     if (GRP == 0) {
       if (idx < 8) dma_x(idx * 4 + gw);
-      else if (idx < 12) dma_w(16 + (idx - 8) * 4 + gw);
-      else if (idx == 12) dma_xscale();
+      else if (idx == 8) dma_xscale();
       else dma_wscale();
     } else {
-      dma_w(idx * 4 + gw);
+      if (idx < 4) dma_w(16 + idx * 4 + gw, true);
+      else dma_w((idx - 4) * 4 + gw, false);
     }
-    if (idx == NDMA - 1) cursor_next();
+    if (idx == NDMA - 1) {
+      if (GRP == 1) keep_prev();
+      cursor_next();
+    }
   };
 
-  // Prologue: slab 0 of the first tile (every wave its share), then the stagger.
+  // Prologue: slab 0 of the first tile (group 0 the activations and scales, group 1 all weight rows), then the
+  // stagger: group 1 runs one phase behind group 0 and sends W0(1) now; W1(1) and W0(2) follow in its L(0).
   c.kt = 0; c.step = 0;
   cursor_tile(0);
+  if (GRP == 0) {
 #pragma unroll
-  for (int i = 0; i < NDMA; ++i) dma_one(i);
+    for (int i = 0; i < NDMA; ++i) dma_one(i);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_w(i * 4 + gw, false);
+    cursor_next();
+  }
   wait_vm<0>();
   __syncthreads();
   if (GRP == 1) {
-    // group 1 runs one phase behind group 0: W0(1) goes out now, W0(2) in L(0), ...
 #pragma unroll
-    for (int i = 0; i < NDMA; ++i) dma_one(i);
+    for (int i = 0; i < 4; ++i) dma_w(i * 4 + gw, false);
+    keep_prev();
+    cursor_next();
     __syncthreads();
   }
 
@@ -353,7 +373,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         }
         __builtin_amdgcn_sched_barrier(0);
         wait_lgkm0();  // all of slab `step` is in this wave's registers
-        if (GRP == 1) wait_vm<NDMA>();  // W0(step + 1) has landed; W0(step + 2) may still be in flight
+        if (GRP == 1) wait_vm<NDMA>();  // first step: W0(1) of the prologue has landed; later nothing older is left
         __syncthreads();
         // ---------------- C phase: MFMAs only ----------------
         __builtin_amdgcn_s_setprio(1);
@@ -397,7 +417,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         }
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
-        if (GRP == 0) wait_vm<0>();  // X(step + 1), W1(step + 1): issued at the start of this step
+        wait_vm<0>();  // group 0: X(step + 1); group 1: W1(step + 1), W0(step + 2); issued in this step's load phase
         __syncthreads();
       }
 
