@@ -48,6 +48,9 @@ bool use_streaming_kernel(int64_t M, int G, int64_t ntn256, int num_wg) {
 
 }  // namespace
 
+// The ping-pong kernels form slab offsets with 24-bit multiplies: an operand row must be shorter than 16 MB.
+constexpr int64_t PINGPONG_MAX_ROW_BYTES = 1 << 24;
+
 extern "C" {
 
 int moe_gg_abi_version(void) { return MOE_GG_ABI_VERSION; }
@@ -122,12 +125,14 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
     // to occupy the CUs, also for experts of 16 .. 128 rows (short tiles skip most of their work and
     // the kernel then streams weights at 5 TB/s); smaller tiles only pay for small problems.
     const int64_t t256 = (M / 256 + (G + 1) / 2) * ntn256;
-    if (t256 * 4 >= (int64_t)num_wg * 3) variant = MOE_GG_GG_PINGPONG_256;
+    if (t256 * 4 >= (int64_t)num_wg * 3 && K < PINGPONG_MAX_ROW_BYTES / 2) variant = MOE_GG_GG_PINGPONG_256;
     else if (t256 * 4 >= num_wg) variant = MOE_GG_GG_TILED_128;
     else variant = MOE_GG_GG_TILED_64;
   }
   switch (variant) {
-    case MOE_GG_GG_PINGPONG_256: return (int)gg_bf16_pingpong_launch(p, num_wg, s);
+    case MOE_GG_GG_PINGPONG_256:
+      if (K >= PINGPONG_MAX_ROW_BYTES / 2) return MOE_GG_EUNSUPPORTED;
+      return (int)gg_bf16_pingpong_launch(p, num_wg, s);
     case MOE_GG_GG_TILED_256: return (int)gg_bf16_tiled_launch(p, 256, num_wg, s);
     case MOE_GG_GG_TILED_128: return (int)gg_bf16_tiled_launch(p, 128, num_wg, s);
     case MOE_GG_GG_TILED_64: return (int)gg_bf16_tiled_launch(p, 64, num_wg, s);
@@ -149,6 +154,7 @@ int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* 
   if (K == 0) return MOE_GG_ESHAPE;
   if (G > MOE_GG_MAX_GROUPS_ABI) return MOE_GG_EUNSUPPORTED;
   if (K % 128 != 0 || (scale_mode == MOE_GG_SCALE_BLOCK128 && N % 128 != 0)) return MOE_GG_EUNSUPPORTED;
+  if (K >= PINGPONG_MAX_ROW_BYTES) return MOE_GG_EUNSUPPORTED;
   if (!aligned(x, 16) || !aligned(w, 16) || !aligned(y, 2) || !aligned(x_scale, 4) || !aligned(w_scale, 4) ||
       !aligned(m_sizes, 4))
     return MOE_GG_EALIGN;
@@ -257,7 +263,9 @@ int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const
   if (G == 0 || M == 0 || n == 0) return MOE_GG_OK;
   if (!x || !w || !y || !m_sizes) return MOE_GG_EINVAL;
   if (G > MOE_GG_MAX_GROUPS_ABI || M > INT32_MAX || ldy > INT32_MAX) return MOE_GG_EUNSUPPORTED;
-  if (K == 0 || K % 64 != 0 || n % 4 != 0 || (int64_t)2 * n * K >= INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (K == 0 || K % 64 != 0 || n % 4 != 0 || (int64_t)2 * n * K >= INT32_MAX || K >= PINGPONG_MAX_ROW_BYTES / 2 ||
+      2 * (int64_t)n >= PINGPONG_MAX_ROW_BYTES)
+    return MOE_GG_EUNSUPPORTED;
   if (!aligned(x, 16) || !aligned(w, 16) || !aligned(y, 2) || !aligned(m_sizes, 4)) return MOE_GG_EALIGN;
   const DeviceInfo* di = nullptr;
   int rc = current_device_info(&di);

@@ -105,6 +105,15 @@ DEVINL MoeGgTile uni_tile(MoeGgTile t) {
   return t;
 }
 
+// a * b + c for a, b < 2^24 (row index and row pitch in bytes): one full-rate VALU instruction where the 32-bit
+// multiply takes a quarter-rate one. The partner wave's MFMAs share the VALU issue port with these.
+// (Written as an instruction: from the plain expression the compiler may still pick the 64-bit multiply-add.)
+DEVINL uint32_t mad24(uint32_t a, uint32_t b, uint32_t c) {
+  uint32_t d;
+  asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(b), "v"(c));
+  return d;
+}
+
 struct Shared {
   const int32_t* row_off;
   const int32_t* tile_off;   // forward: prefix of the long tiles; WGRAD: prefix of the padded 64-column blocks
@@ -248,7 +257,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   // Block b (8 rows) of the cursor slab's activation / weight rows.
   auto dma_x = [&](int b) {
     if (b * 8 > c.x_last) return;  // block entirely below the tile's last row: its fragments are never used
-    const uint32_t off = (uint32_t)min(b * 8 + d_r, c.x_last) * KROW + d_c16;
+    const uint32_t off = mad24((uint32_t)min(b * 8 + d_r, c.x_last), KROW, d_c16);
     dma16(c.xg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + b * 1024);
   };
   // Weight rows: of the cursor slab, or (prev) of the slab before it, whose state group 1 keeps in wp_*.
@@ -259,7 +268,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     uint32_t row;
     if (SWIGLU) row = (uint32_t)min((b >> 3) * 32 + (b & 3) * 8 + d_r, w_last) + (((b >> 2) & 1) ? (uint32_t)NCOLS : 0u);
     else row = (uint32_t)min(b * 8 + d_r, w_last);
-    const uint32_t off = row * KROW + d_c16;
+    const uint32_t off = mad24(row, KROW, d_c16);
     dma16((prev ? wp_wg : c.wg) + (prev ? wp_kt : c.kt) * 128, off,
           lds_base + ((prev ? wp_step : c.step) & 1) * STAGE + X_BYTES + b * 1024);
   };
