@@ -109,6 +109,8 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
   const bool decode_ok = K % 128 == 0;
   const int64_t ntn256 = (N + 255) / 256;
+  // The ping-pong kernel tabulates each workgroup's tile sequence and forms slab offsets with 24-bit multiplies.
+  const bool pingpong_ok = K < PINGPONG_MAX_ROW_BYTES / 2 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg);
   if (variant < 0 && decode_ok && use_streaming_kernel(M, G, ntn256, num_wg)) variant = MOE_GG_GG_DECODE;
   if (variant == MOE_GG_GG_DECODE) {
     if (!decode_ok) return MOE_GG_EUNSUPPORTED;
@@ -125,13 +127,14 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
     // to occupy the CUs, also for experts of 16 .. 128 rows (short tiles skip most of their work and
     // the kernel then streams weights at 5 TB/s); smaller tiles only pay for small problems.
     const int64_t t256 = (M / 256 + (G + 1) / 2) * ntn256;
-    if (t256 * 4 >= (int64_t)num_wg * 3 && K < PINGPONG_MAX_ROW_BYTES / 2) variant = MOE_GG_GG_PINGPONG_256;
+    if (t256 * 4 >= (int64_t)num_wg * 3 && pingpong_ok) variant = MOE_GG_GG_PINGPONG_256;
+    else if (t256 * 4 >= (int64_t)num_wg * 3) variant = MOE_GG_GG_TILED_256;
     else if (t256 * 4 >= num_wg) variant = MOE_GG_GG_TILED_128;
     else variant = MOE_GG_GG_TILED_64;
   }
   switch (variant) {
     case MOE_GG_GG_PINGPONG_256:
-      if (K >= PINGPONG_MAX_ROW_BYTES / 2) return MOE_GG_EUNSUPPORTED;
+      if (!pingpong_ok) return MOE_GG_EUNSUPPORTED;
       return (int)gg_bf16_pingpong_launch(p, num_wg, s);
     case MOE_GG_GG_TILED_256: return (int)gg_bf16_tiled_launch(p, 256, num_wg, s);
     case MOE_GG_GG_TILED_128: return (int)gg_bf16_tiled_launch(p, 128, num_wg, s);
@@ -175,8 +178,13 @@ int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* 
   // and a workgroup whose expert belongs to the other kernel exits after reading m_sizes. Otherwise the
   // ping-pong kernel does everything.
   int variant = g_variant[MOE_GG_OP_GG_FP8].load();
+  // The ping-pong kernel tabulates each workgroup's tile sequence: beyond its capacity the 128 x 128 kernel runs.
+  const bool pingpong_ok = moe_gg_two_list_fits(M, G, 256, (N + 255) / 256, num_wg);
   if (variant < 0)
-    variant = use_streaming_kernel(M, G, (N + 255) / 256, num_wg) ? MOE_GG_FP8_STREAM_PINGPONG : MOE_GG_FP8_PINGPONG;
+    variant = !pingpong_ok ? MOE_GG_FP8_TILED_128
+              : use_streaming_kernel(M, G, (N + 255) / 256, num_wg) ? MOE_GG_FP8_STREAM_PINGPONG : MOE_GG_FP8_PINGPONG;
+  else if (variant != MOE_GG_FP8_TILED_128 && variant != MOE_GG_FP8_STREAM_TILED && !pingpong_ok)
+    return MOE_GG_EUNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
   if (variant == MOE_GG_FP8_TILED_128) return (int)gg_fp8_launch(p, scale_mode, num_wg, s);
   if (variant == MOE_GG_FP8_PINGPONG) return (int)gg_fp8_pingpong_launch(p, scale_mode, num_wg, s);
@@ -278,6 +286,7 @@ int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const
   p.xcds = di->xcds;
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
+  if (!moe_gg_two_list_fits(M, G, 256, (n + 127) / 128, num_wg)) return MOE_GG_EUNSUPPORTED;
   return (int)gg_bf16_pingpong_swiglu_launch(p, num_wg, (hipStream_t)stream);
 }
 
@@ -359,7 +368,11 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   const int v = g_variant[MOE_GG_OP_GG_BF16].load();
   if (v == MOE_GG_GG_TILED_256) return (int)gg_bf16_wgrad_launch(p, 256, num_wg, s);
   if (v == MOE_GG_GG_TILED_128) return (int)gg_bf16_wgrad_launch(p, 128, num_wg, s);
-  if (v == MOE_GG_GG_PINGPONG_256 || (v < 0 && t256 * 4 >= (int64_t)num_wg * 3)) return (int)gg_bf16_pingpong_wgrad_launch(p, num_wg, s);
+  const bool pingpong_ok = t256 <= (int64_t)(MOE_GG_SEQ_CAP - 1) * num_wg;  // its per-workgroup tile table
+  if (v == MOE_GG_GG_PINGPONG_256 && !pingpong_ok) return MOE_GG_EUNSUPPORTED;
+  if (v == MOE_GG_GG_PINGPONG_256 || (v < 0 && pingpong_ok && t256 * 4 >= (int64_t)num_wg * 3))
+    return (int)gg_bf16_pingpong_wgrad_launch(p, num_wg, s);
+  if (v < 0 && t256 >= num_wg) return (int)gg_bf16_wgrad_launch(p, 256, num_wg, s);
   return (int)gg_bf16_wgrad_launch(p, 128, num_wg, s);
 }
 
@@ -455,9 +468,8 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     while ((n_long + n_low) * num_workgroups < total && moe_gg_tile_of(wg, num_workgroups, xcds, n_long + n_low) < total) ++n_low;
     const int n_my = n_long + n_low, phase = moe_gg_low_phase(wg, xcds);
     for (int seq = 0; seq < n_my; ++seq) {
-      const int lb = moe_gg_low_before(seq, n_my, n_low, phase);
-      const bool low = moe_gg_low_before(seq + 1, n_my, n_low, phase) > lb;
-      const int L = moe_gg_tile_of(wg, num_workgroups, xcds, low ? n_long + lb : seq - lb);
+      const int L = moe_gg_tile_of(wg, num_workgroups, xcds, moe_gg_seq_round(seq, n_my, n_low, phase));
+      const bool low = L >= nl;
       if (written >= max_tiles) return written;
       int g, tm, tn;
       if (!low) {

@@ -118,10 +118,9 @@ struct Shared {
   const int32_t* row_off;
   const int32_t* tile_off;   // forward: prefix of the long tiles; WGRAD: prefix of the padded 64-column blocks
   const int32_t* part_off;   // forward: prefix of the low tiles (one row of tiles per group at most)
+  const int32_t* seq_tab;    // the workgroup's tiles in the order it computes them: (group, row tile | column tile << 16)
   char* lds;
-  int n_my;      // tiles of this workgroup
-  int n_low_my;  // of which low tiles (forward only)
-  int phase;     // 0 .. 255: where in the workgroup's sequence its low tiles sit (the same for all workgroups of an XCD)
+  int n_my;       // tiles of this workgroup (<= MOE_GG_SEQ_CAP, the launcher's duty)
 };
 
 // Slab-load cursor of one wave: which slab (tile round, K step) its next load instructions fetch.
@@ -154,61 +153,32 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   const uint32_t KROW = WGRAD ? (uint32_t)p.M * 2u : (uint32_t)p.K * (FP8 ? 1u : 2u);  // bytes per operand row
   const int KT_fwd = (int)((uint32_t)p.K * (FP8 ? 1u : 2u) / 128u);  // K steps of every forward tile
   const int NCOLS = WGRAD ? p.K : (SWIGLU ? N / 2 : N);               // output columns of a group
-  const int wg_ntm = moe_gg_cdiv(N, BM);                             // WGRAD: tiles along the rows of dW
-  const int wg_tpg = wg_ntm * moe_gg_cdiv(p.K, BN);                  // WGRAD: tiles per expert
   const int nwg = gridDim.x;
   // Tile of a round. Forward: rows of x / rows of w[g]. WGRAD: rows of dY^T (n) / rows of X^T (k), both at the
   // column offset of the expert's padded block; t.row0 = first row of the expert's block of dW, t.rows = N.
   struct TileRef { MoeGgTile t; int KT; int64_t xoff, woff; };
-  // The workgroup's own sequence: its long tiles in round order with its low tiles spread evenly between
-  // them. low_before(i) = number of low tiles among the first i sequence positions; low tile j sits at
-  // position floor((j + phase / 256) * n_my / n_low_my). The phase differs between XCDs, so the low tiles
-  // (which stream a whole weight tile from memory for a few rows) are spread over the launch instead of
-  // running all at once, while the workgroups of one XCD still take theirs together and stay in step.
-  // (The block-scaled kernel has no registers left for this arithmetic: it keeps all tiles in the first list.)
-  auto low_before = [&](int i) { return BLOCK ? 0 : moe_gg_low_before(i, sh.n_my, sh.n_low_my, sh.phase); };
+  // The workgroup's own sequence (moe_gg_seq_round): its long tiles in round order with its low tiles spread
+  // evenly between them, at a phase that differs between XCDs, so that memory-bound low tiles and compute-bound
+  // long tiles run side by side on the chip, while the workgroups of one XCD take theirs together and stay in
+  // step. Tile ids: long tiles 0 .. n_long - 1, then the low tiles.
   auto tile_ref = [&](int seq) {
     TileRef r;
-    const int lb = uni(low_before(seq));
-    const bool low = uni(low_before(seq + 1)) > lb;
-    // Tile ids: long tiles 0 .. n_long - 1, then the low tiles; ids are dealt round-robin, so this workgroup's
-    // low tiles are its last rounds.
-    const int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, low ? (sh.n_my - sh.n_low_my) + lb : seq - lb);
+    // Decoded in the prologue: group, row tile | column tile << 16.
+    const int g = uni(sh.seq_tab[2 * seq]);
+    const int mn = uni(sh.seq_tab[2 * seq + 1]);
+    r.t.g = g; r.t.tm = mn & 0xFFFF; r.t.tn = (int)((uint32_t)mn >> 16);
     if (WGRAD) {
-      const int g = uni(L / wg_tpg);
-      const int rem = L - g * wg_tpg;
-      r.t.g = g; r.t.tn = uni(rem / wg_ntm); r.t.tm = rem - r.t.tn * wg_ntm;
       r.t.row0 = g * N; r.t.rows = N;
       const int b0 = uni(sh.tile_off[g]);
       r.KT = uni(sh.tile_off[g + 1]) - b0;
       r.xoff = (int64_t)(r.t.tm * BM) * KROW + (int64_t)b0 * 128;
       r.woff = (int64_t)(r.t.tn * BN) * KROW + (int64_t)b0 * 128;
     } else {
-      // Tile list: the long tiles of all groups (group, then column tile, then row tile), then the low tiles
-      // (group, column tile; see moe_gg_long_row_tiles), dealt to the workgroups round-robin:
-      // every workgroup gets the same number (+- 1) of long tiles, and the low tiles go on where the long
-      // ones stopped.
-      MoeGgTile t;
-      if (BLOCK || !low) {
-        t.g = moe_gg_find_group(sh.tile_off, p.G, L);
-        t.row0 = sh.row_off[t.g];
-        t.rows = sh.row_off[t.g + 1] - t.row0;
-        const int idx = L - sh.tile_off[t.g];
-        const int nf = BLOCK ? moe_gg_cdiv(t.rows, BM) : moe_gg_long_row_tiles(t.rows, BM);
-        t.tn = idx / nf;
-        t.tm = idx - t.tn * nf;
-      } else {
-        const int Lp = L - uni(sh.tile_off[p.G]);
-        t.g = moe_gg_find_group(sh.part_off, p.G, Lp);
-        t.row0 = sh.row_off[t.g];
-        t.rows = sh.row_off[t.g + 1] - t.row0;
-        t.tn = Lp - sh.part_off[t.g];
-        t.tm = t.rows / BM;
-      }
-      r.t = uni_tile(t);
+      r.t.row0 = uni(sh.row_off[g]);
+      r.t.rows = uni(sh.row_off[g + 1]) - r.t.row0;
       r.KT = KT_fwd;
       r.xoff = (int64_t)(r.t.row0 + r.t.tm * BM) * KROW;
-      r.woff = ((int64_t)r.t.g * N + r.t.tn * TILE_COLS) * KROW;
+      r.woff = ((int64_t)g * N + r.t.tn * TILE_COLS) * KROW;
     }
     return r;
   };
@@ -546,13 +516,9 @@ DEVINL void pingpong_body(const GgParams& p) {
     const int ntn = OP == OP_BF16_SWIGLU ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
     const int skip = p.skip_rows;
     build_row_offsets(p.m_sizes, p.G, p.M, row_off);
-    if (OP == OP_FP8_BLOCK) {
-      build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_cdiv(rows, BM) * ntn : 0; });
-    } else {
-      build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
-      build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
-      total_low = uni(part_off[p.G]);
-    }
+    build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
+    build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
+    total_low = uni(part_off[p.G]);
     total = uni(tile_off[p.G]);
   }
   const int nwg = gridDim.x;
@@ -562,8 +528,38 @@ DEVINL void pingpong_body(const GgParams& p) {
   while ((n_long + n_low) * nwg < total + total_low && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < total + total_low)
     ++n_low;
   if (n_long + n_low == 0) return;
+  // The sequence of this workgroup (moe_gg_seq_round), decoded once into a table: the arithmetic runs per thread
+  // here; in the K loop it would occupy scalar registers that the loop needs.
+  // Tile ids: the long tiles of all groups (group, then column tile, then row tile), then the low tiles (group,
+  // column tile; see moe_gg_long_row_tiles), dealt to the workgroups round-robin: every workgroup gets the same
+  // number (+- 1) of long tiles, and the low tiles go on where the long ones stopped.
+  __shared__ int32_t seq_tab[2 * MOE_GG_SEQ_CAP];
+  const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
+  for (int i = threadIdx.x; i < n_my; i += NT) {
+    const int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
+    int g, tm, tn;
+    if (OP == OP_BF16_WGRAD) {
+      const int ntm = moe_gg_cdiv(p.N, BM), tpg = ntm * moe_gg_cdiv(p.K, BN);
+      g = L / tpg;
+      const int rem = L - g * tpg;
+      tn = rem / ntm; tm = rem - tn * ntm;
+    } else if (L < total) {
+      g = moe_gg_find_group(tile_off, p.G, L);
+      const int idx = L - tile_off[g];
+      const int nf = moe_gg_long_row_tiles(row_off[g + 1] - row_off[g], BM);
+      tn = idx / nf; tm = idx - tn * nf;
+    } else {
+      const int Lp = L - total;
+      g = moe_gg_find_group(part_off, p.G, Lp);
+      tn = Lp - part_off[g];
+      tm = (row_off[g + 1] - row_off[g]) / BM;
+    }
+    seq_tab[2 * i] = g;
+    seq_tab[2 * i + 1] = tm | (tn << 16);
+  }
+  __syncthreads();
 
-  Shared sh{row_off, tile_off, part_off, lds, n_long + n_low, n_low, moe_gg_low_phase(blockIdx.x, p.xcds)};
+  Shared sh{row_off, tile_off, part_off, seq_tab, lds, n_my};
   const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
   if (grp == 0) run_group<0, OP>(p, sh);
   else run_group<1, OP>(p, sh);

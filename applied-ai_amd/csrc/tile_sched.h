@@ -88,13 +88,15 @@ MOE_GG_HD int moe_gg_tile_of(int wg, int nwg, int xcds, int round) {
 }
 
 // ---- Two-list order of the ping-pong kernel ---------------------------------------------------------
-// Row tiles of a group that go into the list of long tiles: all of them, except a last tile of fewer than
-// BM / 2 rows when the group has at least two full tiles before it. Such a low tile goes into the list of low
-// tiles. (A low tile streams its whole weight tile for a few rows; next to its full neighbours it finds their
-// weight slabs in the L2, away from them it reads them again, which only pays for tall groups, where the
-// better balance is worth more than one more pass over the group's weights.)
+// Row tiles of a group that go into the list of long tiles. A tile of fewer than BM / 2 rows is a low tile
+// (it streams its whole weight tile for a few rows: bound by memory, not by the matrix pipes) and goes into
+// the second list when nothing is lost by taking it away from its neighbours: when it is the only row tile of
+// its group, or the last one of a group with at least two full tiles before it. (Next to its full neighbours a
+// low tile finds their weight slabs in the L2; away from them it reads them again, which only pays for tall
+// groups, where the better balance is worth more than one more pass over the group's weights.)
 MOE_GG_HD int moe_gg_long_row_tiles(int rows, int BM) {
   const int full = rows / BM, rem = rows - full * BM;
+  if (full == 0) return rem >= BM / 2 ? 1 : 0;
   return full + ((rem >= BM / 2 || (rem > 0 && full < 2)) ? 1 : 0);
 }
 MOE_GG_HD int moe_gg_low_row_tiles(int rows, int BM) { return moe_gg_cdiv(rows, BM) - moe_gg_long_row_tiles(rows, BM); }
@@ -104,11 +106,25 @@ MOE_GG_HD int moe_gg_low_row_tiles(int rows, int BM) { return moe_gg_cdiv(rows, 
 // low tile j sits at position floor((j + phase / 256) * n_my / n_low_my), 0 <= phase < 256.
 MOE_GG_HD int moe_gg_low_before(int i, int n_my, int n_low_my, int phase) {
   if (n_low_my == 0) return 0;
-  const int den = 256 * n_my;
-  const int num = i * n_low_my * 256 - phase * n_my;
-  const int c = num <= 0 ? 0 : (num + den - 1) / den;
-  return c < n_low_my ? c : n_low_my;
+  const long long den = 256LL * n_my;
+  const long long num = (long long)i * n_low_my * 256 - (long long)phase * n_my;
+  const long long c = num <= 0 ? 0 : (num + den - 1) / den;
+  return c < n_low_my ? (int)c : n_low_my;
 }
 // Phase of a workgroup: the same for all workgroups of an XCD (they take their low tiles together and stay in
-// step), different between XCDs (the low tiles, which are memory-bound, are spread over the launch).
+// step), different between XCDs (memory-bound and compute-bound tiles then run side by side on the chip).
 MOE_GG_HD int moe_gg_low_phase(int wg, int xcds) { return ((wg % xcds) * 256 + 128) / xcds; }
+
+// Round (argument of moe_gg_tile_of over the concatenated list: long tiles, then low tiles) of sequence
+// position seq. The kernel tabulates a workgroup's sequence, which may have at most MOE_GG_SEQ_CAP positions;
+// moe_gg_two_list_fits tells a launcher, from the shape alone, whether that holds for every m_sizes.
+#define MOE_GG_SEQ_CAP 1024
+MOE_GG_HD int moe_gg_seq_round(int seq, int n_my, int n_low_my, int phase) {
+  const int lb = moe_gg_low_before(seq, n_my, n_low_my, phase);
+  const bool low = moe_gg_low_before(seq + 1, n_my, n_low_my, phase) > lb;
+  return low ? (n_my - n_low_my) + lb : seq - lb;
+}
+// Upper bound of the tile count: sum of ceil(m_g / BM) <= M / BM + G row tiles, times the column tiles.
+MOE_GG_HD bool moe_gg_two_list_fits(int64_t M, int G, int BM, int n_tiles_n, int num_wg) {
+  return (M / BM + G) * (int64_t)n_tiles_n <= (int64_t)(MOE_GG_SEQ_CAP - 1) * num_wg;
+}
