@@ -374,10 +374,11 @@ hipError_t launch(const W4Params& p, hipStream_t stream) {
   // expert with more rows than one pass covers is done in several passes over its weights).
   dim3 grid((p.N + 63) / 64, p.m_sizes ? p.G : 1), block(64 * WAVES);
   const int M = p.m_sizes ? (p.M + p.G - 1) / p.G : p.M;
-  // M <= 16 and group size 128: one activation fragment, all loads issued one group ahead (deeper queues
-  // and more waves measured slower). Larger M keeps up to four activation fragments per pass so that the
-  // weights are unpacked once per four fragments.
+  // Group size 128: one activation fragment per pass for M <= 16, two for more rows (32 rows per pass over the
+  // weights; four fragments do not fit the registers), all loads issued one group ahead (deeper queues and
+  // more waves measured slower). Other group sizes: up to four activation fragments per pass.
   if (M <= 16 && p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES>), grid, block, 0, stream, p);
+  else if (p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 2, 1, WAVES>), grid, block, 0, stream, p);
   else if (M <= 16) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 1>), grid, block, 0, stream, p);
   else if (M <= 32) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 2>), grid, block, 0, stream, p);
   else hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 4>), grid, block, 0, stream, p);

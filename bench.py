@@ -127,7 +127,7 @@ def secondary_workloads(torch, A, dev):
         byt = K * N // 2 + (K // 128) * N * 2 + (K // 128) * N // 2 + M * K * 2 + M * N * 2
         out.append({"workload": f"W4A16 split-K M={M} K=4096 N=14336 group 128",
                     "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
-                    "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128" if M <= 16 else "w4a16_splitk_anygroup", "achieved": round(byt / ms / 1e6, 1),
+                    "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128", "achieved": round(byt / ms / 1e6, 1),
                                  "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
                                  "traffic": None}})
     del qws
