@@ -336,18 +336,40 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   void* dyc = ws;
 
   hipError_t e;
+  int num_wg = di->cus - di->cus % di->xcds;
+  int xcds = di->xcds;
+  if (num_wg <= 0) { num_wg = di->cus; xcds = 1; }
+  const int v = g_variant[MOE_GG_OP_GG_BF16].load();
   if (M > 0) {
-    // grad_x: the forward kernels on (dY [M, N], w^T [G*K, N]).
-    e = transpose_batched_launch(w, wt, G, N, K, s);
-    if (e != hipSuccess) return (int)e;
     const void* dy = grad_out;
     if (grad_layout == MOE_GG_OUT_BLOCK) {
       e = compact_block_launch(grad_out, dyc, m_sizes, G, (int)M, N, ld_go, N, s);
       if (e != hipSuccess) return (int)e;
       dy = dyc;
     }
-    rc = moe_gg_grouped_gemm_bf16(dy, wt, grad_x, m_sizes, G, M, K, N, K, MOE_GG_OUT_MN, stream);
-    if (rc != MOE_GG_OK) return rc;
+    // grad_x = dY [M, N] times w[g] [N, K]. With enough 256 x 256 tiles the ping-pong kernel reads w as it is
+    // (transposing LDS reads); otherwise, or when a kernel variant is pinned, the forward kernels run on a
+    // transposed copy w^T [G*K, N].
+    const int64_t ntn256 = (K + 255) / 256;
+    const int64_t t256 = (M / 256 + (G + 1) / 2) * ntn256;
+    const bool nt_ok = v < 0 && N % 64 == 0 && K % 8 == 0 && (int64_t)N < PINGPONG_MAX_ROW_BYTES / 2 &&
+                       (int64_t)K < PINGPONG_MAX_ROW_BYTES / 2 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg) &&
+                       t256 * 4 >= (int64_t)num_wg * 3;
+    if (nt_ok) {
+      GgParams q{};
+      q.x = dy; q.w = w; q.y = grad_x; q.m_sizes = m_sizes;
+      q.G = G; q.M = (int)M; q.N = K; q.K = N;
+      q.ldy = K;
+      q.vec_store = aligned(grad_x, 8) && K % 4 == 0;
+      q.xcds = xcds;
+      e = gg_bf16_pingpong_nt_launch(q, num_wg, s);
+      if (e != hipSuccess) return (int)e;
+    } else {
+      e = transpose_batched_launch(w, wt, G, N, K, s);
+      if (e != hipSuccess) return (int)e;
+      rc = moe_gg_grouped_gemm_bf16(dy, wt, grad_x, m_sizes, G, M, K, N, K, MOE_GG_OUT_MN, stream);
+      if (rc != MOE_GG_OK) return rc;
+    }
     // grad_w: dY^T and x^T with every expert padded to whole 64-row blocks.
     e = transpose_padded_launch(grad_out, dyt, m_sizes, G, (int)M, N, ld_go, grad_layout == MOE_GG_OUT_BLOCK ? N : 0, ldm, s);
     if (e != hipSuccess) return (int)e;
@@ -360,12 +382,9 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   p.ldy = K;
   p.col_block = 0;
   p.vec_store = aligned(grad_w, 8) && K % 4 == 0;
-  p.xcds = di->xcds;
+  p.xcds = xcds;
   p.skip_rows = (int)M;
-  int num_wg = di->cus - di->cus % p.xcds;
-  if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
   const int64_t t256 = (int64_t)G * ((N + 255) / 256) * ((K + 255) / 256);
-  const int v = g_variant[MOE_GG_OP_GG_BF16].load();
   if (v == MOE_GG_GG_TILED_256) return (int)gg_bf16_wgrad_launch(p, 256, num_wg, s);
   if (v == MOE_GG_GG_TILED_128) return (int)gg_bf16_wgrad_launch(p, 128, num_wg, s);
   const bool pingpong_ok = t256 <= (int64_t)(MOE_GG_SEQ_CAP - 1) * num_wg;  // its per-workgroup tile table

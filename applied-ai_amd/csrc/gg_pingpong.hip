@@ -71,7 +71,17 @@ constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x
 // 32 output columns: weight-tile row 64 wn + 32 h + c (h = 0 gate, 1 up) is output column 32 wn + c.
 // Both products are rounded to bf16 before the activation, as they are when the GEMM output is stored first.
 // p.N = 2n.
-constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4;
+// OP_BF16_NT: the product with weights that are NOT stored along the reduction, y[m][c] = sum_r x[m][r] * w[g][r][c]
+// with w [G * R, C] row-major (p.K = R, p.N = C): the input gradient of the layer, dX = dY w, read from the
+// forward weights as they are (kernels/MoE/group_GEMM/triton/tgroup_gemm_backwards.py:27-199 reads a transposed
+// copy). A K step's weight slab is 64 rows r of 256 columns; each half (128 columns, 256-byte rows) is written
+// into its LDS region row by row and read with ds_read_b64_tr_b16, which hands lane l of a 16-lane group column
+// l of a 4-row block: two such reads give the lane the eight consecutive r of its column that the MFMA wants.
+// Rows of 256 bytes cover all LDS banks, so the 32-byte column blocks are XOR-swizzled with
+// (r & 3) | ((r >> 3) & 1) << 2: the 16 rows one instruction touches then fall on 8 different bank groups twice
+// (512 bytes per instruction: the minimum).
+constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4, OP_BF16_NT = 5;
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
 // 64 lanes x 16 B (or 4 B) from global memory straight into LDS: lane l's bytes land at lds_addr + 16 l
 // (4 l). Issued from inline assembly so that the compiler does not serialise the in-flight slab against
@@ -142,6 +152,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   constexpr bool BLOCK = OP == OP_FP8_BLOCK;
   constexpr bool WGRAD = OP == OP_BF16_WGRAD;
   constexpr bool SWIGLU = OP == OP_BF16_SWIGLU;
+  constexpr bool WNT = OP == OP_BF16_NT;  // weights not transposed
   constexpr int TILE_COLS = SWIGLU ? BN / 2 : BN;  // output columns of a tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -178,7 +189,8 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       r.t.rows = uni(sh.row_off[g + 1]) - r.t.row0;
       r.KT = KT_fwd;
       r.xoff = (int64_t)(r.t.row0 + r.t.tm * BM) * KROW;
-      r.woff = ((int64_t)g * N + r.t.tn * TILE_COLS) * KROW;
+      if (WNT) r.woff = ((int64_t)g * p.K * N + r.t.tn * TILE_COLS) * 2;  // w[g][0][n0]
+      else r.woff = ((int64_t)g * N + r.t.tn * TILE_COLS) * KROW;
     }
     return r;
   };
@@ -233,8 +245,21 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   // Weight rows: of the cursor slab, or (prev) of the slab before it, whose state group 1 keeps in wp_*.
   const char* wp_wg = nullptr;
   int wp_last = 0, wp_kt = 0, wp_step = 0;
+  const uint32_t WROW = (uint32_t)N * 2u;  // OP_BF16_NT: bytes per weight row (one r, all columns)
   auto dma_w = [&](int b, bool prev) {
     const int w_last = prev ? wp_last : c.w_last;
+    if (WNT) {
+      // Block b: rows 4 (b & 15) .. + 3 of the slab's 64, column half b >> 4; lane -> row lane / 16, physical
+      // 16-byte slot lane % 16, which holds logical chunk slot ^ (swizzle(row) << 1). Chunks beyond the last
+      // valid column re-read that one (their columns are never stored).
+      const int bb = b & 15;
+      const uint32_t sw = (uint32_t)((lane >> 4) | (((bb >> 1) & 1) << 2));
+      const uint32_t chunk = (uint32_t)min((int)(((b >> 4) << 4) + ((lane & 15) ^ (sw << 1))), w_last >> 3);
+      const uint32_t off = mad24((uint32_t)(bb * 4 + (lane >> 4)), WROW, chunk << 4);
+      dma16((prev ? wp_wg : c.wg) + (int64_t)(prev ? wp_kt : c.kt) * (64 * (int64_t)WROW), off,
+            lds_base + ((prev ? wp_step : c.step) & 1) * STAGE + X_BYTES + b * 1024);
+      return;
+    }
     uint32_t row;
     if (SWIGLU) row = (uint32_t)min((b >> 3) * 32 + (b & 3) * 8 + d_r, w_last) + (((b >> 2) & 1) ? (uint32_t)NCOLS : 0u);
     else row = (uint32_t)min(b * 8 + d_r, w_last);
@@ -327,6 +352,13 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         const char* xs = sh.lds + (step & 1) * STAGE + wm * 2048;
         const char* ws = sh.lds + (step & 1) * STAGE + X_BYTES + wn * (FN * 2048);
         u32x4_t wf[2][FN], xf[2][FM];
+        // OP_BF16_NT: the lane's address inside the wave's column half for fragment f: row block of its k quarter, row
+        // lane % 16 / 4 of a 4-row block, swizzled 32-byte column block, 8-byte piece lane % 4.
+        auto wt_addr = [&](int f) {
+          const int ti = (lane & 15) >> 2, ts = ti | ((fq & 1) << 2);
+          return lds_base + (uint32_t)((step & 1) * STAGE + X_BYTES + (wn >> 1) * 16384 + fq * 2048 + ti * 256 +
+                                       (((((wn & 1) << 2) + f) ^ ts) << 5) + (lane & 3) * 8);
+        };
         int issued = 0;
 #pragma unroll
         for (int q = 0; q < 24; ++q) {
@@ -340,7 +372,14 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
           }
           const int kk = q / 12, f = q % 12;
           const int ro = kk ? (rd0 ^ 64) : rd0;
-          if (f < FN) wf[kk][f] = *(const u32x4_t*)(ws + f * 2048 + ro);
+          if (f < FN && WNT) {
+            typedef __attribute__((address_space(3))) i16x4_t* lds_i16x4_ptr;
+            const uint32_t a = wt_addr(f) + kk * 8192;
+            const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)a);
+            const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)(a + 1024));
+            const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
+            wf[kk][f] = u32x4_t{l2[0], l2[1], h2[0], h2[1]};
+          } else if (f < FN) wf[kk][f] = *(const u32x4_t*)(ws + f * 2048 + ro);
           else xf[kk][f - FN] = *(const u32x4_t*)(xs + (f - FN) * (WM * 2048) + ro);
         }
         float sc[FM];
@@ -568,6 +607,7 @@ DEVINL void pingpong_body(const GgParams& p) {
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_body<OP_BF16>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong_nt(GgParams p) { pingpong_body<OP_BF16_NT>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise(GgParams p) { pingpong_body<OP_FP8_ROW>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpong_body<OP_FP8_BLOCK>(p); }
 
@@ -585,6 +625,11 @@ hipError_t gg_bf16_pingpong_wgrad_launch(const GgParams& p, int num_wg, hipStrea
 
 hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream) {
   hipLaunchKernelGGL(gg_bf16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t gg_bf16_pingpong_nt_launch(const GgParams& p, int num_wg, hipStream_t stream) {
+  hipLaunchKernelGGL(gg_bf16_pingpong_nt, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
 

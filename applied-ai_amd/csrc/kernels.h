@@ -85,6 +85,9 @@ hipError_t compact_block_launch(const void* src, void* dst, const int32_t* m_siz
                                 int col_block, hipStream_t stream);
 // y [M, n] = silu(x w_gate^T) * (x w_up^T) with w [G * 2n, K] (gate rows first); p.N = 2n, p.ldy >= n, p.col_block unused.
 hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream);
+// y [M, N] = x [M, K] times w[g] [K, N] (weights row-major along N, not along the reduction): p.w = [G * K, N].
+// K % 64 == 0, N % 8 == 0.
+hipError_t gg_bf16_pingpong_nt_launch(const GgParams& p, int num_wg, hipStream_t stream);
 hipError_t gg_bf16_pingpong_wgrad_launch(const GgParams& p, int num_wg, hipStream_t stream);
 // dW = dY^T X per expert on the transposed, padded operands; p.x = dY^T [N, ldm], p.w = X^T [K, ldm], p.M = ldm,
 // p.skip_rows = number of gradient rows (bound for m_sizes), p.y = dW [G * N, K] with p.ldy = K. block in {256, 128}.

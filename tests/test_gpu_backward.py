@@ -109,3 +109,29 @@ def test_errors():
         A.grouped_gemm_backward(go[:, :100], x, w, m)
     with pytest.raises(RuntimeError):
         A.grouped_gemm_backward(go.cpu(), x, w, m)
+
+
+@pytest.mark.parametrize("sizes,M,N,K", [
+    ([513, 255, 1, 0, 700, 128, 64, 1290], 3000, 256, 3080),    # partial column tiles (K % 256 = 8), ragged rows
+    ([1012, 1039, 1048, 1036], 4160, 1024, 4096),
+    ([300] * 8, 2400, 512, 512),                                # too few tiles: both runs take the transposed copy
+])
+def test_grad_x_from_untransposed_weights_equals_the_transposed_copy_path(sizes, M, N, K):
+    """With enough tiles grad_x comes from the kernel that reads w as stored (transposing LDS reads); pinning a
+    kernel variant selects the path through a transposed copy of w. Same products, same accumulation order per
+    tile: bit-identical, and both within the bar of the oracle (run_case)."""
+    import applied_ai_amd as A
+    from applied_ai_amd import _lib
+
+    if K > 512:
+        # the library's rule for the direct kernel on a 256-CU part: enough 256 x 256 tiles of grad_x
+        assert (M // 256 + (len(sizes) + 1) // 2) * ((K + 255) // 256) * 4 >= 256 * 3
+    gx_nt, gw_nt = run_case(sizes, M, N, K, seed=33, scale=0.5)
+    L = _lib.lib()
+    try:
+        assert L.moe_gg_set_variant(0, 0) == 0      # ping-pong forward kernel on w^T
+        gx_t, gw_t = run_case(sizes, M, N, K, seed=33, scale=0.5)
+    finally:
+        L.moe_gg_set_variant(0, -1)
+    np.testing.assert_array_equal(gx_nt, gx_t)
+    np.testing.assert_array_equal(gw_nt, gw_t)
