@@ -38,13 +38,17 @@ int current_device_info(const DeviceInfo** out) {
 
 bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
-// The dedicated small-M kernels (weights streamed straight into MFMA operands, split-K inside the workgroup)
-// beat the ping-pong kernel only for a few rows per expert (measured: up to about 12) or when the launch has
+// fp8: the dedicated small-M kernel (weights streamed straight into MFMA operands, split-K inside the workgroup)
+// beats the ping-pong kernel only for a few rows per expert (measured: up to about 12) or when the launch has
 // too few 256 x 256 tiles to give every CU several (few experts, narrow N); never above 40 rows per expert.
 bool use_streaming_kernel(int64_t M, int G, int64_t ntn256, int num_wg) {
   if (M > (int64_t)G * 40) return false;
   return M <= (int64_t)G * 12 || (int64_t)G * ntn256 < 4 * (int64_t)num_wg;
 }
+// bf16: the small-M kernel streams weights at 5.8-6.0 TB/s with one or two activation fragments per pass (up
+// to 24 rows per expert on average) and beats every tiled kernel there (measured for 8-64 experts, N and K of
+// 2048-14336); with four fragments it falls behind them.
+bool use_decode_kernel(int64_t M, int G) { return M <= (int64_t)G * 24; }
 
 }  // namespace
 
@@ -111,7 +115,7 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
   const int64_t ntn256 = (N + 255) / 256;
   // The ping-pong kernel tabulates each workgroup's tile sequence and forms slab offsets with 24-bit multiplies.
   const bool pingpong_ok = K < PINGPONG_MAX_ROW_BYTES / 2 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg);
-  if (variant < 0 && decode_ok && use_streaming_kernel(M, G, ntn256, num_wg)) variant = MOE_GG_GG_DECODE;
+  if (variant < 0 && decode_ok && use_decode_kernel(M, G)) variant = MOE_GG_GG_DECODE;
   if (variant == MOE_GG_GG_DECODE) {
     if (!decode_ok) return MOE_GG_EUNSUPPORTED;
     const int64_t avg = (M + G - 1) / G;

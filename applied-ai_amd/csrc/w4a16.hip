@@ -319,7 +319,9 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
               xb[i][3] = __builtin_amdgcn_perm(xv[3], xv[1], 0x07060302u);  // k 3, 7
             }
             const u32x4_t w4 = wb[d];
-            if (more) load_step(d, (gi + GA) * SPG + e);
+            // Refill two K steps at a time: their activation fragments are the two halves of the same 128-byte
+            // lines, and issued back to back the second load still finds the line in the vector L1.
+            if (more && (e & 1)) { load_step(d - 1, (gi + GA) * SPG + e - 1); load_step(d, (gi + GA) * SPG + e); }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               u32x4_t bf;
