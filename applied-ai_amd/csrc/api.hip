@@ -344,38 +344,59 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   int xcds = di->xcds;
   if (num_wg <= 0) { num_wg = di->cus; xcds = 1; }
   const int v = g_variant[MOE_GG_OP_GG_BF16].load();
+  const int x_col_block = grad_layout == MOE_GG_OUT_BLOCK ? N : 0;
+  // Both gradients can be computed from the operands as stored (ping-pong kernels with transposing LDS reads)
+  // when there are enough 256 x 256 tiles and the row pitches allow 16-byte pieces; no workspace is touched then.
+  // Otherwise, or when a kernel variant is pinned, the operands are transposed into the workspace first.
+  const bool direct_shapes = v < 0 && N % 8 == 0 && K % 8 == 0 && ld_go % 8 == 0 &&
+                             ld_go < PINGPONG_MAX_ROW_BYTES / 2 && (int64_t)K < PINGPONG_MAX_ROW_BYTES / 2 &&
+                             (int64_t)N < PINGPONG_MAX_ROW_BYTES / 2;
   if (M > 0) {
-    const void* dy = grad_out;
-    if (grad_layout == MOE_GG_OUT_BLOCK) {
-      e = compact_block_launch(grad_out, dyc, m_sizes, G, (int)M, N, ld_go, N, s);
-      if (e != hipSuccess) return (int)e;
-      dy = dyc;
-    }
-    // grad_x = dY [M, N] times w[g] [N, K]. With enough 256 x 256 tiles the ping-pong kernel reads w as it is
-    // (transposing LDS reads); otherwise, or when a kernel variant is pinned, the forward kernels run on a
-    // transposed copy w^T [G*K, N].
+    // grad_x = dY [M, N] times w[g] [N, K].
     const int64_t ntn256 = (K + 255) / 256;
     const int64_t t256 = (M / 256 + (G + 1) / 2) * ntn256;
-    const bool nt_ok = v < 0 && N % 64 == 0 && K % 8 == 0 && (int64_t)N < PINGPONG_MAX_ROW_BYTES / 2 &&
-                       (int64_t)K < PINGPONG_MAX_ROW_BYTES / 2 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg) &&
+    const bool nt_ok = direct_shapes && N % 64 == 0 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg) &&
                        t256 * 4 >= (int64_t)num_wg * 3;
     if (nt_ok) {
       GgParams q{};
-      q.x = dy; q.w = w; q.y = grad_x; q.m_sizes = m_sizes;
+      q.x = grad_out; q.w = w; q.y = grad_x; q.m_sizes = m_sizes;
       q.G = G; q.M = (int)M; q.N = K; q.K = N;
       q.ldy = K;
+      q.ldx = (int)ld_go; q.x_col_block = x_col_block;
       q.vec_store = aligned(grad_x, 8) && K % 4 == 0;
       q.xcds = xcds;
       e = gg_bf16_pingpong_nt_launch(q, num_wg, s);
       if (e != hipSuccess) return (int)e;
     } else {
+      // The forward kernels on (dY [M, N] dense, w^T [G*K, N]).
+      const void* dy = grad_out;
+      if (grad_layout == MOE_GG_OUT_BLOCK) {
+        e = compact_block_launch(grad_out, dyc, m_sizes, G, (int)M, N, ld_go, N, s);
+        if (e != hipSuccess) return (int)e;
+        dy = dyc;
+      }
       e = transpose_batched_launch(w, wt, G, N, K, s);
       if (e != hipSuccess) return (int)e;
       rc = moe_gg_grouped_gemm_bf16(dy, wt, grad_x, m_sizes, G, M, K, N, K, MOE_GG_OUT_MN, stream);
       if (rc != MOE_GG_OK) return rc;
     }
-    // grad_w: dY^T and x^T with every expert padded to whole 64-row blocks.
-    e = transpose_padded_launch(grad_out, dyt, m_sizes, G, (int)M, N, ld_go, grad_layout == MOE_GG_OUT_BLOCK ? N : 0, ldm, s);
+  }
+  // grad_w[g] = dY_g^T X_g.
+  const int64_t t256 = (int64_t)G * ((N + 255) / 256) * ((K + 255) / 256);
+  const bool pingpong_ok = t256 <= (int64_t)(MOE_GG_SEQ_CAP - 1) * num_wg;  // its per-workgroup tile table
+  if (M > 0 && direct_shapes && pingpong_ok && t256 * 4 >= (int64_t)num_wg * 3) {
+    GgParams q{};
+    q.x = grad_out; q.w = x; q.y = grad_w; q.m_sizes = m_sizes;
+    q.G = G; q.M = (int)M; q.N = N; q.K = K;
+    q.ldy = K;
+    q.ldx = (int)ld_go; q.x_col_block = x_col_block;
+    q.vec_store = aligned(grad_w, 8) && K % 4 == 0;
+    q.xcds = xcds;
+    return (int)gg_bf16_pingpong_wgrad_direct_launch(q, num_wg, s);
+  }
+  if (M > 0) {
+    // dY^T and x^T with every expert padded to whole 64-row blocks.
+    e = transpose_padded_launch(grad_out, dyt, m_sizes, G, (int)M, N, ld_go, x_col_block, ldm, s);
     if (e != hipSuccess) return (int)e;
     e = transpose_padded_launch(x, xt, m_sizes, G, (int)M, K, K, 0, ldm, s);
     if (e != hipSuccess) return (int)e;
@@ -388,10 +409,8 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   p.vec_store = aligned(grad_w, 8) && K % 4 == 0;
   p.xcds = xcds;
   p.skip_rows = (int)M;
-  const int64_t t256 = (int64_t)G * ((N + 255) / 256) * ((K + 255) / 256);
   if (v == MOE_GG_GG_TILED_256) return (int)gg_bf16_wgrad_launch(p, 256, num_wg, s);
   if (v == MOE_GG_GG_TILED_128) return (int)gg_bf16_wgrad_launch(p, 128, num_wg, s);
-  const bool pingpong_ok = t256 <= (int64_t)(MOE_GG_SEQ_CAP - 1) * num_wg;  // its per-workgroup tile table
   if (v == MOE_GG_GG_PINGPONG_256 && !pingpong_ok) return MOE_GG_EUNSUPPORTED;
   if (v == MOE_GG_GG_PINGPONG_256 || (v < 0 && pingpong_ok && t256 * 4 >= (int64_t)num_wg * 3))
     return (int)gg_bf16_pingpong_wgrad_launch(p, num_wg, s);

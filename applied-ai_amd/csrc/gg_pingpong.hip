@@ -80,7 +80,13 @@ constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x
 // Rows of 256 bytes cover all LDS banks, so the 32-byte column blocks are XOR-swizzled with
 // (r & 3) | ((r >> 3) & 1) << 2: the 16 rows one instruction touches then fall on 8 different bank groups twice
 // (512 bytes per instruction: the minimum).
-constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4, OP_BF16_NT = 5;
+// OP_BF16_WGRAD_DIRECT: the weight gradient read from dY [M, ldx] and X [M, K] as stored: both operands have the
+// reduction index (the row m) as their slow dimension, so both slabs are 64 rows by 256 columns in the layout of
+// OP_BF16_NT and both fragment kinds come from transposing reads. A tile reduces over the rows of its expert:
+// max(1, ceil(m_g / 64)) K steps; rows beyond the expert's last one re-read that row (the loads stay inside the
+// tensors), and group 0 overwrites them with zeros in the dY slab once it has landed, so they add nothing.
+constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4, OP_BF16_NT = 5,
+              OP_BF16_WGRAD_DIRECT = 6;
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
 // 64 lanes x 16 B (or 4 B) from global memory straight into LDS: lane l's bytes land at lds_addr + 16 l
@@ -143,6 +149,7 @@ struct Cursor {
   int w_last;       // last valid weight row of the tile
   int ws_second;    // block mode: byte offset of the second column block's scales (0 if there is none)
   int KT;           // K steps of the cursor's tile
+  int rows_g;       // WGRAD_DIRECT: rows of the tile's expert (its reduction length)
   int round, kt, step;
 };
 
@@ -152,7 +159,8 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   constexpr bool BLOCK = OP == OP_FP8_BLOCK;
   constexpr bool WGRAD = OP == OP_BF16_WGRAD;
   constexpr bool SWIGLU = OP == OP_BF16_SWIGLU;
-  constexpr bool WNT = OP == OP_BF16_NT;  // weights not transposed
+  constexpr bool WG2 = OP == OP_BF16_WGRAD_DIRECT;
+  constexpr bool WNT = OP == OP_BF16_NT || WG2;  // weight slab: 64 reduction rows by 256 columns (transposing reads)
   constexpr int TILE_COLS = SWIGLU ? BN / 2 : BN;  // output columns of a tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -163,11 +171,14 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   const int N = p.N;
   const uint32_t KROW = WGRAD ? (uint32_t)p.M * 2u : (uint32_t)p.K * (FP8 ? 1u : 2u);  // bytes per operand row
   const int KT_fwd = (int)((uint32_t)p.K * (FP8 ? 1u : 2u) / 128u);  // K steps of every forward tile
-  const int NCOLS = WGRAD ? p.K : (SWIGLU ? N / 2 : N);               // output columns of a group
+  const int NCOLS = (WGRAD || WG2) ? p.K : (SWIGLU ? N / 2 : N);      // output columns of a group
+  // Bytes between rows of the x operand: the two backward kernels read the output gradient with its own leading
+  // dimension and, for the [M, N * G] layout, at the expert's column block.
+  const uint32_t XPITCH = (WG2 || OP == OP_BF16_NT) ? (uint32_t)p.ldx * 2u : KROW;
   const int nwg = gridDim.x;
   // Tile of a round. Forward: rows of x / rows of w[g]. WGRAD: rows of dY^T (n) / rows of X^T (k), both at the
   // column offset of the expert's padded block; t.row0 = first row of the expert's block of dW, t.rows = N.
-  struct TileRef { MoeGgTile t; int KT; int64_t xoff, woff; };
+  struct TileRef { MoeGgTile t; int KT, rows_g; int64_t xoff, woff; };
   // The workgroup's own sequence (moe_gg_seq_round): its long tiles in round order with its low tiles spread
   // evenly between them, at a phase that differs between XCDs, so that memory-bound low tiles and compute-bound
   // long tiles run side by side on the chip, while the workgroups of one XCD take theirs together and stay in
@@ -178,7 +189,18 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const int g = uni(sh.seq_tab[2 * seq]);
     const int mn = uni(sh.seq_tab[2 * seq + 1]);
     r.t.g = g; r.t.tm = mn & 0xFFFF; r.t.tn = (int)((uint32_t)mn >> 16);
-    if (WGRAD) {
+    r.rows_g = 0;
+    if (WG2) {
+      // Output: rows tm * 256 .. of the expert's block of dW (n), columns tn * 256 .. (k). Operands: the expert's
+      // rows of dY at columns g * x_col_block + tm * 256 .., and of X at columns tn * 256 ...
+      int row0 = uni(sh.row_off[g]);
+      r.rows_g = uni(sh.row_off[g + 1]) - row0;
+      if (r.rows_g == 0) row0 = min(row0, p.M - 1);  // an expert without rows: one K step of zeros, loads in bounds
+      r.t.row0 = g * N; r.t.rows = N;
+      r.KT = max(1, moe_gg_cdiv(r.rows_g, 64));
+      r.xoff = (int64_t)row0 * XPITCH + ((int64_t)g * p.x_col_block + r.t.tm * BM) * 2;
+      r.woff = (int64_t)row0 * (int64_t)p.K * 2 + (int64_t)r.t.tn * BN * 2;
+    } else if (WGRAD) {
       r.t.row0 = g * N; r.t.rows = N;
       const int b0 = uni(sh.tile_off[g]);
       r.KT = uni(sh.tile_off[g + 1]) - b0;
@@ -188,7 +210,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       r.t.row0 = uni(sh.row_off[g]);
       r.t.rows = uni(sh.row_off[g + 1]) - r.t.row0;
       r.KT = KT_fwd;
-      r.xoff = (int64_t)(r.t.row0 + r.t.tm * BM) * KROW;
+      r.xoff = (int64_t)(r.t.row0 + r.t.tm * BM) * XPITCH + (OP == OP_BF16_NT ? (int64_t)g * p.x_col_block * 2 : 0);
       if (WNT) r.woff = ((int64_t)g * p.K * N + r.t.tn * TILE_COLS) * 2;  // w[g][0][n0]
       else r.woff = ((int64_t)g * N + r.t.tn * TILE_COLS) * KROW;
     }
@@ -219,6 +241,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const MoeGgTile& t = tr.t;
     const int m0 = t.tm * BM, n0 = t.tn * TILE_COLS;
     c.KT = tr.KT;
+    c.rows_g = tr.rows_g;
     c.x_last = min(t.rows - m0, BM) - 1;
     c.w_last = min(NCOLS - n0, TILE_COLS) - 1;  // SWIGLU: last valid output column of the tile
     c.xg = uni_ptr(xp + tr.xoff);
@@ -237,15 +260,29 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     }
   };
   // Block b (8 rows) of the cursor slab's activation / weight rows.
+  // WGRAD_DIRECT: what group 0 has to zero in the slab it loaded last: rows zf_valid .. 63 of stage zf_stage.
+  int zf_valid = 64, zf_stage = 0;
   auto dma_x = [&](int b) {
+    if (WG2) {
+      // As the weight slab of OP_BF16_NT (see dma_w): block b = rows 4 (b & 15) .. + 3 of the slab's 64 rows of
+      // dY, column half b >> 4. Rows beyond the expert's last one re-read it.
+      const int bb = b & 15;
+      const uint32_t sw = (uint32_t)((lane >> 4) | (((bb >> 1) & 1) << 2));
+      const uint32_t chunk = (uint32_t)min((int)(((b >> 4) << 4) + ((lane & 15) ^ (sw << 1))), c.x_last >> 3);
+      const int rlast = max(c.rows_g - 1 - c.kt * 64, 0);
+      const uint32_t off = mad24((uint32_t)min(bb * 4 + (lane >> 4), rlast), XPITCH, chunk << 4);
+      dma16(c.xg + (int64_t)c.kt * (64 * (int64_t)XPITCH), off, lds_base + (c.step & 1) * STAGE + b * 1024);
+      return;
+    }
     if (b * 8 > c.x_last) return;  // block entirely below the tile's last row: its fragments are never used
-    const uint32_t off = mad24((uint32_t)min(b * 8 + d_r, c.x_last), KROW, d_c16);
+    const uint32_t off = mad24((uint32_t)min(b * 8 + d_r, c.x_last), XPITCH, d_c16);
     dma16(c.xg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + b * 1024);
   };
   // Weight rows: of the cursor slab, or (prev) of the slab before it, whose state group 1 keeps in wp_*.
   const char* wp_wg = nullptr;
   int wp_last = 0, wp_kt = 0, wp_step = 0;
-  const uint32_t WROW = (uint32_t)N * 2u;  // OP_BF16_NT: bytes per weight row (one r, all columns)
+  const uint32_t WROW = (uint32_t)(WG2 ? p.K : N) * 2u;  // slab layouts of OP_BF16_NT: bytes per weight row
+  int wp_rows_g = 0;
   auto dma_w = [&](int b, bool prev) {
     const int w_last = prev ? wp_last : c.w_last;
     if (WNT) {
@@ -255,7 +292,9 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       const int bb = b & 15;
       const uint32_t sw = (uint32_t)((lane >> 4) | (((bb >> 1) & 1) << 2));
       const uint32_t chunk = (uint32_t)min((int)(((b >> 4) << 4) + ((lane & 15) ^ (sw << 1))), w_last >> 3);
-      const uint32_t off = mad24((uint32_t)(bb * 4 + (lane >> 4)), WROW, chunk << 4);
+      int r = bb * 4 + (lane >> 4);
+      if (WG2) r = min(r, max((prev ? wp_rows_g : c.rows_g) - 1 - (prev ? wp_kt : c.kt) * 64, 0));
+      const uint32_t off = mad24((uint32_t)r, WROW, chunk << 4);
       dma16((prev ? wp_wg : c.wg) + (int64_t)(prev ? wp_kt : c.kt) * (64 * (int64_t)WROW), off,
             lds_base + ((prev ? wp_step : c.step) & 1) * STAGE + X_BYTES + b * 1024);
       return;
@@ -267,7 +306,21 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     dma16((prev ? wp_wg : c.wg) + (prev ? wp_kt : c.kt) * 128, off,
           lds_base + ((prev ? wp_step : c.step) & 1) * STAGE + X_BYTES + b * 1024);
   };
-  auto keep_prev = [&]() { wp_wg = c.wg; wp_last = c.w_last; wp_kt = c.kt; wp_step = c.step; };
+  auto keep_prev = [&]() { wp_wg = c.wg; wp_last = c.w_last; wp_kt = c.kt; wp_step = c.step; wp_rows_g = c.rows_g; };
+  // WGRAD_DIRECT, group 0, after its loads have landed: zero the rows of the dY slab that lie beyond the expert's
+  // last row (only the last K step of a tile has any). Every wave clears the blocks it loaded itself.
+  auto zero_fill = [&]() {
+    if (!WG2 || GRP != 0) return;
+    if (zf_valid < 64) {
+#pragma unroll
+      for (int idx = 0; idx < 8; ++idx) {
+        const int b = idx * 4 + gw;
+        if ((b & 15) * 4 + (lane >> 4) >= zf_valid)
+          *(u32x4_t*)(sh.lds + zf_stage * STAGE + b * 1024 + lane * 16) = u32x4_t{0u, 0u, 0u, 0u};
+      }
+      wait_lgkm0();
+    }
+  };
   // Block scales of the cursor slab: wave gw of group 0 fetches the activation scales of rows
   // 64 gw .. 64 gw + 63 (one per lane) and a private copy of the two weight-block scales (lanes 0-31 the
   // first column block, lanes 32-63 the second).
@@ -296,6 +349,10 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     }
     if (idx == NDMA - 1) {
       if (GRP == 1) keep_prev();
+      if (WG2 && GRP == 0) {
+        zf_valid = c.kt == c.KT - 1 ? c.rows_g - c.kt * 64 : 64;
+        zf_stage = c.step & 1;
+      }
       cursor_next();
     }
   };
@@ -313,6 +370,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     cursor_next();
   }
   wait_vm<0>();
+  zero_fill();
   __syncthreads();
   if (GRP == 1) {
 #pragma unroll
@@ -354,10 +412,26 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         u32x4_t wf[2][FN], xf[2][FM];
         // OP_BF16_NT: the lane's address inside the wave's column half for fragment f: row block of its k quarter, row
         // lane % 16 / 4 of a 4-row block, swizzled 32-byte column block, 8-byte piece lane % 4.
+        // The swizzle term of the lane (bits 5-7) is folded into one per-step base; a fragment's column block is an
+        // XOR on those bits. The base passes through an empty asm so that the addresses are formed here, per step,
+        // and not kept in registers across the K loop.
+        const int tr_ti = (lane & 15) >> 2, tr_ts = tr_ti | ((fq & 1) << 2);
+        uint32_t tr_base = lds_base + (uint32_t)((step & 1) * STAGE + fq * 2048 + tr_ti * 256 + (tr_ts << 5) + (lane & 3) * 8);
+        asm volatile("" : "+v"(tr_base));
         auto wt_addr = [&](int f) {
-          const int ti = (lane & 15) >> 2, ts = ti | ((fq & 1) << 2);
-          return lds_base + (uint32_t)((step & 1) * STAGE + X_BYTES + (wn >> 1) * 16384 + fq * 2048 + ti * 256 +
-                                       (((((wn & 1) << 2) + f) ^ ts) << 5) + (lane & 3) * 8);
+          return (tr_base ^ (uint32_t)((((wn & 1) << 2) + f) << 5)) + (uint32_t)(X_BYTES + (wn >> 1) * 16384);
+        };
+        // WGRAD_DIRECT: the same for activation fragment i: tile row block 2 i + wm = column block (2 i + wm) % 8 of
+        // half i / 4 of the dY slab.
+        auto xt_addr = [&](int i) {
+          return (tr_base ^ (uint32_t)((((i & 3) << 1) + wm) << 5)) + (uint32_t)((i >> 2) * 16384);
+        };
+        auto tr_pair = [&](uint32_t a) {
+          typedef __attribute__((address_space(3))) i16x4_t* lds_i16x4_ptr;
+          const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)a);
+          const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)(a + 1024));
+          const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
+          return u32x4_t{l2[0], l2[1], h2[0], h2[1]};
         };
         int issued = 0;
 #pragma unroll
@@ -372,14 +446,9 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
           }
           const int kk = q / 12, f = q % 12;
           const int ro = kk ? (rd0 ^ 64) : rd0;
-          if (f < FN && WNT) {
-            typedef __attribute__((address_space(3))) i16x4_t* lds_i16x4_ptr;
-            const uint32_t a = wt_addr(f) + kk * 8192;
-            const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)a);
-            const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(uintptr_t)(a + 1024));
-            const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
-            wf[kk][f] = u32x4_t{l2[0], l2[1], h2[0], h2[1]};
-          } else if (f < FN) wf[kk][f] = *(const u32x4_t*)(ws + f * 2048 + ro);
+          if (f < FN && WNT) wf[kk][f] = tr_pair(wt_addr(f) + kk * 8192);
+          else if (f < FN) wf[kk][f] = *(const u32x4_t*)(ws + f * 2048 + ro);
+          else if (WG2) xf[kk][f - FN] = tr_pair(xt_addr(f - FN) + kk * 8192);
           else xf[kk][f - FN] = *(const u32x4_t*)(xs + (f - FN) * (WM * 2048) + ro);
         }
         float sc[FM];
@@ -436,6 +505,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
         wait_vm<0>();  // group 0: X(step + 1); group 1: W1(step + 1), W0(step + 2); issued in this step's load phase
+        zero_fill();
         __syncthreads();
       }
 
@@ -444,7 +514,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       // 32-bit lane offset. The lane indices pass through an empty asm so that the address arithmetic
       // is redone here for every tile instead of being hoisted out of the tile loop, where it would
       // occupy (and spill) registers during the K loop.
-      bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + (WGRAD ? 0 : (int64_t)t.g * p.col_block) + n0;
+      bf16_t* yg = yp + (int64_t)(t.row0 + m0) * p.ldy + ((WGRAD || WG2) ? 0 : (int64_t)t.g * p.col_block) + n0;
       int er = fr, eq = fq;
       asm volatile("" : "+v"(er), "+v"(eq));
       // Row-wise fp8 scales (groupgemm.py:374-384): y *= x_scale[m] * w_scale[g * N + n].
@@ -547,7 +617,10 @@ DEVINL void pingpong_body(const GgParams& p) {
   __shared__ int32_t part_off[MOE_GG_MAX_GROUPS + 1];
 
   int total, total_low = 0;
-  if (OP == OP_BF16_WGRAD) {
+  if (OP == OP_BF16_WGRAD_DIRECT) {
+    build_row_offsets(p.m_sizes, p.G, p.M, row_off);
+    total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
+  } else if (OP == OP_BF16_WGRAD) {
     // tile_off counts the 64-column blocks of the padded operands (at least one per expert).
     build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
     total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
@@ -577,7 +650,7 @@ DEVINL void pingpong_body(const GgParams& p) {
   for (int i = threadIdx.x; i < n_my; i += NT) {
     const int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
     int g, tm, tn;
-    if (OP == OP_BF16_WGRAD) {
+    if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
       const int ntm = moe_gg_cdiv(p.N, BM), tpg = ntm * moe_gg_cdiv(p.K, BN);
       g = L / tpg;
       const int rem = L - g * tpg;
@@ -608,6 +681,7 @@ __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_bo
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_nt(GgParams p) { pingpong_body<OP_BF16_NT>(p); }
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad_direct(GgParams p) { pingpong_body<OP_BF16_WGRAD_DIRECT>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise(GgParams p) { pingpong_body<OP_FP8_ROW>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpong_body<OP_FP8_BLOCK>(p); }
 
@@ -630,6 +704,11 @@ hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStre
 
 hipError_t gg_bf16_pingpong_nt_launch(const GgParams& p, int num_wg, hipStream_t stream) {
   hipLaunchKernelGGL(gg_bf16_pingpong_nt, dim3(num_wg), dim3(NT), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t gg_bf16_pingpong_wgrad_direct_launch(const GgParams& p, int num_wg, hipStream_t stream) {
+  hipLaunchKernelGGL(gg_bf16_pingpong_wgrad_direct, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
 

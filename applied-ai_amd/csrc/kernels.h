@@ -19,6 +19,8 @@ struct GgParams {
   int vec_store;  // 1 when 8-byte aligned row segments can be stored as one dwordx2
   int xcds;       // number of XCDs the persistent grid is spread over
   int skip_rows;  // tiled fp8 kernel: experts with at most this many rows are left to the streaming kernel
+  int ldx;          // gg_bf16_pingpong_nt / _wgrad_direct: leading dimension of x (the output gradient)
+  int x_col_block;  // gg_bf16_pingpong_nt / _wgrad_direct: expert g reads x at column offset g * x_col_block
 };
 
 // block_m in {256, 128, 64}; the matching tile width is gg_bf16_tiled_block_n(block_m).
@@ -85,9 +87,13 @@ hipError_t compact_block_launch(const void* src, void* dst, const int32_t* m_siz
                                 int col_block, hipStream_t stream);
 // y [M, n] = silu(x w_gate^T) * (x w_up^T) with w [G * 2n, K] (gate rows first); p.N = 2n, p.ldy >= n, p.col_block unused.
 hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream);
-// y [M, N] = x [M, K] times w[g] [K, N] (weights row-major along N, not along the reduction): p.w = [G * K, N].
-// K % 64 == 0, N % 8 == 0.
+// y [M, N] = x [M, K] times w[g] [K, N] (weights row-major along N, not along the reduction): p.w = [G * K, N];
+// x has leading dimension p.ldx and expert g reads it at column offset g * p.x_col_block. K % 64 == 0, N % 8 == 0.
 hipError_t gg_bf16_pingpong_nt_launch(const GgParams& p, int num_wg, hipStream_t stream);
+// dW[g] [N, K] = dY_g^T X_g read from the operands as stored: p.x = dY [M, ldx] (expert g at column offset
+// g * x_col_block), p.w = X [M, K], p.M = number of rows, p.y = dW [G * N, K], p.ldy = K. N % 8 == 0, K % 8 == 0,
+// ldx % 8 == 0.
+hipError_t gg_bf16_pingpong_wgrad_direct_launch(const GgParams& p, int num_wg, hipStream_t stream);
 hipError_t gg_bf16_pingpong_wgrad_launch(const GgParams& p, int num_wg, hipStream_t stream);
 // dW = dY^T X per expert on the transposed, padded operands; p.x = dY^T [N, ldm], p.w = X^T [K, ldm], p.M = ldm,
 // p.skip_rows = number of gradient rows (bound for m_sizes), p.y = dW [G * N, K] with p.ldy = K. block in {256, 128}.

@@ -153,7 +153,8 @@ int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int
  *   (zeros for an expert without rows).
  *   workspace: device scratch of at least moe_gg_grouped_gemm_backward_workspace(...) bytes, 256-byte aligned,
  *   owned by the caller (the library never allocates); it holds w^T and the transposed, zero-padded copies of
- *   grad_out and x that make every operand contiguous along its reduction dimension.
+ *   grad_out and x that make every operand contiguous along its reduction dimension. Large calls read the
+ *   operands as stored and leave the workspace untouched.
  * Requires N % 4 == 0 and K % 4 == 0; N % 64 == 0 for the fast grad_x kernels.
  */
 size_t moe_gg_grouped_gemm_backward_workspace(int G, int64_t M, int N, int K, int grad_layout);

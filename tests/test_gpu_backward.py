@@ -115,17 +115,22 @@ def test_errors():
     ([513, 255, 1, 0, 700, 128, 64, 1290], 3000, 256, 3080),    # partial column tiles (K % 256 = 8), ragged rows
     ([1012, 1039, 1048, 1036], 4160, 1024, 4096),
     ([300] * 8, 2400, 512, 512),                                # too few tiles: both runs take the transposed copy
+    # 48 experts, ragged (empty ones, single rows, sizes around multiples of 64), N and K with partial tiles:
+    # grad_w comes from dY and x as stored (enough tiles of grad_w), grad_x from the transposed copy
+    ([0, 1, 63, 64, 65, 127, 128, 129, 200, 0, 31, 257] * 4, 5400, 264, 520),
 ])
-def test_grad_x_from_untransposed_weights_equals_the_transposed_copy_path(sizes, M, N, K):
-    """With enough tiles grad_x comes from the kernel that reads w as stored (transposing LDS reads); pinning a
-    kernel variant selects the path through a transposed copy of w. Same products, same accumulation order per
-    tile: bit-identical, and both within the bar of the oracle (run_case)."""
+def test_gradients_from_operands_as_stored_equal_the_transposed_copy_paths(sizes, M, N, K):
+    """With enough tiles the gradients come from the kernels that read w, dY and x as stored (transposing LDS
+    reads); pinning a kernel variant selects the paths through transposed copies in the workspace. Same products,
+    same accumulation order per tile: bit-identical, and both within the bar of the oracle (run_case)."""
     import applied_ai_amd as A
     from applied_ai_amd import _lib
 
-    if K > 512:
+    if K > 520:
         # the library's rule for the direct kernel on a 256-CU part: enough 256 x 256 tiles of grad_x
         assert (M // 256 + (len(sizes) + 1) // 2) * ((K + 255) // 256) * 4 >= 256 * 3
+    if K == 520:
+        assert len(sizes) * ((N + 255) // 256) * ((K + 255) // 256) * 4 >= 256 * 3   # same rule for grad_w
     gx_nt, gw_nt = run_case(sizes, M, N, K, seed=33, scale=0.5)
     L = _lib.lib()
     try:
