@@ -504,7 +504,10 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         }
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
-        wait_vm<0>();  // group 0: X(step + 1); group 1: W1(step + 1), W0(step + 2); issued in this step's load phase
+        // Group 0: X(step + 1), issued in this step's load phase, is read in the next phase. Group 1: of its loads of
+        // this step's load phase only W1(step + 1), issued first, is read that soon; the four W0(step + 2) loads may
+        // stay in flight until the end of its next load phase (the wait there leaves only that phase's own loads).
+        if (GRP == 0) wait_vm<0>(); else wait_vm<4>();
         zero_fill();
         __syncthreads();
       }
