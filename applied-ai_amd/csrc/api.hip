@@ -38,6 +38,14 @@ int current_device_info(const DeviceInfo** out) {
 
 bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
+// How wide the kernels may store row segments of y: 2 = 16 bytes, 1 = 8 bytes, 0 = element by element. col_step
+// is the distance between the column offsets the call may add (N for the per-expert column blocks, else 0).
+int vec_store_level(const void* y, int64_t ldy, int64_t col_step) {
+  if (aligned(y, 16) && ldy % 8 == 0 && col_step % 8 == 0) return 2;
+  if (aligned(y, 8) && ldy % 4 == 0 && col_step % 4 == 0) return 1;
+  return 0;
+}
+
 // fp8: the dedicated small-M kernel (weights streamed straight into MFMA operands, split-K inside the workgroup)
 // beats the ping-pong kernel only for a few rows per expert (measured: up to about 12) or when the launch has
 // too few 256 x 256 tiles to give every CU several (few experts, narrow N); never above 40 rows per expert.
@@ -101,7 +109,7 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
   p.G = G; p.M = (int)M; p.N = N; p.K = K;
   p.ldy = (int)ldy;
   p.col_block = out_layout == MOE_GG_OUT_BLOCK ? N : 0;
-  p.vec_store = aligned(y, 8) && ldy % 4 == 0 && N % 4 == 0;
+  p.vec_store = vec_store_level(y, ldy, N);
   p.xcds = di->xcds;
 
   hipStream_t s = (hipStream_t)stream;
@@ -173,7 +181,7 @@ int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* 
   p.G = G; p.M = (int)M; p.N = N; p.K = K;
   p.ldy = (int)ldy;
   p.col_block = out_layout == MOE_GG_OUT_BLOCK ? N : 0;
-  p.vec_store = aligned(y, 8) && ldy % 4 == 0 && N % 4 == 0;
+  p.vec_store = vec_store_level(y, ldy, N);
   p.xcds = di->xcds;
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
@@ -286,7 +294,7 @@ int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const
   p.x = x; p.w = w; p.y = y; p.m_sizes = m_sizes;
   p.G = G; p.M = (int)M; p.N = 2 * n; p.K = K;
   p.ldy = (int)ldy;
-  p.vec_store = aligned(y, 8) && ldy % 4 == 0;
+  p.vec_store = vec_store_level(y, ldy, 0);
   p.xcds = di->xcds;
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
@@ -363,7 +371,7 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
       q.G = G; q.M = (int)M; q.N = K; q.K = N;
       q.ldy = K;
       q.ldx = (int)ld_go; q.x_col_block = x_col_block;
-      q.vec_store = aligned(grad_x, 8) && K % 4 == 0;
+      q.vec_store = vec_store_level(grad_x, K, 0);
       q.xcds = xcds;
       e = gg_bf16_pingpong_nt_launch(q, num_wg, s);
       if (e != hipSuccess) return (int)e;
@@ -390,7 +398,7 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
     q.G = G; q.M = (int)M; q.N = N; q.K = K;
     q.ldy = K;
     q.ldx = (int)ld_go; q.x_col_block = x_col_block;
-    q.vec_store = aligned(grad_w, 8) && K % 4 == 0;
+    q.vec_store = vec_store_level(grad_w, K, 0);
     q.xcds = xcds;
     return (int)gg_bf16_pingpong_wgrad_direct_launch(q, num_wg, s);
   }
@@ -406,7 +414,7 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   p.G = G; p.M = (int)ldm; p.N = N; p.K = K;
   p.ldy = K;
   p.col_block = 0;
-  p.vec_store = aligned(grad_w, 8) && K % 4 == 0;
+  p.vec_store = vec_store_level(grad_w, K, 0);
   p.xcds = xcds;
   p.skip_rows = (int)M;
   if (v == MOE_GG_GG_TILED_256) return (int)gg_bf16_wgrad_launch(p, 256, num_wg, s);

@@ -570,6 +570,25 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
           if (mrow + er < rows_valid) {
             float am = 1.f;
             if (OP == OP_FP8_ROW) am = xrow_scale[mrow + er];
+            if (p.vec_store == 2) {
+            // Lanes l and l ^ 16 (column quarters 2q, 2q + 1 of the same row) trade halves so that each stores 16
+            // bytes: the even one columns 8 q' .. + 7 of fragment j, the odd one those of fragment j + 1.
+#pragma unroll
+            for (int j = 0; j < FN; j += 2) {
+              f32x4_t v0 = acc[j][i], v1 = acc[j + 1][i];
+              if (OP == OP_FP8_ROW) { v0 = v0 * am * bs[j]; v1 = v1 * am * bs[j + 1]; }
+              const uint32_t a0 = pack_bf16x2(v0[0], v0[1]), a1 = pack_bf16x2(v0[2], v0[3]);
+              const uint32_t b0 = pack_bf16x2(v1[0], v1[1]), b1 = pack_bf16x2(v1[2], v1[3]);
+              const bool odd = eq & 1;
+              const uint32_t s0 = odd ? a0 : b0, s1 = odd ? a1 : b1;   // what the partner stores
+              const uint32_t r0 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)s0, 0x401F);  // lane ^ 16
+              const uint32_t r1 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)s1, 0x401F);
+              u32x4_t o;
+              if (odd) o = u32x4_t{r0, r1, b0, b1}; else o = u32x4_t{a0, a1, r0, r1};
+              // even: fragment j, columns 16 j + 4 eq .. + 7; odd: fragment j + 1, columns 16 (j + 1) + 4 (eq - 1) ..
+              *(u32x4_t*)(ybase + voff + (odd ? (j + 1) * 16 - 4 : j * 16)) = o;
+            }
+            } else {
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
               f32x4_t v = acc[j][i];
@@ -578,6 +597,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
               o[0] = pack_bf16x2(v[0], v[1]);
               o[1] = pack_bf16x2(v[2], v[3]);
               *(u32x2_t*)(ybase + voff + j * 16) = o;
+            }
             }
           }
         }

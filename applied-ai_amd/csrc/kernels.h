@@ -16,7 +16,7 @@ struct GgParams {
   int G, M, N, K;
   int ldy;
   int col_block;
-  int vec_store;  // 1 when 8-byte aligned row segments can be stored as one dwordx2
+  int vec_store;  // 1: 8-byte aligned row segments can be stored as one dwordx2; 2: also 16-byte ones as dwordx4
   int xcds;       // number of XCDs the persistent grid is spread over
   int skip_rows;  // tiled fp8 kernel: experts with at most this many rows are left to the streaming kernel
   int ldx;          // gg_bf16_pingpong_nt / _wgrad_direct: leading dimension of x (the output gradient)
