@@ -530,9 +530,9 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
           const int m = (i * WM + wm) * 16 + er;
           if (m < rows_valid) {
             bf16_t* yrow = yg + (int64_t)m * p.ldy;
+            u32x2_t q[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-              const int n = wn * 32 + j * 16 + eq * 4;
               const f32x4_t gv = acc[j][i], uv = acc[j + 2][i];
               const uint32_t g01 = pack_bf16x2(gv[0], gv[1]), g23 = pack_bf16x2(gv[2], gv[3]);
               const uint32_t u01 = pack_bf16x2(uv[0], uv[1]), u23 = pack_bf16x2(uv[2], uv[3]);
@@ -543,15 +543,31 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
               float o[4];
 #pragma unroll
               for (int rr = 0; rr < 4; ++rr) o[rr] = g[rr] / (1.f + __expf(-g[rr])) * u[rr];
-              if (p.vec_store && n + 3 < cols_valid) {
-                u32x2_t q;
-                q[0] = pack_bf16x2(o[0], o[1]);
-                q[1] = pack_bf16x2(o[2], o[3]);
-                *(u32x2_t*)(yrow + n) = q;
-              } else {
+              q[j][0] = pack_bf16x2(o[0], o[1]);
+              q[j][1] = pack_bf16x2(o[2], o[3]);
+            }
+            if (p.vec_store == 2 && cols_valid == TILE_COLS) {
+              // 16-byte stores: lanes l and l ^ 16 trade halves as in the plain epilogue below.
+              const bool odd = eq & 1;
+              const uint32_t r0 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)(odd ? q[0][0] : q[1][0]), 0x401F);
+              const uint32_t r1 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)(odd ? q[0][1] : q[1][1]), 0x401F);
+              u32x4_t o4;
+              if (odd) o4 = u32x4_t{r0, r1, q[1][0], q[1][1]}; else o4 = u32x4_t{q[0][0], q[0][1], r0, r1};
+              *(u32x4_t*)(yrow + wn * 32 + eq * 4 + (odd ? 16 - 4 : 0)) = o4;
+            } else {
 #pragma unroll
-                for (int rr = 0; rr < 4; ++rr)
-                  if (n + rr < cols_valid) yrow[n + rr] = (bf16_t)o[rr];
+              for (int j = 0; j < 2; ++j) {
+                const int n = wn * 32 + j * 16 + eq * 4;
+                if (p.vec_store && n + 3 < cols_valid) {
+                  *(u32x2_t*)(yrow + n) = q[j];
+                } else {
+#pragma unroll
+                  for (int rr = 0; rr < 4; ++rr)
+                    if (n + rr < cols_valid) {
+                      const uint32_t w2 = q[j][rr >> 1];
+                      ((uint16_t*)yrow)[n + rr] = (uint16_t)((rr & 1) ? (w2 >> 16) : (w2 & 0xFFFFu));
+                    }
+                }
               }
             }
           }
