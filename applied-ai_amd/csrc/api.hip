@@ -494,7 +494,7 @@ int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, i
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                           int block_n, int num_workgroups, int xcds, int32_t* out,
                                           int max_tiles) {
-  if (!m_sizes_host || !out || G <= 0 || G > MOE_GG_MAX_GROUPS_ABI || block_m <= 0 || block_n <= 0 ||
+  if (!m_sizes_host || !out || G <= 0 || G > MOE_GG_MAX_GROUPS_ABI || block_m != 256 || block_n <= 0 ||
       num_workgroups <= 0 || xcds <= 0 || num_workgroups % xcds != 0 || M < 0 || N <= 0)
     return MOE_GG_EINVAL;
   static thread_local int32_t row_off[MOE_GG_MAX_GROUPS_ABI + 1], long_off[MOE_GG_MAX_GROUPS_ABI + 1],
@@ -510,33 +510,49 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     ns += moe_gg_low_row_tiles(m, block_m) * ntn;
   }
   row_off[G] = (int32_t)r; long_off[G] = nl; low_off[G] = ns;
-  const int total = nl + ns;
+  const int tail_s = moe_gg_tail_pieces(nl, num_workgroups);
+  const int tail_first = moe_gg_tail_first(nl, num_workgroups);
+  const int long_ids = moe_gg_long_ids(nl, num_workgroups);
+  const int total = long_ids + ns;
   int written = 0;
   for (int wg = 0; wg < num_workgroups; ++wg) {
     int n_long = 0, n_low = 0;
-    while (n_long * num_workgroups < nl && moe_gg_tile_of(wg, num_workgroups, xcds, n_long) < nl) ++n_long;
+    while (n_long * num_workgroups < long_ids && moe_gg_tile_of(wg, num_workgroups, xcds, n_long) < long_ids) ++n_long;
     while ((n_long + n_low) * num_workgroups < total && moe_gg_tile_of(wg, num_workgroups, xcds, n_long + n_low) < total) ++n_low;
     const int n_my = n_long + n_low, phase = moe_gg_low_phase(wg, xcds);
     for (int seq = 0; seq < n_my; ++seq) {
-      const int L = moe_gg_tile_of(wg, num_workgroups, xcds, moe_gg_seq_round(seq, n_my, n_low, phase));
-      const bool low = L >= nl;
+      int L = moe_gg_tile_of(wg, num_workgroups, xcds, moe_gg_seq_round(seq, n_my, n_low, phase));
       if (written >= max_tiles) return written;
-      int g, tm, tn;
-      if (!low) {
-        if (L >= nl) return MOE_GG_EINVAL;  // cannot happen: a long position maps to a long tile id
+      int g, m0, h, tn;
+      if (L < long_ids) {
+        int piece = 0;
+        if (L >= tail_first) {
+          piece = (L - tail_first) % tail_s;
+          L = tail_first + (L - tail_first) / tail_s;
+        }
         g = moe_gg_find_group(long_off, G, L);
         const int idx = L - long_off[g];
-        const int nf = moe_gg_long_row_tiles(row_off[g + 1] - row_off[g], block_m);
-        tn = idx / nf; tm = idx - tn * nf;
+        const int rows = row_off[g + 1] - row_off[g];
+        const int nf = moe_gg_long_row_tiles(rows, block_m);
+        tn = idx / nf;
+        m0 = (idx - tn * nf) * block_m;
+        h = rows - m0 < block_m ? rows - m0 : block_m;
+        if (tail_s > 1 && L >= tail_first) {
+          int off;
+          moe_gg_piece_rows(h, tail_s, piece, &off, &h);
+          m0 += off;
+        }
       } else {
-        const int Lp = L - nl;
-        if (Lp < 0 || Lp >= ns) return MOE_GG_EINVAL;
+        const int Lp = L - long_ids;
+        if (Lp >= ns) return MOE_GG_EINVAL;  // cannot happen
         g = moe_gg_find_group(low_off, G, Lp);
         tn = Lp - low_off[g];
-        tm = (row_off[g + 1] - row_off[g]) / block_m;
+        const int rows = row_off[g + 1] - row_off[g];
+        m0 = rows / block_m * block_m;
+        h = rows - m0;
       }
       int32_t* o = out + (size_t)written * 5;
-      o[0] = wg; o[1] = g; o[2] = tm; o[3] = tn; o[4] = row_off[g];
+      o[0] = wg; o[1] = g; o[2] = m0; o[3] = h; o[4] = tn;
       ++written;
     }
   }

@@ -178,17 +178,20 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   const int nwg = gridDim.x;
   // Tile of a round. Forward: rows of x / rows of w[g]. WGRAD: rows of dY^T (n) / rows of X^T (k), both at the
   // column offset of the expert's padded block; t.row0 = first row of the expert's block of dW, t.rows = N.
-  struct TileRef { MoeGgTile t; int KT, rows_g; int64_t xoff, woff; };
+  struct TileRef { MoeGgTile t; int KT, rows_g, m0, h; int64_t xoff, woff; };  // m0, h: first row inside the group, rows
   // The workgroup's own sequence (moe_gg_seq_round): its long tiles in round order with its low tiles spread
   // evenly between them, at a phase that differs between XCDs, so that memory-bound low tiles and compute-bound
   // long tiles run side by side on the chip, while the workgroups of one XCD take theirs together and stay in
   // step. Tile ids: long tiles 0 .. n_long - 1, then the low tiles.
   auto tile_ref = [&](int seq) {
     TileRef r;
-    // Decoded in the prologue: group, row tile | column tile << 16.
-    const int g = uni(sh.seq_tab[2 * seq]);
+    // Decoded in the prologue: group | rows << 16, first row / 64 | column tile << 16.
+    const int gh = uni(sh.seq_tab[2 * seq]);
     const int mn = uni(sh.seq_tab[2 * seq + 1]);
-    r.t.g = g; r.t.tm = mn & 0xFFFF; r.t.tn = (int)((uint32_t)mn >> 16);
+    const int g = gh & 0xFFFF;
+    r.h = (int)((uint32_t)gh >> 16);
+    r.m0 = (mn & 0xFFFF) * 64;
+    r.t.g = g; r.t.tm = 0; r.t.tn = (int)((uint32_t)mn >> 16);
     r.rows_g = 0;
     if (WG2) {
       // Output: rows tm * 256 .. of the expert's block of dW (n), columns tn * 256 .. (k). Operands: the expert's
@@ -198,19 +201,19 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       if (r.rows_g == 0) row0 = min(row0, p.M - 1);  // an expert without rows: one K step of zeros, loads in bounds
       r.t.row0 = g * N; r.t.rows = N;
       r.KT = max(1, moe_gg_cdiv(r.rows_g, 64));
-      r.xoff = (int64_t)row0 * XPITCH + ((int64_t)g * p.x_col_block + r.t.tm * BM) * 2;
+      r.xoff = (int64_t)row0 * XPITCH + ((int64_t)g * p.x_col_block + r.m0) * 2;
       r.woff = (int64_t)row0 * (int64_t)p.K * 2 + (int64_t)r.t.tn * BN * 2;
     } else if (WGRAD) {
       r.t.row0 = g * N; r.t.rows = N;
       const int b0 = uni(sh.tile_off[g]);
       r.KT = uni(sh.tile_off[g + 1]) - b0;
-      r.xoff = (int64_t)(r.t.tm * BM) * KROW + (int64_t)b0 * 128;
+      r.xoff = (int64_t)r.m0 * KROW + (int64_t)b0 * 128;
       r.woff = (int64_t)(r.t.tn * BN) * KROW + (int64_t)b0 * 128;
     } else {
       r.t.row0 = uni(sh.row_off[g]);
       r.t.rows = uni(sh.row_off[g + 1]) - r.t.row0;
       r.KT = KT_fwd;
-      r.xoff = (int64_t)(r.t.row0 + r.t.tm * BM) * XPITCH + (OP == OP_BF16_NT ? (int64_t)g * p.x_col_block * 2 : 0);
+      r.xoff = (int64_t)(r.t.row0 + r.m0) * XPITCH + (OP == OP_BF16_NT ? (int64_t)g * p.x_col_block * 2 : 0);
       if (WNT) r.woff = ((int64_t)g * p.K * N + r.t.tn * TILE_COLS) * 2;  // w[g][0][n0]
       else r.woff = ((int64_t)g * N + r.t.tn * TILE_COLS) * KROW;
     }
@@ -239,10 +242,10 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     if (round >= sh.n_my) return;  // past the last tile: keep re-loading the last tile (never read)
     const TileRef tr = tile_ref(round);
     const MoeGgTile& t = tr.t;
-    const int m0 = t.tm * BM, n0 = t.tn * TILE_COLS;
+    const int m0 = tr.m0, n0 = t.tn * TILE_COLS;
     c.KT = tr.KT;
     c.rows_g = tr.rows_g;
-    c.x_last = min(t.rows - m0, BM) - 1;
+    c.x_last = max(tr.h, 1) - 1;  // (a piece without rows loads row 0 and stores nothing)
     c.w_last = min(NCOLS - n0, TILE_COLS) - 1;  // SWIGLU: last valid output column of the tile
     c.xg = uni_ptr(xp + tr.xoff);
     c.wg = uni_ptr(wp + tr.woff);
@@ -385,8 +388,8 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const TileRef tr = tile_ref(r);
     const MoeGgTile& t = tr.t;
     const int KT = tr.KT;
-    const int m0 = t.tm * BM, n0 = t.tn * TILE_COLS;
-    const int rows_valid = min(t.rows - m0, BM);
+    const int m0 = tr.m0, n0 = t.tn * TILE_COLS;
+    const int rows_valid = tr.h;
     const int cols_valid = min(NCOLS - n0, TILE_COLS);
     // Activation fragments of this wave that hold at least one valid row (fragments are dealt
     // alternately to wm = 0 / 1, so a short tile shortens every wave's C phase alike).
@@ -674,9 +677,14 @@ DEVINL void pingpong_body(const GgParams& p) {
   }
   const int nwg = gridDim.x;
   // Tiles of this workgroup in each list: rounds 0 .. n - 1 (tile ids grow with the round).
+  // (Forward kernels: the long tiles of a sparsely filled last round are cut into row pieces, moe_gg_tail_pieces.)
+  const bool fwd = OP != OP_BF16_WGRAD && OP != OP_BF16_WGRAD_DIRECT;
+  const int tail_s = fwd ? moe_gg_tail_pieces(total, nwg) : 1;
+  const int tail_first = fwd ? moe_gg_tail_first(total, nwg) : total;
+  const int long_ids = fwd ? moe_gg_long_ids(total, nwg) : total;
   int n_long = 0, n_low = 0;
-  while (n_long * nwg < total && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < total) ++n_long;
-  while ((n_long + n_low) * nwg < total + total_low && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < total + total_low)
+  while (n_long * nwg < long_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < long_ids) ++n_long;
+  while ((n_long + n_low) * nwg < long_ids + total_low && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < long_ids + total_low)
     ++n_low;
   if (n_long + n_low == 0) return;
   // The sequence of this workgroup (moe_gg_seq_round), decoded once into a table: the arithmetic runs per thread
@@ -687,26 +695,43 @@ DEVINL void pingpong_body(const GgParams& p) {
   __shared__ int32_t seq_tab[2 * MOE_GG_SEQ_CAP];
   const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
   for (int i = threadIdx.x; i < n_my; i += NT) {
-    const int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
-    int g, tm, tn;
+    int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
+    int g, m0, h, tn;  // group, first row inside the group, rows, column tile
     if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
       const int ntm = moe_gg_cdiv(p.N, BM), tpg = ntm * moe_gg_cdiv(p.K, BN);
       g = L / tpg;
       const int rem = L - g * tpg;
-      tn = rem / ntm; tm = rem - tn * ntm;
-    } else if (L < total) {
+      tn = rem / ntm;
+      m0 = (rem - tn * ntm) * BM;
+      h = min(p.N - m0, BM);
+    } else if (L < long_ids) {
+      int piece = 0;
+      if (L >= tail_first) {  // a piece of a tile of the last round
+        piece = (L - tail_first) % tail_s;
+        L = tail_first + (L - tail_first) / tail_s;
+      }
       g = moe_gg_find_group(tile_off, p.G, L);
       const int idx = L - tile_off[g];
-      const int nf = moe_gg_long_row_tiles(row_off[g + 1] - row_off[g], BM);
-      tn = idx / nf; tm = idx - tn * nf;
+      const int rows = row_off[g + 1] - row_off[g];
+      const int nf = moe_gg_long_row_tiles(rows, BM);
+      tn = idx / nf;
+      m0 = (idx - tn * nf) * BM;
+      h = min(rows - m0, BM);
+      if (tail_s > 1 && L >= tail_first) {
+        int off;
+        moe_gg_piece_rows(h, tail_s, piece, &off, &h);
+        m0 += off;
+      }
     } else {
-      const int Lp = L - total;
+      const int Lp = L - long_ids;
       g = moe_gg_find_group(part_off, p.G, Lp);
       tn = Lp - part_off[g];
-      tm = (row_off[g + 1] - row_off[g]) / BM;
+      const int rows = row_off[g + 1] - row_off[g];
+      m0 = rows / BM * BM;
+      h = rows - m0;
     }
-    seq_tab[2 * i] = g;
-    seq_tab[2 * i + 1] = tm | (tn << 16);
+    seq_tab[2 * i] = g | (h << 16);
+    seq_tab[2 * i + 1] = (m0 / 64) | (tn << 16);
   }
   __syncthreads();
 

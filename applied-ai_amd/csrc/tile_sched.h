@@ -124,7 +124,34 @@ MOE_GG_HD int moe_gg_seq_round(int seq, int n_my, int n_low_my, int phase) {
   const bool low = moe_gg_low_before(seq + 1, n_my, n_low_my, phase) > lb;
   return low ? (n_my - n_low_my) + lb : seq - lb;
 }
-// Upper bound of the tile count: sum of ceil(m_g / BM) <= M / BM + G row tiles, times the column tiles.
+// Upper bound of the tile count: sum of ceil(m_g / BM) <= M / BM + G row tiles, times the column tiles (a last
+// round cut into pieces has at most num_wg ids). Row offsets inside a group are tabulated in units of 64 rows
+// in 16 bits.
 MOE_GG_HD bool moe_gg_two_list_fits(int64_t M, int G, int BM, int n_tiles_n, int num_wg) {
-  return (M / BM + G) * (int64_t)n_tiles_n <= (int64_t)(MOE_GG_SEQ_CAP - 1) * num_wg;
+  return M < (1 << 22) && (M / BM + G) * (int64_t)n_tiles_n <= (int64_t)(MOE_GG_SEQ_CAP - 2) * num_wg;
 }
+
+// Tail split. With n_long long tiles on num_wg workgroups the last round holds n_long % num_wg tiles; when it is
+// at most half full, each of its tiles is cut into 2 or 4 pieces of rows (multiples of 64) that different
+// workgroups compute, so the round takes about a half or a quarter as long (a piece loads its whole weight tile
+// but runs only its share of the MFMAs). Ids: 0 .. first - 1 whole tiles, then pieces: first + t * s + piece.
+MOE_GG_HD int moe_gg_tail_pieces(int n_long, int num_wg) {
+  const int tail = n_long % num_wg;
+  if (tail == 0 || tail * 2 > num_wg) return 1;
+  return tail * 4 <= num_wg ? 4 : 2;
+}
+MOE_GG_HD int moe_gg_tail_first(int n_long, int num_wg) {
+  return moe_gg_tail_pieces(n_long, num_wg) == 1 ? n_long : n_long - n_long % num_wg;
+}
+MOE_GG_HD int moe_gg_long_ids(int n_long, int num_wg) {
+  const int first = moe_gg_tail_first(n_long, num_wg);
+  return first + (n_long - first) * moe_gg_tail_pieces(n_long, num_wg);
+}
+// Piece p of s of a tile with rv valid rows (BM = 256): first row and number of rows (0 if the tile is too low).
+MOE_GG_HD void moe_gg_piece_rows(int rv, int s, int p, int* off, int* h) {
+  const int per = 256 / s;
+  *off = p * per;
+  const int left = rv - *off;
+  *h = left < 0 ? 0 : (left > per ? per : left);
+}
+

@@ -230,9 +230,10 @@ int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,
                                 int max_tiles);
-/* The same for the 256 x 256 ping-pong kernels (bf16, fp8 row-wise), which keep two tile lists (long tiles, low
- * tiles) and give every workgroup its low tiles spread between its long ones; the quintuples of a workgroup come
- * in the order in which it computes them. */
+/* The same for the 256 x 256 ping-pong kernels (block_m must be 256), which keep two tile lists (long tiles, low
+ * tiles), give every workgroup its low tiles spread between its long ones, and cut the long tiles of a sparsely
+ * filled last round into row pieces. Quintuples here: (workgroup, group, first row inside the group, rows,
+ * tile_n), for each workgroup in the order in which it computes them; a piece may have 0 rows. */
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                           int block_n, int num_workgroups, int xcds, int32_t* out,
                                           int max_tiles);

@@ -150,14 +150,16 @@ def test_scheduler_rejects_bad_arguments(lib):
 
 @pytest.mark.parametrize("m_sizes,N,nwg", [
     ([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], 14336, 256),   # Mixtral prefill: 4 experts end in a low tile
+    ([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], 4096, 256),    # 2.x rounds: the last one is cut into pieces
     ([25, 50, 25], 512, 8),                                          # only low tiles
     ([600, 0, 513, 255, 1, 2048 + 17], 1000, 16),
     ([700] * 40, 2048, 256),
     ([530], 256, 8),                                                 # fewer tiles than workgroups
 ])
 def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
-    """The ping-pong kernels' order: every (group, row tile, column tile) exactly once; a low tile has fewer than 128
-    rows and is the only row tile of its group or the last one of a group with at least two full tiles; every
+    """The ping-pong kernels' order: every output row of every group exactly once per column tile; a low tile has
+    fewer than 128 rows and is the only row tile of its group or the last one of a group with at least two full
+    tiles; the long tiles of a last round that is at most half full are cut into 2 or 4 row pieces; every
     workgroup gets the same number of tiles (+- 1), its low tiles spread through its sequence."""
     ms = np.ascontiguousarray(m_sizes, dtype=np.int32)
     M = int(ms.sum())
@@ -167,24 +169,41 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
                                                   out.ctypes.data_as(I32P), cap)
     assert n >= 0
     tiles = out[:n].tolist()
-    off = O.offsets(m_sizes)
-    expect = {(g, tm, tn) for g, m in enumerate(m_sizes) for tm in range(-(-m // 256)) for tn in range(-(-N // 256))}
-    got = [tuple(t[1:4]) for t in tiles]
-    assert len(got) == len(set(got)) == len(expect) and set(got) == expect
-    assert all(t[4] == off[t[1]] for t in tiles)
+    ntn = -(-N // 256)
+    # exact cover: per (group, column tile) the row ranges tile [0, m_g) without overlap
+    cover = {}
+    for wg, g, m0, h, tn in tiles:
+        assert 0 <= tn < ntn and m0 % 64 == 0 and 0 <= h <= 256 and m0 // 256 == (m0 + max(h, 1) - 1) // 256
+        cover.setdefault((g, tn), []).append((m0, h))
+    for g, m in enumerate(m_sizes):
+        for tn in range(ntn):
+            pieces = sorted(p for p in cover.get((g, tn), []) if p[1] > 0)
+            pos = 0
+            for m0, h in pieces:
+                assert m0 == pos, (g, tn, pieces)
+                pos += h
+            assert pos == m, (g, tn, pieces)
 
-    def is_low(g, tm):
+    def is_low(g, m0, h):
         m = m_sizes[g]
-        return tm == m // 256 and 0 < m % 256 < 128 and (m // 256 >= 2 or m // 256 == 0)
+        return m0 == m // 256 * 256 and h == m % 256 and 0 < h < 128 and (m // 256 >= 2 or m // 256 == 0)
 
     per_wg = {}
-    for wg, g, tm, tn, _ in tiles:
-        per_wg.setdefault(wg, []).append(is_low(g, tm))
+    for wg, g, m0, h, tn in tiles:
+        per_wg.setdefault(wg, []).append(is_low(g, m0, h))
     counts = [len(v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
     assert max(counts) - min(counts) <= 1
     lows = [sum(v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
     assert max(lows) - min(lows) <= 1
-    if m_sizes[0] == 1012:
+    # pieces: only when the last round of long tiles is at most half full; then 2 or 4 per tile
+    n_long = sum((m // 256 + (1 if (m % 256 >= 128 or (0 < m % 256 and m // 256 < 2 and m // 256 > 0)) else 0)) * ntn
+                 for m in m_sizes)
+    n_pieces = sum(1 for wg, g, m0, h, tn in tiles if not is_low(g, m0, h) and (h < min(256, m_sizes[g] - m0 // 256 * 256)
+                                                                               or m0 % 256))
+    tail = n_long % nwg
+    if tail == 0 or tail * 2 > nwg:
+        assert n_pieces == 0
+    if m_sizes[0] == 1012 and N == 14336:
         # 7 long tiles and at most one low tile per workgroup: the XCDs (wg % 8) take their low tile at 8 different
         # positions of the sequence, the workgroups of one XCD at the same one
         pos = {}
@@ -193,3 +212,6 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
                 pos.setdefault(wg % 8, set()).add(v.index(True))
         assert all(len(p) == 1 for p in pos.values())
         assert len(pos) == 7 and len({next(iter(p)) for p in pos.values()}) == 7   # 224 low tiles: 7 XCDs of 32
+    if m_sizes[0] == 1012 and N == 4096:
+        # 512 long tiles = 2 rounds and no tail; with the 64 low tiles nothing is cut
+        assert n_pieces == 0
