@@ -513,7 +513,8 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
   const int tail_s = moe_gg_tail_pieces(nl, num_workgroups);
   const int tail_first = moe_gg_tail_first(nl, num_workgroups);
   const int long_ids = moe_gg_long_ids(nl, num_workgroups);
-  const int total = long_ids + ns;
+  const int low_c = moe_gg_low_col_pieces(long_ids, ns, num_workgroups);
+  const int total = long_ids + ns * low_c;
   int written = 0;
   for (int wg = 0; wg < num_workgroups; ++wg) {
     int n_long = 0, n_low = 0;
@@ -523,7 +524,7 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     for (int seq = 0; seq < n_my; ++seq) {
       int L = moe_gg_tile_of(wg, num_workgroups, xcds, moe_gg_seq_round(seq, n_my, n_low, phase));
       if (written >= max_tiles) return written;
-      int g, m0, h, tn;
+      int g, m0, h, n0, nc = block_n;
       if (L < long_ids) {
         int piece = 0;
         if (L >= tail_first) {
@@ -534,25 +535,31 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
         const int idx = L - long_off[g];
         const int rows = row_off[g + 1] - row_off[g];
         const int nf = moe_gg_long_row_tiles(rows, block_m);
-        tn = idx / nf;
+        const int tn = idx / nf;
+        n0 = tn * block_n;
         m0 = (idx - tn * nf) * block_m;
         h = rows - m0 < block_m ? rows - m0 : block_m;
         if (tail_s > 1 && L >= tail_first) {
           int off;
           moe_gg_piece_rows(h, tail_s, piece, &off, &h);
-          m0 += off;
+          if (h > 0) m0 += off;
         }
       } else {
-        const int Lp = L - long_ids;
+        const int Lp = (L - long_ids) / low_c, piece = (L - long_ids) % low_c;
         if (Lp >= ns) return MOE_GG_EINVAL;  // cannot happen
         g = moe_gg_find_group(low_off, G, Lp);
-        tn = Lp - low_off[g];
+        nc = block_n / low_c;
+        n0 = (Lp - low_off[g]) * block_n + piece * nc;
         const int rows = row_off[g + 1] - row_off[g];
         m0 = rows / block_m * block_m;
         h = rows - m0;
+        if (n0 >= N) {
+          n0 = (Lp - low_off[g]) * block_n;
+          h = 0;
+        }
       }
-      int32_t* o = out + (size_t)written * 5;
-      o[0] = wg; o[1] = g; o[2] = m0; o[3] = h; o[4] = tn;
+      int32_t* o = out + (size_t)written * 6;
+      o[0] = wg; o[1] = g; o[2] = m0; o[3] = h; o[4] = n0; o[5] = nc;
       ++written;
     }
   }

@@ -178,20 +178,23 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   const int nwg = gridDim.x;
   // Tile of a round. Forward: rows of x / rows of w[g]. WGRAD: rows of dY^T (n) / rows of X^T (k), both at the
   // column offset of the expert's padded block; t.row0 = first row of the expert's block of dW, t.rows = N.
-  struct TileRef { MoeGgTile t; int KT, rows_g, m0, h; int64_t xoff, woff; };  // m0, h: first row inside the group, rows
+  // m0, h: first row inside the group, rows; n0, nc: first column, columns (a whole tile or a piece of one)
+  struct TileRef { MoeGgTile t; int KT, rows_g, m0, h, n0, nc; int64_t xoff, woff; };
   // The workgroup's own sequence (moe_gg_seq_round): its long tiles in round order with its low tiles spread
   // evenly between them, at a phase that differs between XCDs, so that memory-bound low tiles and compute-bound
   // long tiles run side by side on the chip, while the workgroups of one XCD take theirs together and stay in
   // step. Tile ids: long tiles 0 .. n_long - 1, then the low tiles.
   auto tile_ref = [&](int seq) {
     TileRef r;
-    // Decoded in the prologue: group | rows << 16, first row / 64 | column tile << 16.
+    // Decoded in the prologue: group | rows << 16 | columns / 32 << 26, first row / 64 | first column / 32 << 16.
     const int gh = uni(sh.seq_tab[2 * seq]);
     const int mn = uni(sh.seq_tab[2 * seq + 1]);
     const int g = gh & 0xFFFF;
-    r.h = (int)((uint32_t)gh >> 16);
+    r.h = (gh >> 16) & 0x3FF;
+    r.nc = (int)((uint32_t)gh >> 26) * 32;
     r.m0 = (mn & 0xFFFF) * 64;
-    r.t.g = g; r.t.tm = 0; r.t.tn = (int)((uint32_t)mn >> 16);
+    r.n0 = (int)((uint32_t)mn >> 16) * 32;
+    r.t.g = g; r.t.tm = 0; r.t.tn = 0;
     r.rows_g = 0;
     if (WG2) {
       // Output: rows tm * 256 .. of the expert's block of dW (n), columns tn * 256 .. (k). Operands: the expert's
@@ -202,20 +205,20 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       r.t.row0 = g * N; r.t.rows = N;
       r.KT = max(1, moe_gg_cdiv(r.rows_g, 64));
       r.xoff = (int64_t)row0 * XPITCH + ((int64_t)g * p.x_col_block + r.m0) * 2;
-      r.woff = (int64_t)row0 * (int64_t)p.K * 2 + (int64_t)r.t.tn * BN * 2;
+      r.woff = (int64_t)row0 * (int64_t)p.K * 2 + (int64_t)r.n0 * 2;
     } else if (WGRAD) {
       r.t.row0 = g * N; r.t.rows = N;
       const int b0 = uni(sh.tile_off[g]);
       r.KT = uni(sh.tile_off[g + 1]) - b0;
       r.xoff = (int64_t)r.m0 * KROW + (int64_t)b0 * 128;
-      r.woff = (int64_t)(r.t.tn * BN) * KROW + (int64_t)b0 * 128;
+      r.woff = (int64_t)r.n0 * KROW + (int64_t)b0 * 128;
     } else {
       r.t.row0 = uni(sh.row_off[g]);
       r.t.rows = uni(sh.row_off[g + 1]) - r.t.row0;
       r.KT = KT_fwd;
       r.xoff = (int64_t)(r.t.row0 + r.m0) * XPITCH + (OP == OP_BF16_NT ? (int64_t)g * p.x_col_block * 2 : 0);
-      if (WNT) r.woff = ((int64_t)g * p.K * N + r.t.tn * TILE_COLS) * 2;  // w[g][0][n0]
-      else r.woff = ((int64_t)g * N + r.t.tn * TILE_COLS) * KROW;
+      if (WNT) r.woff = ((int64_t)g * p.K * N + r.n0) * 2;  // w[g][0][n0]
+      else r.woff = ((int64_t)g * N + r.n0) * KROW;
     }
     return r;
   };
@@ -242,11 +245,11 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     if (round >= sh.n_my) return;  // past the last tile: keep re-loading the last tile (never read)
     const TileRef tr = tile_ref(round);
     const MoeGgTile& t = tr.t;
-    const int m0 = tr.m0, n0 = t.tn * TILE_COLS;
+    const int m0 = tr.m0, n0 = tr.n0;
     c.KT = tr.KT;
     c.rows_g = tr.rows_g;
     c.x_last = max(tr.h, 1) - 1;  // (a piece without rows loads row 0 and stores nothing)
-    c.w_last = min(NCOLS - n0, TILE_COLS) - 1;  // SWIGLU: last valid output column of the tile
+    c.w_last = max(min(NCOLS - n0, tr.nc), 1) - 1;  // SWIGLU: last valid output column of the tile
     c.xg = uni_ptr(xp + tr.xoff);
     c.wg = uni_ptr(wp + tr.woff);
     if (BLOCK) {
@@ -388,9 +391,9 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     const TileRef tr = tile_ref(r);
     const MoeGgTile& t = tr.t;
     const int KT = tr.KT;
-    const int m0 = tr.m0, n0 = t.tn * TILE_COLS;
+    const int m0 = tr.m0, n0 = tr.n0;
     const int rows_valid = tr.h;
-    const int cols_valid = min(NCOLS - n0, TILE_COLS);
+    const int cols_valid = min(NCOLS - n0, tr.nc);
     // Activation fragments of this wave that hold at least one valid row (fragments are dealt
     // alternately to wm = 0 / 1, so a short tile shortens every wave's C phase alike).
     const int nfm = min(FM, max(0, ((rows_valid + 15) / 16 - wm + WM - 1) / WM));
@@ -682,9 +685,11 @@ DEVINL void pingpong_body(const GgParams& p) {
   const int tail_s = fwd ? moe_gg_tail_pieces(total, nwg) : 1;
   const int tail_first = fwd ? moe_gg_tail_first(total, nwg) : total;
   const int long_ids = fwd ? moe_gg_long_ids(total, nwg) : total;
+  const int low_c = fwd ? moe_gg_low_col_pieces(long_ids, total_low, nwg) : 1;
+  const int low_ids = total_low * low_c;
   int n_long = 0, n_low = 0;
   while (n_long * nwg < long_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < long_ids) ++n_long;
-  while ((n_long + n_low) * nwg < long_ids + total_low && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < long_ids + total_low)
+  while ((n_long + n_low) * nwg < long_ids + low_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < long_ids + low_ids)
     ++n_low;
   if (n_long + n_low == 0) return;
   // The sequence of this workgroup (moe_gg_seq_round), decoded once into a table: the arithmetic runs per thread
@@ -696,12 +701,14 @@ DEVINL void pingpong_body(const GgParams& p) {
   const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
   for (int i = threadIdx.x; i < n_my; i += NT) {
     int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
-    int g, m0, h, tn;  // group, first row inside the group, rows, column tile
+    constexpr int TC = OP == OP_BF16_SWIGLU ? BN / 2 : BN;  // output columns of a tile
+    int g, m0, h, n0, nc = TC;  // group, first row inside the group, rows, first column, columns
     if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
       const int ntm = moe_gg_cdiv(p.N, BM), tpg = ntm * moe_gg_cdiv(p.K, BN);
       g = L / tpg;
       const int rem = L - g * tpg;
-      tn = rem / ntm;
+      const int tn = rem / ntm;
+      n0 = tn * BN;
       m0 = (rem - tn * ntm) * BM;
       h = min(p.N - m0, BM);
     } else if (L < long_ids) {
@@ -714,24 +721,32 @@ DEVINL void pingpong_body(const GgParams& p) {
       const int idx = L - tile_off[g];
       const int rows = row_off[g + 1] - row_off[g];
       const int nf = moe_gg_long_row_tiles(rows, BM);
-      tn = idx / nf;
+      const int tn = idx / nf;
+      n0 = tn * TC;
       m0 = (idx - tn * nf) * BM;
       h = min(rows - m0, BM);
       if (tail_s > 1 && L >= tail_first) {
         int off;
         moe_gg_piece_rows(h, tail_s, piece, &off, &h);
-        m0 += off;
+        if (h > 0) m0 += off;  // a piece without rows keeps the tile's first row: its loads must stay in bounds
       }
     } else {
-      const int Lp = L - long_ids;
+      // Low tiles, each cut into low_c column pieces when that fills the round (moe_gg_low_col_pieces).
+      const int Lp = (L - long_ids) / low_c, piece = (L - long_ids) % low_c;
       g = moe_gg_find_group(part_off, p.G, Lp);
-      tn = Lp - part_off[g];
+      const int tn = Lp - part_off[g];
+      nc = TC / low_c;
+      n0 = tn * TC + piece * nc;
       const int rows = row_off[g + 1] - row_off[g];
       m0 = rows / BM * BM;
       h = rows - m0;
+      if (n0 >= (OP == OP_BF16_SWIGLU ? p.N / 2 : p.N)) {  // a piece beyond the last column: no rows, loads in bounds
+        n0 = tn * TC;
+        h = 0;
+      }
     }
-    seq_tab[2 * i] = g | (h << 16);
-    seq_tab[2 * i + 1] = (m0 / 64) | (tn << 16);
+    seq_tab[2 * i] = g | (h << 16) | ((nc / 32) << 26);
+    seq_tab[2 * i + 1] = (m0 / 64) | ((n0 / 32) << 16);
   }
   __syncthreads();
 

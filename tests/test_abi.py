@@ -155,57 +155,53 @@ def test_scheduler_rejects_bad_arguments(lib):
     ([600, 0, 513, 255, 1, 2048 + 17], 1000, 16),
     ([700] * 40, 2048, 256),
     ([530], 256, 8),                                                 # fewer tiles than workgroups
+    ([100, 28], 128, 256),                                           # column pieces that would start beyond N
+    ([130, 128], 200, 64),                                           # row pieces of tiles with 128-130 rows
 ])
 def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
-    """The ping-pong kernels' order: every output row of every group exactly once per column tile; a low tile has
-    fewer than 128 rows and is the only row tile of its group or the last one of a group with at least two full
-    tiles; the long tiles of a last round that is at most half full are cut into 2 or 4 row pieces; every
-    workgroup gets the same number of tiles (+- 1), its low tiles spread through its sequence."""
+    """The ping-pong kernels' order: every output element of every group exactly once; a low tile has fewer than
+    128 rows and is the only row tile of its group or the last one of a group with at least two full tiles; the
+    long tiles of a last round that is at most half full are cut into 2 or 4 row pieces, and low tiles into 2 or
+    4 column pieces when those still fit into the round; every workgroup gets the same number of tiles (+- 1)."""
     ms = np.ascontiguousarray(m_sizes, dtype=np.int32)
     M = int(ms.sum())
     cap = 1 << 16
-    out = np.zeros((cap, 5), dtype=np.int32)
+    out = np.zeros((cap, 6), dtype=np.int32)
     n = lib.moe_gg_host_enumerate_tiles_two_lists(ms.ctypes.data_as(I32P), len(ms), M, N, 256, 256, nwg, 8,
                                                   out.ctypes.data_as(I32P), cap)
     assert n >= 0
     tiles = out[:n].tolist()
-    ntn = -(-N // 256)
-    # exact cover: per (group, column tile) the row ranges tile [0, m_g) without overlap
-    cover = {}
-    for wg, g, m0, h, tn in tiles:
-        assert 0 <= tn < ntn and m0 % 64 == 0 and 0 <= h <= 256 and m0 // 256 == (m0 + max(h, 1) - 1) // 256
-        cover.setdefault((g, tn), []).append((m0, h))
+    # every tile or piece, also one without rows, starts inside its group's rows and inside the columns: the kernel
+    # loads from there
+    for wg, g, m0, h, n0, nc in tiles:
+        assert 0 <= n0 < N and 0 <= m0 < max(m_sizes[g], 1) and 0 <= h <= 256, (g, m0, h, n0, nc)
+    # exact cover: every (group, row, column) once
     for g, m in enumerate(m_sizes):
-        for tn in range(ntn):
-            pieces = sorted(p for p in cover.get((g, tn), []) if p[1] > 0)
-            pos = 0
-            for m0, h in pieces:
-                assert m0 == pos, (g, tn, pieces)
-                pos += h
-            assert pos == m, (g, tn, pieces)
+        seen = np.zeros((m, N), dtype=np.int32)
+        for wg, tg, m0, h, n0, nc in tiles:
+            if tg == g and h > 0:
+                assert m0 % 64 == 0 and n0 % 32 == 0 and nc in (64, 128, 256) and m0 + h <= m
+                seen[m0:m0 + h, n0:min(n0 + nc, N)] += 1
+        assert (seen == 1).all(), g
 
     def is_low(g, m0, h):
         m = m_sizes[g]
         return m0 == m // 256 * 256 and h == m % 256 and 0 < h < 128 and (m // 256 >= 2 or m // 256 == 0)
 
     per_wg = {}
-    for wg, g, m0, h, tn in tiles:
+    for wg, g, m0, h, n0, nc in tiles:
         per_wg.setdefault(wg, []).append(is_low(g, m0, h))
     counts = [len(v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
     assert max(counts) - min(counts) <= 1
     lows = [sum(v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
     assert max(lows) - min(lows) <= 1
-    # pieces: only when the last round of long tiles is at most half full; then 2 or 4 per tile
-    n_long = sum((m // 256 + (1 if (m % 256 >= 128 or (0 < m % 256 and m // 256 < 2 and m // 256 > 0)) else 0)) * ntn
-                 for m in m_sizes)
-    n_pieces = sum(1 for wg, g, m0, h, tn in tiles if not is_low(g, m0, h) and (h < min(256, m_sizes[g] - m0 // 256 * 256)
-                                                                               or m0 % 256))
-    tail = n_long % nwg
-    if tail == 0 or tail * 2 > nwg:
-        assert n_pieces == 0
+    col_pieces = sum(1 for t in tiles if t[5] < 256)
+    row_pieces = sum(1 for wg, g, m0, h, n0, nc in tiles if not is_low(g, m0, h) and (m0 % 256 or h < min(256, m_sizes[g] - m0)))
     if m_sizes[0] == 1012 and N == 14336:
         # 7 long tiles and at most one low tile per workgroup: the XCDs (wg % 8) take their low tile at 8 different
-        # positions of the sequence, the workgroups of one XCD at the same one
+        # positions of the sequence, the workgroups of one XCD at the same one; 224 low tiles do not leave room
+        # for column pieces
+        assert col_pieces == 0 and row_pieces == 0
         pos = {}
         for wg, v in per_wg.items():
             if any(v):
@@ -213,5 +209,8 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
         assert all(len(p) == 1 for p in pos.values())
         assert len(pos) == 7 and len({next(iter(p)) for p in pos.values()}) == 7   # 224 low tiles: 7 XCDs of 32
     if m_sizes[0] == 1012 and N == 4096:
-        # 512 long tiles = 2 rounds and no tail; with the 64 low tiles nothing is cut
-        assert n_pieces == 0
+        # 512 long tiles = 2 full rounds; the 64 low tiles are cut into 4 column pieces each: a third, full round
+        assert row_pieces == 0 and col_pieces == 256 and len(tiles) == 768
+    if m_sizes == [530]:
+        # 2 long tiles on 8 workgroups: 4 row pieces each; the low tile (18 rows) is not cut (no room left)
+        assert row_pieces == 8
