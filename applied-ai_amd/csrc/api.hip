@@ -513,8 +513,7 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
   const int tail_s = moe_gg_tail_pieces(nl, num_workgroups);
   const int tail_first = moe_gg_tail_first(nl, num_workgroups);
   const int long_ids = moe_gg_long_ids(nl, num_workgroups);
-  const int low_c = moe_gg_low_col_pieces(long_ids, ns, num_workgroups);
-  const int total = long_ids + ns * low_c;
+  const int total = long_ids + ns;
   int written = 0;
   for (int wg = 0; wg < num_workgroups; ++wg) {
     int n_long = 0, n_low = 0;
@@ -545,18 +544,13 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
           if (h > 0) m0 += off;
         }
       } else {
-        const int Lp = (L - long_ids) / low_c, piece = (L - long_ids) % low_c;
+        const int Lp = L - long_ids;
         if (Lp >= ns) return MOE_GG_EINVAL;  // cannot happen
         g = moe_gg_find_group(low_off, G, Lp);
-        nc = block_n / low_c;
-        n0 = (Lp - low_off[g]) * block_n + piece * nc;
+        n0 = (Lp - low_off[g]) * block_n;
         const int rows = row_off[g + 1] - row_off[g];
         m0 = rows / block_m * block_m;
         h = rows - m0;
-        if (n0 >= N) {
-          n0 = (Lp - low_off[g]) * block_n;
-          h = 0;
-        }
       }
       int32_t* o = out + (size_t)written * 6;
       o[0] = wg; o[1] = g; o[2] = m0; o[3] = h; o[4] = n0; o[5] = nc;

@@ -685,8 +685,7 @@ DEVINL void pingpong_body(const GgParams& p) {
   const int tail_s = fwd ? moe_gg_tail_pieces(total, nwg) : 1;
   const int tail_first = fwd ? moe_gg_tail_first(total, nwg) : total;
   const int long_ids = fwd ? moe_gg_long_ids(total, nwg) : total;
-  const int low_c = fwd ? moe_gg_low_col_pieces(long_ids, total_low, nwg) : 1;
-  const int low_ids = total_low * low_c;
+  const int low_ids = total_low;
   int n_long = 0, n_low = 0;
   while (n_long * nwg < long_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < long_ids) ++n_long;
   while ((n_long + n_low) * nwg < long_ids + low_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < long_ids + low_ids)
@@ -731,19 +730,15 @@ DEVINL void pingpong_body(const GgParams& p) {
         if (h > 0) m0 += off;  // a piece without rows keeps the tile's first row: its loads must stay in bounds
       }
     } else {
-      // Low tiles, each cut into low_c column pieces when that fills the round (moe_gg_low_col_pieces).
-      const int Lp = (L - long_ids) / low_c, piece = (L - long_ids) % low_c;
+      // Low tiles. (Cutting few low tiles into column pieces for more workgroups was measured: no gain, a low
+      // tile is bound by the per-step cost of the K loop, not by the bytes it streams.)
+      const int Lp = L - long_ids;
       g = moe_gg_find_group(part_off, p.G, Lp);
       const int tn = Lp - part_off[g];
-      nc = TC / low_c;
-      n0 = tn * TC + piece * nc;
+      n0 = tn * TC;
       const int rows = row_off[g + 1] - row_off[g];
       m0 = rows / BM * BM;
       h = rows - m0;
-      if (n0 >= (OP == OP_BF16_SWIGLU ? p.N / 2 : p.N)) {  // a piece beyond the last column: no rows, loads in bounds
-        n0 = tn * TC;
-        h = 0;
-      }
     }
     seq_tab[2 * i] = g | (h << 16) | ((nc / 32) << 26);
     seq_tab[2 * i + 1] = (m0 / 64) | ((n0 / 32) << 16);

@@ -148,16 +148,6 @@ MOE_GG_HD int moe_gg_long_ids(int n_long, int num_wg) {
   const int first = moe_gg_tail_first(n_long, num_wg);
   return first + (n_long - first) * moe_gg_tail_pieces(n_long, num_wg);
 }
-// Low tiles stream a whole 256-column weight tile for a few rows: memory-bound work. When all of them, cut into 4
-// (or 2) column pieces, still fit into the round in which the long ids end, they are cut, so that 4 (2) times as
-// many CUs pull the same bytes.
-MOE_GG_HD int moe_gg_low_col_pieces(int long_ids, int n_low, int num_wg) {
-  if (n_low == 0) return 1;
-  const int room = num_wg - long_ids % num_wg;
-  if ((int64_t)n_low * 4 <= room) return 4;
-  if ((int64_t)n_low * 2 <= room) return 2;
-  return 1;
-}
 // Piece p of s of a tile with rv valid rows (BM = 256): first row and number of rows (0 if the tile is too low).
 MOE_GG_HD void moe_gg_piece_rows(int rv, int s, int p, int* off, int* h) {
   const int per = 256 / s;

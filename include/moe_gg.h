@@ -232,7 +232,7 @@ int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, i
                                 int max_tiles);
 /* The same for the 256 x 256 ping-pong kernels (block_m must be 256), which keep two tile lists (long tiles, low
  * tiles), give every workgroup its low tiles spread between its long ones, and cut the long tiles of a sparsely
- * filled last round into row pieces and few low tiles into column pieces. Six int32 per tile here: (workgroup,
+ * filled last round into row pieces. Six int32 per tile here: (workgroup,
  * group, first row inside the group, rows, first column, columns), for each workgroup in the order in which it
  * computes them; a piece may have 0 rows, and the columns may reach beyond N. */
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,

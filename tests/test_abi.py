@@ -155,14 +155,14 @@ def test_scheduler_rejects_bad_arguments(lib):
     ([600, 0, 513, 255, 1, 2048 + 17], 1000, 16),
     ([700] * 40, 2048, 256),
     ([530], 256, 8),                                                 # fewer tiles than workgroups
-    ([100, 28], 128, 256),                                           # column pieces that would start beyond N
+    ([100, 28], 128, 256),                                           # N smaller than a tile
     ([130, 128], 200, 64),                                           # row pieces of tiles with 128-130 rows
 ])
 def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
     """The ping-pong kernels' order: every output element of every group exactly once; a low tile has fewer than
     128 rows and is the only row tile of its group or the last one of a group with at least two full tiles; the
-    long tiles of a last round that is at most half full are cut into 2 or 4 row pieces, and low tiles into 2 or
-    4 column pieces when those still fit into the round; every workgroup gets the same number of tiles (+- 1)."""
+    long tiles of a last round that is at most half full are cut into 2 or 4 row pieces; every workgroup gets the
+    same number of tiles (+- 1)."""
     ms = np.ascontiguousarray(m_sizes, dtype=np.int32)
     M = int(ms.sum())
     cap = 1 << 16
@@ -180,7 +180,7 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
         seen = np.zeros((m, N), dtype=np.int32)
         for wg, tg, m0, h, n0, nc in tiles:
             if tg == g and h > 0:
-                assert m0 % 64 == 0 and n0 % 32 == 0 and nc in (64, 128, 256) and m0 + h <= m
+                assert m0 % 64 == 0 and n0 % 256 == 0 and nc == 256 and m0 + h <= m
                 seen[m0:m0 + h, n0:min(n0 + nc, N)] += 1
         assert (seen == 1).all(), g
 
@@ -199,8 +199,7 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
     row_pieces = sum(1 for wg, g, m0, h, n0, nc in tiles if not is_low(g, m0, h) and (m0 % 256 or h < min(256, m_sizes[g] - m0)))
     if m_sizes[0] == 1012 and N == 14336:
         # 7 long tiles and at most one low tile per workgroup: the XCDs (wg % 8) take their low tile at 8 different
-        # positions of the sequence, the workgroups of one XCD at the same one; 224 low tiles do not leave room
-        # for column pieces
+        # positions of the sequence, the workgroups of one XCD at the same one
         assert col_pieces == 0 and row_pieces == 0
         pos = {}
         for wg, v in per_wg.items():
@@ -209,8 +208,8 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
         assert all(len(p) == 1 for p in pos.values())
         assert len(pos) == 7 and len({next(iter(p)) for p in pos.values()}) == 7   # 224 low tiles: 7 XCDs of 32
     if m_sizes[0] == 1012 and N == 4096:
-        # 512 long tiles = 2 full rounds; the 64 low tiles are cut into 4 column pieces each: a third, full round
-        assert row_pieces == 0 and col_pieces == 256 and len(tiles) == 768
+        # 512 long tiles = 2 full rounds, then the 64 low tiles: nothing is cut
+        assert row_pieces == 0 and col_pieces == 0 and len(tiles) == 576
     if m_sizes == [530]:
-        # 2 long tiles on 8 workgroups: 4 row pieces each; the low tile (18 rows) is not cut (no room left)
+        # 2 long tiles on 8 workgroups: 4 row pieces each; then the low tile (18 rows)
         assert row_pieces == 8
