@@ -62,6 +62,9 @@ bool use_decode_kernel(int64_t M, int G) { return M <= (int64_t)G * 24; }
 
 // The ping-pong kernels form slab offsets with 24-bit multiplies: an operand row must be shorter than 16 MB.
 constexpr int64_t PINGPONG_MAX_ROW_BYTES = 1 << 24;
+// bf16 forward: largest expert count for which the small-M kernel is launched behind the ping-pong kernel for the
+// low tiles (moe_gg_tails_apart).
+constexpr int TAILS_APART_MAX_GROUPS = 32;
 
 extern "C" {
 
@@ -123,6 +126,7 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
   const int64_t ntn256 = (N + 255) / 256;
   // The ping-pong kernel tabulates each workgroup's tile sequence and forms slab offsets with 24-bit multiplies.
   const bool pingpong_ok = K < PINGPONG_MAX_ROW_BYTES / 2 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg);
+  const bool automatic = variant < 0;
   if (variant < 0 && decode_ok && use_decode_kernel(M, G)) variant = MOE_GG_GG_DECODE;
   if (variant == MOE_GG_GG_DECODE) {
     if (!decode_ok) return MOE_GG_EUNSUPPORTED;
@@ -145,9 +149,17 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
     else variant = MOE_GG_GG_TILED_64;
   }
   switch (variant) {
-    case MOE_GG_GG_PINGPONG_256:
+    case MOE_GG_GG_PINGPONG_256: {
       if (!pingpong_ok) return MOE_GG_EUNSUPPORTED;
-      return (int)gg_bf16_pingpong_launch(p, num_wg, s);
+      // Automatic choice only: few low tiles that would take a round of their own go to the small-M kernel
+      // (moe_gg_tails_apart, decided on the device by both kernels). Its grid has N / 32 workgroups per expert,
+      // most of which leave at once: only worth launching for a few experts.
+      const bool tails = automatic && decode_ok && G <= TAILS_APART_MAX_GROUPS;
+      p.tails_apart = tails ? num_wg : 0;
+      const hipError_t e = gg_bf16_pingpong_launch(p, num_wg, s);
+      if (e != hipSuccess || !tails) return (int)e;
+      return (int)gg_bf16_decode_tails_launch(p, s);
+    }
     case MOE_GG_GG_TILED_256: return (int)gg_bf16_tiled_launch(p, 256, num_wg, s);
     case MOE_GG_GG_TILED_128: return (int)gg_bf16_tiled_launch(p, 128, num_wg, s);
     case MOE_GG_GG_TILED_64: return (int)gg_bf16_tiled_launch(p, 64, num_wg, s);
@@ -489,6 +501,22 @@ int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, i
     }
   }
   return written;
+}
+
+int moe_gg_host_tails_apart(const int32_t* m_sizes_host, int G, int64_t M, int N, int num_workgroups) {
+  if (!m_sizes_host || G <= 0 || G > MOE_GG_MAX_GROUPS_ABI || num_workgroups <= 0 || M < 0 || N <= 0)
+    return MOE_GG_EINVAL;
+  const int ntn = moe_gg_cdiv(N, 256);
+  int64_t r = 0, nl = 0, ns = 0, passes = 0;
+  for (int g = 0; g < G; ++g) {
+    const int m = moe_gg_clamp_rows(m_sizes_host[g], r, M);
+    r += m;
+    nl += moe_gg_long_row_tiles(m, 256) * ntn;
+    ns += moe_gg_low_row_tiles(m, 256) * ntn;
+    passes += (int64_t)moe_gg_low_passes(m, 256) * ntn;
+  }
+  if (nl > INT32_MAX || ns > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  return G <= TAILS_APART_MAX_GROUPS && moe_gg_tails_apart((int)nl, (int)ns, passes, num_workgroups) ? 1 : 0;
 }
 
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,

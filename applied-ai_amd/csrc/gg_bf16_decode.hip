@@ -20,13 +20,17 @@
 #include "common.h"
 #include "kernels.h"
 #include "tile_sched.h"
+#include "gg_tables.h"
 
 namespace {
 
-template <int NF, int MF, int WAVES, int DEPTH, bool PAIR>
+// TAIL: the kernel computes the low tiles that the 256 x 256 ping-pong kernel of the same call leaves out
+// (p.tails_apart, moe_gg_tails_apart): of every expert the rows beyond its last full 256-row tile.
+template <int NF, int MF, int WAVES, int DEPTH, bool PAIR, bool TAIL = false>
 __global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
   __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MF][256];
   __shared__ int s_row0, s_rows;
+  __shared__ int32_t tail_row_off[TAIL ? MOE_GG_MAX_GROUPS + 1 : 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -34,8 +38,34 @@ __global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
   const int g = blockIdx.y;
   const int K = p.K, N = p.N;
 
-  // Row range of expert g: prefix sum of m_sizes[0 .. g) (clamped like tile_sched.h does).
-  if (wave == 0) {
+  if (TAIL) {
+    // The ping-pong kernel's own tables and counts, so that both take the same decision.
+    build_row_offsets(p.m_sizes, p.G, p.M, tail_row_off);
+    if (wave == 0) {
+      long long n_long = 0, n_low = 0, passes = 0;
+      for (int i = lane; i < p.G; i += 64) {
+        const int r = tail_row_off[i + 1] - tail_row_off[i];
+        n_long += moe_gg_long_row_tiles(r, 256);
+        n_low += moe_gg_low_row_tiles(r, 256);
+        passes += moe_gg_low_passes(r, 256);
+      }
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) {
+        n_long += __shfl_xor(n_long, d, 64);
+        n_low += __shfl_xor(n_low, d, 64);
+        passes += __shfl_xor(passes, d, 64);
+      }
+      if (lane == 0) {
+        const int ntn = moe_gg_cdiv(N, 256);
+        const int r = tail_row_off[g + 1] - tail_row_off[g];
+        const bool mine = moe_gg_low_row_tiles(r, 256) > 0 &&
+                          moe_gg_tails_apart((int)(n_long * ntn), (int)(n_low * ntn), passes * ntn, p.tails_apart);
+        s_row0 = tail_row_off[g] + r / 256 * 256;
+        s_rows = mine ? r % 256 : 0;
+      }
+    }
+  } else if (wave == 0) {
+    // Row range of expert g: prefix sum of m_sizes[0 .. g) (clamped like tile_sched.h does).
     long long s = 0;
     for (int i = lane; i < g; i += 64) {
       int m = p.m_sizes[i];
@@ -149,6 +179,14 @@ hipError_t launch(const GgParams& p, hipStream_t stream) {
 }  // namespace
 
 // nf: 16-row weight fragments per wave (2 or 4); mf: 16-row activation fragments per pass (1, 2, 4).
+hipError_t gg_bf16_decode_tails_launch(const GgParams& p, hipStream_t stream) {
+  static_assert(MOE_GG_TAIL_PASS_ROWS == 32, "two activation fragments per pass");
+  dim3 grid((p.N + 31) / 32, p.G);
+  if (p.K % 256 == 0) hipLaunchKernelGGL((gg_bf16_decode<2, 2, 4, 8, true, true>), grid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((gg_bf16_decode<2, 2, 4, 8, false, true>), grid, dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
 hipError_t gg_bf16_decode_launch(const GgParams& p, int nf, int mf, hipStream_t stream) {
   if (nf == 2 && mf == 1) return launch<2, 1, 8>(p, stream);
   if (nf == 4 && mf == 1) return launch<4, 1, 4>(p, stream);

@@ -660,6 +660,8 @@ DEVINL void pingpong_body(const GgParams& p) {
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t tile_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t part_off[MOE_GG_MAX_GROUPS + 1];
+  __shared__ int32_t seq_tab[2 * MOE_GG_SEQ_CAP];
+  static_assert(2 * MOE_GG_SEQ_CAP >= MOE_GG_MAX_GROUPS + 1, "seq_tab doubles as a prefix table below");
 
   int total, total_low = 0;
   if (OP == OP_BF16_WGRAD_DIRECT) {
@@ -677,6 +679,12 @@ DEVINL void pingpong_body(const GgParams& p) {
     build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
     total_low = uni(part_off[p.G]);
     total = uni(tile_off[p.G]);
+    if (OP == OP_BF16 && p.tails_apart) {
+      // Few low tiles that would open a round of their own are computed by the small-M kernel of the same call.
+      build_tile_prefix(row_off, p.G, seq_tab, [&](int rows) { return moe_gg_low_passes(rows, BM) * ntn; });
+      if (moe_gg_tails_apart(total, total_low, uni(seq_tab[p.G]), p.tails_apart)) total_low = 0;
+      __syncthreads();  // seq_tab is rewritten below
+    }
   }
   const int nwg = gridDim.x;
   // Tiles of this workgroup in each list: rounds 0 .. n - 1 (tile ids grow with the round).
@@ -696,7 +704,6 @@ DEVINL void pingpong_body(const GgParams& p) {
   // Tile ids: the long tiles of all groups (group, then column tile, then row tile), then the low tiles (group,
   // column tile; see moe_gg_long_row_tiles), dealt to the workgroups round-robin: every workgroup gets the same
   // number (+- 1) of long tiles, and the low tiles go on where the long ones stopped.
-  __shared__ int32_t seq_tab[2 * MOE_GG_SEQ_CAP];
   const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
   for (int i = threadIdx.x; i < n_my; i += NT) {
     int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));

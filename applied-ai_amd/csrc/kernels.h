@@ -21,6 +21,9 @@ struct GgParams {
   int skip_rows;  // tiled fp8 kernel: experts with at most this many rows are left to the streaming kernel
   int ldx;          // gg_bf16_pingpong_nt / _wgrad_direct: leading dimension of x (the output gradient)
   int x_col_block;  // gg_bf16_pingpong_nt / _wgrad_direct: expert g reads x at column offset g * x_col_block
+  // gg_bf16_pingpong + gg_bf16_decode_tails pair: 0, or the ping-pong launch's workgroup count; the low tiles are
+  // then computed by the small-M kernel whenever moe_gg_tails_apart() says so (both kernels evaluate it).
+  int tails_apart;
 };
 
 // block_m in {256, 128, 64}; the matching tile width is gg_bf16_tiled_block_n(block_m).
@@ -34,6 +37,10 @@ hipError_t gg_bf16_generic_launch(const GgParams& p, hipStream_t stream);
 // Small-M split-K kernel; nf = 16-row weight fragments per wave (2 or 4), mf = 16-row activation
 // fragments per pass (1, 2 or 4). Needs K % 128 == 0 and 16-byte aligned x and w.
 hipError_t gg_bf16_decode_launch(const GgParams& p, int nf, int mf, hipStream_t stream);
+// The same kernel over the low tiles only (rows of an expert beyond its last full 256-row tile, when
+// moe_gg_low_row_tiles counts them as a low tile), and only if moe_gg_tails_apart() holds for the launch;
+// p.tails_apart = workgroup count of the ping-pong launch it completes.
+hipError_t gg_bf16_decode_tails_launch(const GgParams& p, hipStream_t stream);
 
 // W4A16 split-K dequant GEMM (w4a16.hip). a, scales, c share one 16-bit float type.
 struct W4Params {

@@ -148,6 +148,21 @@ MOE_GG_HD int moe_gg_long_ids(int n_long, int num_wg) {
   const int first = moe_gg_tail_first(n_long, num_wg);
   return first + (n_long - first) * moe_gg_tail_pieces(n_long, num_wg);
 }
+// Low tiles left to the small-M kernel. A low tile keeps its workgroup busy for all K steps at the pace of the
+// loads (about half the time of a full tile) however few rows it has; when the low tiles are few and do not fit
+// into the free workgroups of the last round of long tiles, they would add a round that most CUs sit out. The
+// small-M kernel (32 rows per pass, every CU streaming) computes those rows faster as long as its passes re-read
+// less than about 3/8 of a round's weight tiles. low_passes: sum over the low tiles of ceil(rows / 32).
+#define MOE_GG_TAIL_PASS_ROWS 32
+MOE_GG_HD int moe_gg_low_passes(int rows, int BM) {
+  return moe_gg_low_row_tiles(rows, BM) * moe_gg_cdiv(rows % BM, MOE_GG_TAIL_PASS_ROWS);
+}
+MOE_GG_HD bool moe_gg_tails_apart(int n_long, int n_low, long long low_passes, int num_wg) {
+  if (n_low <= 0 || low_passes * 8 > (long long)num_wg * 3) return false;
+  const int used = moe_gg_long_ids(n_long, num_wg) % num_wg;
+  return n_low > (used == 0 ? 0 : num_wg - used);
+}
+
 // Piece p of s of a tile with rv valid rows (BM = 256): first row and number of rows (0 if the tile is too low).
 MOE_GG_HD void moe_gg_piece_rows(int rv, int s, int p, int* off, int* h) {
   const int per = 256 / s;

@@ -213,3 +213,28 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
     if m_sizes == [530]:
         # 2 long tiles on 8 workgroups: 4 row pieces each; then the low tile (18 rows)
         assert row_pieces == 8
+
+
+def test_tails_apart_decision():
+    """Host mirror of the device-side decision to leave the low tiles to the small-M kernel: few low tiles that
+    would open a round of their own, and whose 32-row passes re-read at most 3/8 of a round's weight tiles."""
+    import ctypes
+
+    import applied_ai_amd
+
+    L = applied_ai_amd._lib.lib()
+
+    def apart(m_sizes, N, nwg=256):
+        arr = (ctypes.c_int32 * len(m_sizes))(*m_sizes)
+        return L.moe_gg_host_tails_apart(arr, len(m_sizes), sum(m_sizes), N, nwg)
+
+    mixtral = [1012, 1039, 1048, 1036, 998, 1023, 1040, 996]
+    assert apart(mixtral, 4096) == 1            # 512 long tiles = 2 rounds, 64 low tiles, 64 passes
+    assert apart(mixtral, 14336) == 0           # 224 low tiles: they fill a round of their own
+    assert apart([1024] * 8, 4096) == 0         # no low tiles
+    assert apart([1039, 700] + [0] * 6, 4096) == 0   # 112 long tiles: the 16 low tiles fit beside them
+    assert apart([1124] * 4 + [1024] * 4, 4096) == 0  # tails of 100 rows: 4 passes each, 256 > 96
+    assert apart([1151] + [1024] * 6 + [897], 4096) == 1  # one such tail: 64 passes
+    assert apart([40, 2008, 2000, 2000, 2048, 0, 48, 48], 4096) == 1  # experts that are one low tile
+    assert apart(mixtral * 5, 4096) == 0        # more than 32 experts: the second kernel is not launched
+    assert apart(mixtral, 4096, nwg=0) < 0
