@@ -64,7 +64,7 @@ SIGNATURES = {
         _c_int,
         [_i32_p, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _i32_p, _c_int],
     ),
-    "moe_gg_host_tails_apart": (_c_int, [_i32_p, _c_int, _c_i64, _c_int, _c_int]),
+    "moe_gg_host_tails_apart": (_c_int, [_i32_p, _c_int, _c_i64, _c_int, _c_int, _c_int]),
 }
 
 _lib = None

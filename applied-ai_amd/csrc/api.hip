@@ -65,6 +65,9 @@ constexpr int64_t PINGPONG_MAX_ROW_BYTES = 1 << 24;
 // bf16 forward: largest expert count for which the small-M kernel is launched behind the ping-pong kernel for the
 // low tiles (moe_gg_tails_apart).
 constexpr int TAILS_APART_MAX_GROUPS = 32;
+// ... and the shortest reduction: a round of low tiles costs about 0.9 us per 64-wide K step and the second launch
+// 5-15 us also when it finds nothing to do, so below this K there is little to gain.
+constexpr int TAILS_APART_MIN_K = 8192;
 
 extern "C" {
 
@@ -154,7 +157,7 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
       // Automatic choice only: few low tiles that would take a round of their own go to the small-M kernel
       // (moe_gg_tails_apart, decided on the device by both kernels). Its grid has N / 32 workgroups per expert,
       // most of which leave at once: only worth launching for a few experts.
-      const bool tails = automatic && decode_ok && G <= TAILS_APART_MAX_GROUPS;
+      const bool tails = automatic && decode_ok && G <= TAILS_APART_MAX_GROUPS && K >= TAILS_APART_MIN_K;
       p.tails_apart = tails ? num_wg : 0;
       const hipError_t e = gg_bf16_pingpong_launch(p, num_wg, s);
       if (e != hipSuccess || !tails) return (int)e;
@@ -503,8 +506,8 @@ int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, i
   return written;
 }
 
-int moe_gg_host_tails_apart(const int32_t* m_sizes_host, int G, int64_t M, int N, int num_workgroups) {
-  if (!m_sizes_host || G <= 0 || G > MOE_GG_MAX_GROUPS_ABI || num_workgroups <= 0 || M < 0 || N <= 0)
+int moe_gg_host_tails_apart(const int32_t* m_sizes_host, int G, int64_t M, int N, int K, int num_workgroups) {
+  if (!m_sizes_host || G <= 0 || G > MOE_GG_MAX_GROUPS_ABI || num_workgroups <= 0 || M < 0 || N <= 0 || K <= 0)
     return MOE_GG_EINVAL;
   const int ntn = moe_gg_cdiv(N, 256);
   int64_t r = 0, nl = 0, ns = 0, passes = 0;
@@ -516,7 +519,10 @@ int moe_gg_host_tails_apart(const int32_t* m_sizes_host, int G, int64_t M, int N
     passes += (int64_t)moe_gg_low_passes(m, 256) * ntn;
   }
   if (nl > INT32_MAX || ns > INT32_MAX) return MOE_GG_EUNSUPPORTED;
-  return G <= TAILS_APART_MAX_GROUPS && moe_gg_tails_apart((int)nl, (int)ns, passes, num_workgroups) ? 1 : 0;
+  return G <= TAILS_APART_MAX_GROUPS && K >= TAILS_APART_MIN_K && K % 128 == 0 &&
+                 moe_gg_tails_apart((int)nl, (int)ns, passes, num_workgroups)
+             ? 1
+             : 0;
 }
 
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,

@@ -23,8 +23,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM traffic per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what the
 # same counters read for a plain copy of known size (profiles/gg_bf16_pingpong_mixtral_prefill_traffic.md):
-# 1.95 GB fetched + 0.235 GB written.
-PREFILL_TRAFFIC_BYTES = 2.19e9
+# 1.94 GB fetched + 0.235 GB written.
+PREFILL_TRAFFIC_BYTES = 2.18e9
 
 
 def cpu_baseline_prefill(c, n_experts_sample=2):

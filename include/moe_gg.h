@@ -242,9 +242,10 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
 /* bf16 forward, automatic kernel choice with 256 x 256 tiles: 1 if for these (host) m_sizes the low tiles (an
  * expert's rows beyond its last full 256-row tile, when fewer than 128 and the expert has at least two full tiles
  * or no other tile) are computed by the small-M kernel instead of the ping-pong kernel, 0 if not; the tile order
- * above then holds without its low tiles. Both kernels take this decision on the device; this is its host mirror
+ * above then holds without its low tiles. Only calls with at most 32 experts and K >= 8192 (K a multiple of 128)
+ * launch the second kernel. Both kernels take this decision on the device; this is its host mirror
  * (num_workgroups as for the enumerators: the CU count rounded down to a multiple of the XCD count). */
-int moe_gg_host_tails_apart(const int32_t* m_sizes_host, int G, int64_t M, int N, int num_workgroups);
+int moe_gg_host_tails_apart(const int32_t* m_sizes_host, int G, int64_t M, int N, int K, int num_workgroups);
 
 #ifdef __cplusplus
 }

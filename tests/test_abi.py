@@ -224,9 +224,9 @@ def test_tails_apart_decision():
 
     L = applied_ai_amd._lib.lib()
 
-    def apart(m_sizes, N, nwg=256):
+    def apart(m_sizes, N, nwg=256, K=14336):
         arr = (ctypes.c_int32 * len(m_sizes))(*m_sizes)
-        return L.moe_gg_host_tails_apart(arr, len(m_sizes), sum(m_sizes), N, nwg)
+        return L.moe_gg_host_tails_apart(arr, len(m_sizes), sum(m_sizes), N, K, nwg)
 
     mixtral = [1012, 1039, 1048, 1036, 998, 1023, 1040, 996]
     assert apart(mixtral, 4096) == 1            # 512 long tiles = 2 rounds, 64 low tiles, 64 passes
@@ -237,4 +237,5 @@ def test_tails_apart_decision():
     assert apart([1151] + [1024] * 6 + [897], 4096) == 1  # one such tail: 64 passes
     assert apart([40, 2008, 2000, 2000, 2048, 0, 48, 48], 4096) == 1  # experts that are one low tile
     assert apart(mixtral * 5, 4096) == 0        # more than 32 experts: the second kernel is not launched
+    assert apart(mixtral, 4096, K=4096) == 0    # short reduction: the second launch would cost what it saves
     assert apart(mixtral, 4096, nwg=0) < 0
