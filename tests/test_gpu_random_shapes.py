@@ -81,3 +81,58 @@ def test_fast_paths_against_the_generic_kernel(seed):
                     assert ok, ("grad_w", variant, G, R, N, K, worst)
     finally:
         L.moe_gg_set_variant(0, AUTO)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_long_reductions_with_few_low_tiles(seed):
+    """K >= 8192 and at most 32 experts: the automatic choice may leave the low tiles (an expert's few rows beyond
+    its last full 256-row tile) to the small-M kernel, a decision both kernels take on the device. Random expert
+    sizes around whole rounds of tiles, where that decision flips; reference = the ping-pong kernel alone."""
+    import ctypes
+
+    import applied_ai_amd as A
+    from applied_ai_amd import _lib
+
+    L = _lib.lib()
+    rng = random.Random(seed)
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    nwg = cus - cus % 8
+    apart = 0
+    try:
+        for it in range(8):
+            N = rng.choice([256, 512, 1024, 2048])
+            K = rng.choice([8192, 8320])
+            G = rng.choice([2, 5, 8, 16, 32])
+            ntn = N // 256
+            # row tiles: about one round of long tiles, dealt to the experts; then tails
+            tiles = [0] * G
+            for _ in range(nwg // ntn + rng.choice([0, 0, 0, -3, 2])):
+                tiles[rng.randrange(G)] += 1
+            ms = []
+            for t in tiles:
+                kind = rng.choice(["full", "low", "low", "long"])
+                if kind == "low":
+                    ms.append(t * 256 + rng.choice([1, 7, 16, 31, 32, 33, 64, 100, 127]))
+                elif kind == "long" and t > 0:
+                    ms.append(t * 256 - rng.randint(1, 127))
+                else:
+                    ms.append(t * 256)
+            R = sum(ms)
+            arr = (ctypes.c_int32 * G)(*ms)
+            hit = L.moe_gg_host_tails_apart(arr, G, R, N, K, nwg)
+            apart += hit
+            print(f"seed {seed} case {it}: G={G} rows={R} N={N} K={K} apart={hit} m_sizes={ms}", flush=True)
+            x = (torch.randn(R, K, device="cuda", generator=gen) / 8).bfloat16()
+            w = (torch.randn(G * N, K, device="cuda", generator=gen) / 8).bfloat16()
+            m = torch.tensor(ms, dtype=torch.int32, device="cuda")
+            L.moe_gg_set_variant(0, PINGPONG)
+            ref = A.grouped_gemm(x, w, m)
+            L.moe_gg_set_variant(0, AUTO)
+            got = A.grouped_gemm(x, w, m)
+            ok, worst = close(got, ref)
+            assert ok, (G, R, N, K, ms, worst)
+            del x, w, ref, got
+        assert apart >= 2 or cus != 256, "the cases no longer reach the two-kernel path"
+    finally:
+        L.moe_gg_set_variant(0, AUTO)
