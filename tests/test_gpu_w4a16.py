@@ -34,7 +34,7 @@ def test_golden_fixture(zo, M):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,K,N,gs,zo", [
     (1, 256, 128, 128, 1), (16, 256, 128, 128, 0), (64, 256, 128, 128, 1), (5, 1152, 256, 128, 1),
-    (33, 512, 64, 128, 0), (16, 512, 64, 64, 0), (8, 256, 64, 32, 1), (17, 4096, 192, 128, 1),
+    (33, 512, 64, 128, 0), (16, 512, 64, 64, 0), (8, 256, 64, 32, 1), (17, 4096, 192, 128, 1), (100, 512, 128, 128, 1),
 ])
 def test_against_oracle(dtype, M, K, N, gs, zo):
     print(f"case {dtype} M={M} K={K} N={N} group={gs} zero_offset={zo}", flush=True)
