@@ -710,12 +710,17 @@ DEVINL void pingpong_body(const GgParams& p) {
     constexpr int TC = OP == OP_BF16_SWIGLU ? BN / 2 : BN;  // output columns of a tile
     int g, m0, h, n0, nc = TC;  // group, first row inside the group, rows, first column, columns
     if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
-      const int ntm = moe_gg_cdiv(p.N, BM), tpg = ntm * moe_gg_cdiv(p.K, BN);
+      // Tiles of an expert in bands of four column tiles, column tile fastest inside a band: the 32 tiles an XCD
+      // works on at a time are 8 row tiles x 4 column tiles, which share 8 + 4 operand slabs per K step (with the
+      // row tile fastest they were 32 + 1: 3 % slower at the Mixtral shape, the reads from the fabric bound it).
+      const int ntm = moe_gg_cdiv(p.N, BM), ntn = moe_gg_cdiv(p.K, BN), tpg = ntm * ntn;
       g = L / tpg;
       const int rem = L - g * tpg;
-      const int tn = rem / ntm;
-      n0 = tn * BN;
-      m0 = (rem - tn * ntm) * BM;
+      const int band = rem / (4 * ntm), idx = rem - band * (4 * ntm);
+      const int wb = min(4, ntn - band * 4);  // column tiles of this band
+      const int tm = idx / wb;
+      n0 = (band * 4 + idx - tm * wb) * BN;
+      m0 = tm * BM;
       h = min(p.N - m0, BM);
     } else if (L < long_ids) {
       int piece = 0;
