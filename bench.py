@@ -25,6 +25,11 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # same counters read for a plain copy of known size (profiles/gg_bf16_pingpong_mixtral_prefill_traffic.md):
 # 1.94 GB fetched + 0.235 GB written.
 PREFILL_TRAFFIC_BYTES = 2.18e9
+# The same for the other workloads (profiles/bench_all_kernels_traffic.md): fetched + written bytes per launch.
+DECODE_TRAFFIC_BYTES = {"up": 0.951e9 + 1.8e6, "down": 0.957e9 + 0.5e6}
+W4A16_TRAFFIC_BYTES = {1: 32.3e6 + 0.03e6, 16: 32.3e6 + 0.46e6, 64: 48.0e6 + 1.8e6}
+W4A16_GROUPED_TRAFFIC_BYTES = 254.2e6 + 1.8e6
+FP8_BLOCK_TRAFFIC_BYTES = 9.04e9 + 0.27e9
 
 
 def cpu_baseline_prefill(c, n_experts_sample=2):
@@ -123,7 +128,7 @@ def secondary_workloads(torch, A, dev):
                     "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
                     "roofline": {"bound": "hbm", "kernel": "gg_bf16_decode", "achieved": round(byt / ms / 1e6, 1),
                                  "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
-                                 "traffic": None}})
+                                 "traffic": DECODE_TRAFFIC_BYTES[name.split("-")[0]]}})
         del ws
 
     # ---- config 4: W4A16 split-K, K=4096, N=14336, group 128, (q - z) * s ----
@@ -147,7 +152,7 @@ def secondary_workloads(torch, A, dev):
                     "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
                     "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128", "achieved": round(byt / ms / 1e6, 1),
                                  "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
-                                 "traffic": None}})
+                                 "traffic": W4A16_TRAFFIC_BYTES.get(M)}})
     del qws
 
     # ---- W4A16 grouped (int4 experts), Mixtral decode: config 3's 64 rows over 8 experts, config 4's weight format ----
@@ -173,7 +178,7 @@ def secondary_workloads(torch, A, dev):
                 "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
                 "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128 (grid.y = experts)", "achieved": round(byt / ms / 1e6, 1),
                              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
-                             "traffic": None}})
+                             "traffic": W4A16_GROUPED_TRAFFIC_BYTES}})
     del qwe
 
     # ---- config 5: DeepSeek-V3-style fp8 block-scaled, 256 experts top-8, Zipf(1.1) routing ----
@@ -209,7 +214,7 @@ def secondary_workloads(torch, A, dev):
                 "tflops": round(flop / ms / 1e9, 1),
                 "roofline": {"bound": "hbm", "kernel": "gg_fp8_pingpong_block", "achieved": round(byt / ms / 1e6, 1),
                              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
-                             "traffic": None}})
+                             "traffic": FP8_BLOCK_TRAFFIC_BYTES}})
     del xq, wq, xs, ws, y
 
     # ---- whole MoE layer (fused_moe): Mixtral 8x7B, T=4096 top-2, bf16 ----
