@@ -469,7 +469,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         if (GRP == 1) wait_vm<NDMA>();  // first step: W0(1) of the prologue has landed; later nothing older is left
         __syncthreads();
         // ---------------- C phase: MFMAs only ----------------
-        __builtin_amdgcn_s_setprio(1);
+        // (No s_setprio here: with the computing wave at raised priority the kernels ran 0.5-2 % slower.)
         // bf16: one of the two MFMAs (K half kk) of fragment pair (j, i); fp8: its single MFMA.
         auto mma = [&](int j, int i, int kk) {
           if (!FP8) {
@@ -508,7 +508,6 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
             }
           }
         }
-        __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
         // Group 0: X(step + 1), issued in this step's load phase, is read in the next phase. Group 1: of its loads of
         // this step's load phase only W1(step + 1), issued first, is read that soon; the four W0(step + 2) loads may
