@@ -239,3 +239,36 @@ def test_tails_apart_decision():
     assert apart(mixtral * 5, 4096) == 0        # more than 32 experts: the second kernel is not launched
     assert apart(mixtral, 4096, K=4096) == 0    # short reduction: the second launch would cost what it saves
     assert apart(mixtral, 4096, nwg=0) < 0
+
+
+def test_there_is_no_cpu_path():
+    """Host tensors are refused by every entry function of the Python mirror (nothing computes on the CPU), and a
+    missing library is an error at load time, not a silent switch to another implementation."""
+    import torch
+
+    import applied_ai_amd as A
+
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    w = torch.zeros(2 * 8, 64, dtype=torch.bfloat16)
+    m = torch.tensor([2, 2], dtype=torch.int32)
+    for call in (
+        lambda: A.grouped_gemm(x, w, m),
+        lambda: A.grouped_gemm_forward(x, w, m),
+        lambda: A.grouped_gemm_swiglu(x, w, m),
+        lambda: A.grouped_gemm_backward(torch.zeros(4, 8, dtype=torch.bfloat16), x, w, m),
+        lambda: A.silu_and_mul(torch.zeros(4, 16, dtype=torch.bfloat16)),
+        lambda: A.route_group(torch.zeros(4, 2, dtype=torch.int32), 8),
+        lambda: A.float8_groupwise_quantize(torch.zeros(4, 128)),
+        lambda: A.fused_moe(x, torch.zeros(2, 16, 64, dtype=torch.bfloat16), torch.zeros(2, 64, 8, dtype=torch.bfloat16),
+                            torch.zeros(4, 2), torch.zeros(4, 2, dtype=torch.int32)),
+    ):
+        with pytest.raises(RuntimeError, match="HIP device only"):
+            call()
+
+    saved = (A._lib.LIB_PATH, A._lib._lib)
+    try:
+        A._lib.LIB_PATH, A._lib._lib = os.path.join(os.path.dirname(saved[0]), "no_such_library.so"), None
+        with pytest.raises(RuntimeError, match="no fallback"):
+            A._lib.lib()
+    finally:
+        A._lib.LIB_PATH, A._lib._lib = saved
