@@ -187,6 +187,18 @@ def matmul_split_k(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros
     return c
 
 
+def a100_qlinear(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor) -> torch.Tensor:
+    """Drop-in for the reference's data-parallel (not split-K) W4A16 linear layers a100_qlinear / h100_qlinear /
+    small_qlinear (kernels/triton/inference/gptq/a100_qlinear.py:76-121, h100_qlinear.py:87-121,
+    small_benchmark_cuda_graphs.py:109-150): the same packing, group size 128 and (q - (z + 1)) * s as
+    matmul_split_k (a100_qlinear.py:44-65), so one kernel serves all of them; the result has a's dtype."""
+    return matmul_split_k(a, b, scales, zeros, zero_offset=1, groupsize=128)
+
+
+h100_qlinear = a100_qlinear
+small_qlinear = a100_qlinear
+
+
 def matmul_split_k_grouped(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
                            m_sizes: torch.Tensor, zero_offset: int = 1, groupsize: Optional[int] = None) -> torch.Tensor:
     """W4A16 grouped GEMM over expert-sorted rows: c[rows of expert g] = a[rows of g] @ dequant(b[g], scales[g], zeros[g]).

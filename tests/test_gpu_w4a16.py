@@ -97,3 +97,23 @@ def test_invalid_arguments():
         A.matmul_split_k(a, b, s, z, zero_offset=2)
     with pytest.raises(RuntimeError):
         A.matmul_split_k(a.cpu(), b.cpu(), s.cpu(), z.cpu())
+
+
+def test_qlinear_entry_points_of_the_reference():
+    """a100_qlinear / h100_qlinear / small_qlinear (the reference's data-parallel W4A16 layers) share packing,
+    group size 128 and the (q - (z + 1)) * s formula with matmul_split_k: same result, in a's dtype."""
+    import applied_ai_amd as A
+
+    M, K, N = 16, 512, 128
+    rng = np.random.default_rng(3)
+    q = rng.integers(0, 16, size=(K, N)); zz = rng.integers(0, 16, size=(K // 128, N))
+    scales = torch.from_numpy(rng.uniform(0.005, 0.02, size=(K // 128, N)).astype(np.float32)).to(torch.float16)
+    a = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.float16)
+    qw, qz = O.pack_int4_along_k(q), O.pack_int4_along_n(zz)
+    args = (a.cuda(), torch.from_numpy(qw).cuda(), scales.cuda(), torch.from_numpy(qz).cuda())
+    want = A.matmul_split_k(*args)
+    for fn in (A.a100_qlinear, A.h100_qlinear, A.small_qlinear):
+        got = fn(*args)
+        assert got.dtype == torch.float16 and torch.equal(got, want)
+    ref = O.w4a16_gemm(to_np(a), qw, to_np(scales), qz, 128, 1)
+    assert rel_fro(to_np(want), ref) <= TOL
