@@ -236,7 +236,7 @@ SCALE_ROWWISE = 0
 SCALE_BLOCK128 = 1
 
 
-def _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, scale_mode: int) -> torch.Tensor:
+def _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, scale_mode: int, out_layout: int = OUT_MN) -> torch.Tensor:
     # Mirrors _grouped_gemm with scales (dev/triton_groupGEMM/groupgemm.py:407-427, 478-494).
     assert x.is_contiguous()
     assert w.is_contiguous()
@@ -264,11 +264,12 @@ def _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, scale_mode: int) -> torch
     if tuple(x_scale.shape) != want_x or tuple(w_scale.shape) != want_w:
         raise ValueError(f"scale shapes must be {want_x} and {want_w}")
     dev = _require_cuda(x, w, m_sizes, x_scale, w_scale)
-    y = torch.empty((M, N), device=dev, dtype=torch.bfloat16)
+    cols = N * G if out_layout == OUT_BLOCK else N
+    y = torch.empty((M, cols), device=dev, dtype=torch.bfloat16)
     with torch.cuda.device(dev):
         rc = _lib.lib().moe_gg_grouped_gemm_fp8(
             x.data_ptr(), w.data_ptr(), y.data_ptr(), x_scale.data_ptr(), w_scale.data_ptr(), scale_mode,
-            m_sizes.data_ptr(), G, M, N, K, N, OUT_MN, _stream_ptr(dev),
+            m_sizes.data_ptr(), G, M, N, K, cols, out_layout, _stream_ptr(dev),
         )
     _lib.check(rc, "moe_gg_grouped_gemm_fp8")
     return y
@@ -280,6 +281,14 @@ def grouped_gemm_fp8_rowwise(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Te
     y = (x @ w_g.T) * x_scale[:, None] * w_scale[g*N:(g+1)*N][None, :], bf16 out.
     Drop-in for grouped_gemm_fp8_rowwise (dev/triton_groupGEMM/groupgemm.py:524-531)."""
     return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_ROWWISE)
+
+
+def grouped_gemm_fp8_rowwise_forward(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, x_scale: torch.Tensor,
+                                     w_scale: torch.Tensor) -> torch.Tensor:
+    """The same with the [M, N*G] output of the MoE-training copy: expert g writes columns [g*N, (g+1)*N) of its
+    own rows, the rest stays uninitialised. Drop-in for that copy's grouped_gemm_fp8_rowwise
+    (kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:632-639, store at :468-480)."""
+    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_ROWWISE, OUT_BLOCK)
 
 
 def grouped_gemm_fp8_blockwise(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, x_scale: torch.Tensor,

@@ -161,3 +161,29 @@ def test_every_kernel_variant_against_oracle(variant, mode):
         lib.moe_gg_set_variant(1, -1)
     ref = O.grouped_gemm_fp8(xq, wq, xs, ws, m_sizes, mode)
     assert rel_fro(to_np(y), ref) <= TOL
+
+
+def test_rowwise_block_layout_of_the_training_copy():
+    """grouped_gemm_fp8_rowwise_forward writes [M, N*G]: expert g's rows in columns [g*N, (g+1)*N), the same values
+    as the [M, N] entry point (kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:468-480)."""
+    import applied_ai_amd as A
+
+    G, N, K, m_sizes = 4, 256, 512, [0, 300, 1, 83]
+    rng = np.random.default_rng(9)
+    M = sum(m_sizes)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((G * N, K)) * 0.05).astype(np.float32)
+    xs = np.abs(x).max(axis=1) / 448.0; ws = np.abs(w).max(axis=1) / 448.0
+    xq = torch.from_numpy(np.clip(x / xs[:, None], -448, 448)).to(F8).cuda()
+    wq = torch.from_numpy(np.clip(w / ws[:, None], -448, 448)).to(F8).cuda()
+    args = (xq, wq, torch.tensor(m_sizes, dtype=torch.int32, device="cuda"),
+            torch.from_numpy(xs.astype(np.float32)).cuda(), torch.from_numpy(ws.astype(np.float32)).cuda())
+    plain = A.grouped_gemm_fp8_rowwise(*args)
+    wide = A.grouped_gemm_fp8_rowwise_forward(*args)
+    assert wide.shape == (M, N * G)
+    row = 0
+    for g, m in enumerate(m_sizes):
+        assert torch.equal(wide[row:row + m, g * N:(g + 1) * N], plain[row:row + m])
+        row += m
+    ref = O.grouped_gemm_fp8(xq.view(torch.uint8).cpu().numpy(), wq.view(torch.uint8).cpu().numpy(), xs, ws, m_sizes, 0)
+    assert rel_fro(to_np(plain), ref) <= TOL
