@@ -281,6 +281,15 @@ int moe_gg_route_group(const int32_t* flat_ids, int64_t n, int E, int32_t* perm,
   return (int)route_group_launch(flat_ids, (int)n, E, perm, m_sizes, offsets, (hipStream_t)stream);
 }
 
+int moe_gg_align_block_size(const int32_t* perm, const int32_t* m_sizes, int E, int64_t n, int block_size,
+                            int32_t* sorted_ids, int32_t* expert_ids, int32_t* num_post_pad, void* stream) {
+  if (n < 0 || E <= 0 || block_size <= 0) return MOE_GG_EINVAL;
+  if (E > MOE_GG_MAX_ROUTE_EXPERTS || n + (int64_t)E * block_size > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (!m_sizes || !sorted_ids || !expert_ids || !num_post_pad || (n > 0 && !perm)) return MOE_GG_EINVAL;
+  return (int)align_block_size_launch(perm, m_sizes, E, (int)n, block_size, sorted_ids, expert_ids, num_post_pad,
+                                      (hipStream_t)stream);
+}
+
 int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int64_t n, int64_t row_bytes,
                        void* stream) {
   if (n < 0 || k <= 0 || row_bytes < 0) return MOE_GG_EINVAL;

@@ -71,6 +71,10 @@ int gg_fp8_stream_max_rows();
 hipError_t route_topk_launch(const float* logits, int T, int E, int k, int32_t* ids, hipStream_t stream);
 hipError_t route_group_launch(const int32_t* flat, int n, int E, int32_t* perm, int32_t* m_sizes, int32_t* offsets,
                               hipStream_t stream);
+// sorted_ids [n + E * (block_size - 1)], expert_ids [n + E], num_post_pad [1]; perm / m_sizes as route_group_launch wrote them.
+hipError_t align_block_size_launch(const int32_t* perm, const int32_t* m_sizes, int E, int n, int block_size,
+                                   int32_t* sorted_ids, int32_t* expert_ids, int32_t* num_post_pad,
+                                   hipStream_t stream);
 hipError_t gather_rows_launch(const void* x, const int32_t* perm, int k, void* out, int n, int64_t row_bytes,
                               hipStream_t stream);
 // 1 x 128 fp8 quantiser (quant.hip); `groups` groups of 128 consecutive elements.

@@ -12,6 +12,7 @@
 //   x_sorted = x[perm // k]
 // All of it is integer / index work and bit-exact against the CPU oracle.
 #include "common.h"
+#include "gg_tables.h"
 #include "kernels.h"
 
 namespace {
@@ -142,6 +143,36 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const char* __restrict
   for (int64_t c = threadIdx.x; c < row_bytes / 16; c += blockDim.x) d[c] = s[c];
 }
 
+// Padded form of the grouping (moe_align_block_size, kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:138-180):
+// expert e's run of perm padded with the value n up to a multiple of block_size. Every workgroup rebuilds the two
+// prefix tables (rows, padded rows) from m_sizes in LDS; thread i then writes sorted_ids[i] and expert_ids[i].
+__global__ __launch_bounds__(256) void align_block_size_kernel(const int32_t* __restrict__ perm,
+                                                               const int32_t* __restrict__ m_sizes, int E, int n,
+                                                               int block_size, int32_t* __restrict__ sorted_ids,
+                                                               int n_sorted, int32_t* __restrict__ expert_ids,
+                                                               int n_blocks_cap, int32_t* __restrict__ num_post_pad) {
+  __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
+  __shared__ int32_t pad_off[MOE_GG_MAX_GROUPS + 1];
+  build_row_offsets(m_sizes, E, n, row_off);
+  build_tile_prefix(row_off, E, pad_off, [&](int rows) { return moe_gg_cdiv(rows, block_size) * block_size; });
+  const int total = pad_off[E];
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i == 0) num_post_pad[0] = total;
+  if (i < n_sorted) {
+    int v = n;
+    if (i < total) {
+      const int e = moe_gg_find_group(pad_off, E, i);
+      const int j = i - pad_off[e];
+      if (j < row_off[e + 1] - row_off[e]) v = perm[row_off[e] + j];
+    }
+    sorted_ids[i] = v;
+  }
+  if (i < n_blocks_cap) {
+    const long long first = (long long)i * block_size;
+    expert_ids[i] = first < total ? moe_gg_find_group(pad_off, E, (int)first) : -1;
+  }
+}
+
 }  // namespace
 
 hipError_t route_topk_launch(const float* logits, int T, int E, int k, int32_t* ids, hipStream_t stream) {
@@ -161,5 +192,15 @@ hipError_t gather_rows_launch(const void* x, const int32_t* perm, int k, void* o
                               hipStream_t stream) {
   if (n == 0) return hipSuccess;
   hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, stream, (const char*)x, perm, k, (char*)out, n, row_bytes);
+  return hipGetLastError();
+}
+
+hipError_t align_block_size_launch(const int32_t* perm, const int32_t* m_sizes, int E, int n, int block_size,
+                                   int32_t* sorted_ids, int32_t* expert_ids, int32_t* num_post_pad,
+                                   hipStream_t stream) {
+  const int n_sorted = n + E * (block_size - 1), n_blocks_cap = n + E;
+  const int threads = n_sorted > n_blocks_cap ? n_sorted : n_blocks_cap;
+  hipLaunchKernelGGL(align_block_size_kernel, dim3((threads + 255) / 256), dim3(256), 0, stream, perm, m_sizes, E, n,
+                     block_size, sorted_ids, n_sorted, expert_ids, n_blocks_cap, num_post_pad);
   return hipGetLastError();
 }

@@ -51,6 +51,29 @@ def route_group(topk_ids: torch.Tensor, num_experts: int) -> Tuple[torch.Tensor,
     return perm, m_sizes, offsets
 
 
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int,
+                         num_experts: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Drop-in for the reference's moe_align_block_size (kernels/triton/inference/col_major_moe_gemm/
+    v0_moe_fused.py:138-180), which wraps an external op: topk_ids [T, k] -> (sorted_token_ids
+    [T*k + E*(block_size-1)] int32, expert_ids [T*k + E] int32, num_tokens_post_padded [1] int32). The flat positions
+    token*k + j are grouped by ascending expert, stable, each expert's run padded with the value T*k up to a multiple
+    of block_size (worked example :157-165); expert_ids holds the expert of every block (-1 beyond the last one,
+    where the reference leaves the buffer uninitialised)."""
+    ids = topk_ids if topk_ids.dtype == torch.int32 else topk_ids.to(torch.int32)
+    perm, m_sizes, _ = route_group(ids, num_experts)
+    dev = perm.device
+    n = perm.shape[0]
+    sorted_ids = torch.empty((n + num_experts * (block_size - 1),), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((n + num_experts,), dtype=torch.int32, device=dev)
+    num_post_pad = torch.empty((1,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_align_block_size(perm.data_ptr(), m_sizes.data_ptr(), num_experts, n, block_size,
+                                                sorted_ids.data_ptr(), expert_ids.data_ptr(), num_post_pad.data_ptr(),
+                                                _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_align_block_size")
+    return sorted_ids, expert_ids, num_post_pad
+
+
 def gather_sorted(x: torch.Tensor, perm: torch.Tensor, k: int) -> torch.Tensor:
     """x_sorted[i] = x[perm[i] // k]: the token rows in expert-sorted order."""
     if x.dim() != 2 or perm.dtype != torch.int32:

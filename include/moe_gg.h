@@ -137,6 +137,16 @@ int moe_gg_route_topk(const float* logits, int64_t T, int E, int k, int32_t* ids
                       int32_t* offsets, void* stream);
 int moe_gg_route_group(const int32_t* flat_ids, int64_t n, int E, int32_t* perm, int32_t* m_sizes, int32_t* offsets,
                        void* stream);
+/* The padded form of that grouping, with the outputs of the reference's moe_align_block_size
+ * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:138-180; worked example :157-165), from the perm and
+ * m_sizes that moe_gg_route_group / moe_gg_route_topk wrote:
+ *   sorted_ids   device out, int32 [n + E * (block_size - 1)]: expert e's entries of perm, padded with the value n up
+ *                to a multiple of block_size; entries beyond the padded total are n as well
+ *   expert_ids   device out, int32 [n + E]: the expert of every block of block_size entries; -1 beyond the last block
+ *                (the reference leaves those uninitialised)
+ *   num_post_pad device out, int32 [1]: the padded total */
+int moe_gg_align_block_size(const int32_t* perm, const int32_t* m_sizes, int E, int64_t n, int block_size,
+                            int32_t* sorted_ids, int32_t* expert_ids, int32_t* num_post_pad, void* stream);
 /* out[i, :] = x[perm[i] / k, :] for i < n; rows of row_bytes bytes (multiple of 16), x and out 16-byte aligned. */
 int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int64_t n, int64_t row_bytes,
                        void* stream);

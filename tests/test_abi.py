@@ -70,6 +70,9 @@ def test_argument_errors_of_the_other_entry_points(lib):
     assert lib.moe_gg_route_topk(None, 4, 1000, 2, None, None, None, None, None) == -4      # E too large
     assert lib.moe_gg_route_group(None, 4, 0, None, None, None, None) == -1
     assert lib.moe_gg_gather_rows(None, None, 0, None, 4, 16, None) == -1                    # k <= 0
+    assert lib.moe_gg_align_block_size(None, None, 8, 4, 0, None, None, None, None) == -1    # block_size <= 0
+    assert lib.moe_gg_align_block_size(None, None, 1000, 4, 16, None, None, None, None) == -4  # E too large
+    assert lib.moe_gg_align_block_size(None, None, 8, 4, 16, None, None, None, None) == -1   # null pointers
     assert lib.moe_gg_silu_and_mul(None, None, 4, 12, None) == -1                            # null pointers
     assert lib.moe_gg_silu_and_mul(None, None, 0, 12, None) == 0
     assert lib.moe_gg_invert_perm(None, None, -1, None, None) == -1

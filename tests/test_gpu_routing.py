@@ -98,3 +98,34 @@ def test_routed_pipeline_end_to_end():
     operm, om = O.route(oid, E)
     ref = O.grouped_gemm(to_np(x)[operm // k], to_np(w), om)
     np.testing.assert_allclose(to_np(y), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_moe_align_block_size_known_answer():
+    """The worked example of the reference's docstring (v0_moe_fused.py:157-165), padding included."""
+    import applied_ai_amd as A
+
+    kat = json.load(open(os.path.join(GOLD, "moe_align_kat.json")))
+    ids = torch.tensor(kat["topk_ids"], dtype=torch.int32) - 1
+    sorted_ids, expert_ids, post = A.moe_align_block_size(ids.cuda(), kat["block_size"], kat["num_experts"])
+    torch.cuda.synchronize()
+    assert post.cpu().tolist() == [16]
+    assert sorted_ids.shape[0] == 12 + 4 * 3 and expert_ids.shape[0] == 12 + 4
+    assert sorted_ids.cpu().tolist()[:16] == kat["sorted_token_ids"]
+    assert sorted_ids.cpu().tolist()[16:] == [12] * 8
+    assert expert_ids.cpu().tolist() == [0, 1, 2, 3] + [-1] * 12
+
+
+@pytest.mark.parametrize("T,k,E,block", [(1, 2, 8, 16), (37, 2, 8, 16), (4096, 2, 8, 64), (512, 8, 256, 128), (300, 3, 100, 1),
+                                         (0, 2, 8, 16), (1000, 6, 768, 32)])
+def test_moe_align_block_size_against_oracle(T, k, E, block):
+    """Bit-exact against the CPU restatement, which the docstring example pins; int64 ids as torch.topk returns them."""
+    import applied_ai_amd as A
+
+    gen = torch.Generator().manual_seed(T + k + E)
+    ids = torch.stack([torch.randperm(E, generator=gen)[:k] for _ in range(T)]) if T else torch.zeros((0, k), dtype=torch.int64)
+    sorted_ids, expert_ids, post = A.moe_align_block_size(ids.cuda(), block, E)
+    torch.cuda.synchronize()
+    want_sorted, want_expert, want_post = O.moe_align_block_size(ids.numpy().astype(np.int32), block, E)
+    assert post.cpu().tolist() == [want_post]
+    assert np.array_equal(sorted_ids.cpu().numpy(), want_sorted)
+    assert np.array_equal(expert_ids.cpu().numpy(), want_expert)
