@@ -69,6 +69,38 @@ def combine_topk(y: torch.Tensor, perm: torch.Tensor, offsets: torch.Tensor, top
     return out
 
 
+def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, topk_weights: torch.Tensor,
+                            topk_ids: torch.Tensor, sorted_token_ids: torch.Tensor = None,
+                            expert_ids: torch.Tensor = None, num_tokens_post_padded: torch.Tensor = None,
+                            mul_routed_weight: bool = False, top_k: int = 1, config: dict = None) -> None:
+    """One gather-style expert GEMM of the reference's fused MoE with its call signature
+    (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:183-220, kernel :17-135): for every flat
+    position p = token * k + j of topk_ids, C.view(-1, N)[p] = A[p // top_k] @ B[topk_ids[p]].T, times
+    topk_weights.view(-1)[p] if mul_routed_weight (:122-126). A is [M, K] with top_k = k for the first GEMM and
+    [M * k, K] with top_k = 1 for the second; B [E, N, K]; C [M, k, N], written in place. bf16 only.
+
+    The rows are grouped by expert from topk_ids itself (the grouping that sorted_token_ids / expert_ids /
+    num_tokens_post_padded encode with padding; those arguments and config are accepted and not needed), gathered,
+    multiplied by the grouped GEMM and scattered back; the routed weight multiplies the bf16 product."""
+    assert A.is_contiguous() and B.is_contiguous() and C.is_contiguous(), "A, B and C must be contiguous"
+    assert A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and C.dtype == torch.bfloat16, "bf16 only"
+    E, N, K = B.shape
+    assert A.shape[1] == K, "Incompatible dimensions"
+    n = topk_ids.numel()
+    assert C.numel() == n * N and A.shape[0] * top_k == n, "C must be [M, k, N] and A [M * k / top_k, K]"
+    _require_cuda(A, B, C, topk_ids)
+    ids = topk_ids if topk_ids.dtype == torch.int32 else topk_ids.to(torch.int32)
+    perm, m_sizes, offsets = route_group(ids, E)
+    xs = gather_sorted(A, perm, top_k)
+    y = grouped_gemm(xs, B.view(E * N, K), m_sizes)
+    if mul_routed_weight:
+        w = topk_weights if topk_weights.dtype in (torch.float32, torch.bfloat16) else topk_weights.float()
+        w = w.contiguous().view(n, 1)
+    else:
+        w = torch.ones((n, 1), dtype=torch.float32, device=A.device)
+    combine_topk(y, perm, offsets, w, out=C.view(n, N))
+
+
 def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk_weights: torch.Tensor,
               topk_ids: torch.Tensor, inplace: bool = False) -> torch.Tensor:
     """Mixture-of-experts layer with top-k gating; arguments as the reference's fused_moe

@@ -184,3 +184,28 @@ def test_swiglu_errors(lib=None):
         A.grouped_gemm_swiglu(x, w, m)
     with pytest.raises(AssertionError):    # K mismatch
         A.grouped_gemm_swiglu(x[:, :64].contiguous(), w, m)
+
+
+@pytest.mark.parametrize("M,k,E,N,K", [(33, 2, 8, 256, 128), (700, 2, 8, 512, 256), (5, 4, 16, 64, 64)])
+def test_invoke_fused_moe_kernel_both_gemms_of_the_layer(M, k, E, N, K):
+    """The reference's GEMM-level entry (v0_moe_fused.py:183-220) as fused_moe uses it (:271-289): first GEMM with
+    top_k = k on [M, K] rows, second with top_k = 1 on [M * k, N] rows and the routed weights; against a per-row
+    fp32 product, atol = rtol = 1e-2 (test_moe_gemm.py:78-79 uses atol 1e-2)."""
+    import applied_ai_amd as A
+
+    gen = torch.Generator().manual_seed(M + E)
+    x = (torch.randn(M, K, generator=gen) / 4).bfloat16()
+    w1 = (torch.randn(E, N, K, generator=gen) / 4).bfloat16()
+    w2 = (torch.randn(E, K, N, generator=gen) / 4).bfloat16()
+    score = torch.softmax(torch.randn(M, E, generator=gen), dim=-1)
+    tw, ids = torch.topk(score, k)
+    sorted_ids, expert_ids, post = A.moe_align_block_size(ids.cuda(), 16, E)
+    c1 = torch.empty((M, k, N), dtype=torch.bfloat16, device="cuda")
+    A.invoke_fused_moe_kernel(x.cuda(), w1.cuda(), c1, tw.cuda(), ids.cuda(), sorted_ids, expert_ids, post, False, k, {})
+    ref1 = torch.einsum("mk,mjnk->mjn", x.float(), w1.float()[ids])
+    assert torch.allclose(c1.float().cpu(), ref1, rtol=1e-2, atol=1e-2)
+    h = c1.view(M * k, N)
+    c2 = torch.empty((M, k, K), dtype=torch.bfloat16, device="cuda")
+    A.invoke_fused_moe_kernel(h, w2.cuda(), c2, tw.cuda(), ids.cuda(), sorted_ids, expert_ids, post, True, 1, {})
+    ref2 = torch.einsum("mjn,mjkn->mjk", c1.float().cpu(), w2.float()[ids]) * tw[:, :, None]
+    assert torch.allclose(c2.float().cpu(), ref2, rtol=1e-2, atol=1e-2)
