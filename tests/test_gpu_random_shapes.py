@@ -136,3 +136,59 @@ def test_long_reductions_with_few_low_tiles(seed):
         assert apart >= 2 or cus != 256, "the cases no longer reach the two-kernel path"
     finally:
         L.moe_gg_set_variant(0, AUTO)
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_fp8_and_w4a16_random_shapes_against_the_oracle(seed):
+    """Random expert sizes and shapes for the fp8 grouped GEMM (both scale modes, every kernel variant the automatic
+    choice can take) and the grouped W4A16 GEMM, against the CPU oracle; relative Frobenius error <= 2e-2."""
+    import numpy as np
+
+    import applied_ai_amd as A
+    from oracle import oracle as O
+    from tests.gpu_util import rel_fro, to_np
+
+    rng = random.Random(seed)
+    nrng = np.random.default_rng(seed)
+    F8 = torch.float8_e4m3fn
+    for it in range(6):
+        G = rng.choice([1, 3, 8, 24])
+        M = rng.choice([5, 64, 300, 1100])
+        N = rng.choice([128, 256, 384])
+        K = rng.choice([128, 256, 1024])
+        ms = sizes_for(rng, G, M)
+        R = sum(ms)
+        print(f"seed {seed} case {it}: G={G} rows={R} N={N} K={K} m_sizes={ms}", flush=True)
+        m = torch.tensor(ms, dtype=torch.int32, device="cuda")
+        x = nrng.standard_normal((R, K)).astype(np.float32)
+        w = (nrng.standard_normal((G * N, K)) * 0.05).astype(np.float32)
+        for mode in (0, 1):
+            if mode == 1:
+                xq, xs = O.fp8_groupwise_quant(x) if R else (np.zeros((0, K), np.uint8), np.zeros((0, K // 128), np.float32))
+                wq, ws = O.fp8_block_quant_weight(w)
+                fn = A.grouped_gemm_fp8_blockwise
+            else:
+                xs = np.maximum(np.abs(x).max(axis=1, initial=0.0), 1e-12) / 448.0
+                ws = np.abs(w).max(axis=1) / 448.0
+                xq = torch.from_numpy(np.clip(x / xs[:, None], -448, 448)).to(F8).view(torch.uint8).numpy()
+                wq = torch.from_numpy(np.clip(w / ws[:, None], -448, 448)).to(F8).view(torch.uint8).numpy()
+                fn = A.grouped_gemm_fp8_rowwise
+            y = fn(torch.from_numpy(np.ascontiguousarray(xq)).view(F8).cuda(), torch.from_numpy(np.ascontiguousarray(wq)).view(F8).cuda(), m,
+                   torch.from_numpy(np.ascontiguousarray(xs, dtype=np.float32)).cuda(),
+                   torch.from_numpy(np.ascontiguousarray(ws, dtype=np.float32)).cuda())
+            if R:
+                ref = O.grouped_gemm_fp8(xq, wq, xs, ws, ms, mode)
+                assert rel_fro(to_np(y)[:R], ref[:R]) <= 2e-2, (mode, G, R, N, K)
+        # grouped W4A16 on the same expert sizes (N % 64 == 0, group 128)
+        Nq = 128
+        q = nrng.integers(0, 16, size=(G, K, Nq)); zz = nrng.integers(0, 16, size=(G, K // 128, Nq))
+        scales = torch.from_numpy(nrng.uniform(0.005, 0.02, size=(G, K // 128, Nq)).astype(np.float32)).bfloat16()
+        a = torch.from_numpy(x).bfloat16()
+        qw = np.stack([O.pack_int4_along_k(q[g]) for g in range(G)]); qz = np.stack([O.pack_int4_along_n(zz[g]) for g in range(G)])
+        c = A.matmul_split_k_grouped(a.cuda(), torch.from_numpy(qw).cuda(), scales.cuda(), torch.from_numpy(qz).cuda(), m)
+        row = 0
+        for g, mg in enumerate(ms):
+            if mg:
+                ref = O.w4a16_gemm(to_np(a[row:row + mg]), qw[g], to_np(scales[g]), qz[g], 128, 1)
+                assert rel_fro(to_np(c[row:row + mg]), ref) <= 2e-2, ("w4a16", g, mg, K)
+            row += mg
