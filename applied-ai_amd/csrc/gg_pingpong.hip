@@ -178,7 +178,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   const int nwg = gridDim.x;
   // Tile of a round. Forward: rows of x / rows of w[g]. WGRAD: rows of dY^T (n) / rows of X^T (k), both at the
   // column offset of the expert's padded block; t.row0 = first row of the expert's block of dW, t.rows = N.
-  // m0, h: first row inside the group, rows; n0, nc: first column, columns (a whole tile or a piece of one)
+  // m0, h: first row inside the group, rows (a whole tile or a row piece of one); n0, nc: first column, columns
   struct TileRef { MoeGgTile t; int KT, rows_g, m0, h, n0, nc; int64_t xoff, woff; };
   // The workgroup's own sequence (moe_gg_seq_round): its long tiles in round order with its low tiles spread
   // evenly between them, at a phase that differs between XCDs, so that memory-bound low tiles and compute-bound
