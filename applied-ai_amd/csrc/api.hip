@@ -450,13 +450,21 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   return (int)gg_bf16_wgrad_launch(p, 128, num_wg, s);
 }
 
-int moe_gg_silu_and_mul(const void* in, void* out, int64_t rows, int n, void* stream) {
+static int silu_and_mul_any(const void* in, void* out, int64_t rows, int n, bool fp16, void* stream) {
   if (rows < 0 || n < 0) return MOE_GG_EINVAL;
   if (rows == 0 || n == 0) return MOE_GG_OK;
   if (!in || !out) return MOE_GG_EINVAL;
   if (n % 8 != 0) return MOE_GG_ESHAPE;
   if (!aligned(in, 16) || !aligned(out, 16)) return MOE_GG_EALIGN;
-  return (int)silu_and_mul_launch(in, out, rows, n, (hipStream_t)stream);
+  return (int)silu_and_mul_launch(in, out, rows, n, fp16, (hipStream_t)stream);
+}
+
+int moe_gg_silu_and_mul(const void* in, void* out, int64_t rows, int n, void* stream) {
+  return silu_and_mul_any(in, out, rows, n, false, stream);
+}
+
+int moe_gg_silu_and_mul_f16(const void* in, void* out, int64_t rows, int n, void* stream) {
+  return silu_and_mul_any(in, out, rows, n, true, stream);
 }
 
 int moe_gg_invert_perm(const int32_t* perm, int32_t* inv, int64_t n, const int32_t* n_valid, void* stream) {
@@ -467,18 +475,28 @@ int moe_gg_invert_perm(const int32_t* perm, int32_t* inv, int64_t n, const int32
   return (int)invert_perm_launch(perm, inv, (int)n, n_valid, (hipStream_t)stream);
 }
 
-int moe_gg_combine_topk(const void* y, const int32_t* inv, const void* weights, int weights_dtype, void* out,
-                        int64_t T, int k, int d, int64_t n_rows, void* stream) {
+static int combine_topk_any(const void* y, const int32_t* inv, const void* weights, int weights_dtype, bool fp16,
+                            void* out, int64_t T, int k, int d, int64_t n_rows, void* stream) {
   if (T < 0 || k <= 0 || d < 0 || n_rows < 0) return MOE_GG_EINVAL;
-  if (weights_dtype != MOE_GG_DTYPE_FP32 && weights_dtype != MOE_GG_DTYPE_BF16) return MOE_GG_EINVAL;
+  if (weights_dtype != MOE_GG_DTYPE_FP32 && weights_dtype != (fp16 ? MOE_GG_DTYPE_FP16 : MOE_GG_DTYPE_BF16)) return MOE_GG_EINVAL;
   if (T == 0 || d == 0) return MOE_GG_OK;
   if (!y || !inv || !weights || !out) return MOE_GG_EINVAL;
   if (d % 8 != 0) return MOE_GG_ESHAPE;
   if (T > INT32_MAX || n_rows > INT32_MAX || T * k > INT32_MAX) return MOE_GG_EUNSUPPORTED;
   if (!aligned(y, 16) || !aligned(out, 16) || !aligned(weights, weights_dtype == MOE_GG_DTYPE_FP32 ? 4 : 2))
     return MOE_GG_EALIGN;
-  return (int)combine_topk_launch(y, inv, weights, weights_dtype == MOE_GG_DTYPE_BF16, out, (int)T, k, d, (int)n_rows,
-                                  (hipStream_t)stream);
+  return (int)combine_topk_launch(y, inv, weights, weights_dtype != MOE_GG_DTYPE_FP32, fp16, out, (int)T, k, d,
+                                  (int)n_rows, (hipStream_t)stream);
+}
+
+int moe_gg_combine_topk(const void* y, const int32_t* inv, const void* weights, int weights_dtype, void* out,
+                        int64_t T, int k, int d, int64_t n_rows, void* stream) {
+  return combine_topk_any(y, inv, weights, weights_dtype, false, out, T, k, d, n_rows, stream);
+}
+
+int moe_gg_combine_topk_f16(const void* y, const int32_t* inv, const void* weights, int weights_dtype, void* out,
+                            int64_t T, int k, int d, int64_t n_rows, void* stream) {
+  return combine_topk_any(y, inv, weights, weights_dtype, true, out, T, k, d, n_rows, stream);
 }
 
 int moe_gg_fp8_groupwise_quant(const void* in, int dtype, void* out, float* scales, int64_t numel, void* stream) {

@@ -82,10 +82,10 @@ hipError_t fp8_groupwise_quant_launch(const void* in, bool bf16_in, void* out, f
                                       hipStream_t stream);
 
 // MoE layer glue (moe_layer.hip). bf16 data; n and d multiples of 8; 16-byte aligned pointers.
-hipError_t silu_and_mul_launch(const void* in, void* out, int64_t rows, int n, hipStream_t stream);
+hipError_t silu_and_mul_launch(const void* in, void* out, int64_t rows, int n, bool fp16, hipStream_t stream);
 hipError_t invert_perm_launch(const int32_t* perm, int32_t* inv, int n, const int32_t* n_valid, hipStream_t stream);
-hipError_t combine_topk_launch(const void* y, const int32_t* inv, const void* weights, bool weights_bf16, void* out,
-                               int T, int k, int d, int n_rows, hipStream_t stream);
+hipError_t combine_topk_launch(const void* y, const int32_t* inv, const void* weights, bool weights_16bit, bool fp16,
+                               void* out, int T, int k, int d, int n_rows, hipStream_t stream);
 
 // Backward pass (gg_backward.hip, gg_bf16_prefill.hip). bf16.
 // src [B, R, C] -> dst [B, C, R].

@@ -13,9 +13,21 @@ namespace {
 
 DEVINL float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
 DEVINL float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xFFFF0000u); }
+// The two 16-bit floats of a dword, and back (round to nearest even); F16: IEEE half, else bf16.
+template <bool F16> DEVINL float lo16(uint32_t w) {
+  return F16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xFFFFu)) : bf16_lo(w);
+}
+template <bool F16> DEVINL float hi16(uint32_t w) {
+  return F16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)) : bf16_hi(w);
+}
+template <bool F16> DEVINL uint32_t pack16x2(float a, float b) {
+  if (!F16) return pack_bf16x2(a, b);
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)a) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)b) << 16);
+}
 
-// out[r, c] = silu(in[r, c]) * in[r, n + c], in [rows, 2n] bf16, out [rows, n] bf16, n % 8 == 0.
-// silu(v) = v / (1 + exp(-v)) evaluated in fp32; one rounding to bf16 at the end.
+// out[r, c] = silu(in[r, c]) * in[r, n + c], in [rows, 2n], out [rows, n], both bf16 or both fp16, n % 8 == 0.
+// silu(v) = v / (1 + exp(-v)) evaluated in fp32; one rounding to the 16-bit type at the end.
+template <bool F16>
 __global__ __launch_bounds__(256) void silu_and_mul_kernel(const u32x4_t* __restrict__ in, u32x4_t* __restrict__ out,
                                                            int64_t rows, int n8) {
   const int64_t total = rows * n8;
@@ -27,10 +39,10 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const u32x4_t* __rest
     u32x4_t o;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float g0 = bf16_lo(g[e]), g1 = bf16_hi(g[e]);
-      const float a0 = g0 / (1.f + __expf(-g0)) * bf16_lo(u[e]);
-      const float a1 = g1 / (1.f + __expf(-g1)) * bf16_hi(u[e]);
-      o[e] = pack_bf16x2(a0, a1);
+      const float g0 = lo16<F16>(g[e]), g1 = hi16<F16>(g[e]);
+      const float a0 = g0 / (1.f + __expf(-g0)) * lo16<F16>(u[e]);
+      const float a1 = g1 / (1.f + __expf(-g1)) * hi16<F16>(u[e]);
+      o[e] = pack16x2<F16>(a0, a1);
     }
     out[r * n8 + c] = o;
   }
@@ -49,8 +61,9 @@ __global__ __launch_bounds__(256) void invert_perm_kernel(const int32_t* __restr
 }
 
 // out[t, :] = sum_j weight[t, j] * y[inv[t * k + j], :], fp32 accumulation in the order j = 0 .. k-1,
-// bf16 out. One workgroup per token; d % 8 == 0. WBF16: weights are bf16, else fp32.
-template <bool WBF16>
+// 16-bit out. One workgroup per token; d % 8 == 0. F16: y and out are fp16, else bf16. W16: the weights have that
+// 16-bit type too, else they are fp32.
+template <bool W16, bool F16>
 __global__ __launch_bounds__(256) void combine_topk_kernel(const u32x4_t* __restrict__ y, const int32_t* __restrict__ inv,
                                                            const void* __restrict__ weights, u32x4_t* __restrict__ out,
                                                            int k, int d8, int n_rows) {
@@ -62,29 +75,30 @@ __global__ __launch_bounds__(256) void combine_topk_kernel(const u32x4_t* __rest
     for (int j = 0; j < k; ++j) {
       const int row = inv[(int64_t)t * k + j];
       if (row < 0 || row >= n_rows) continue;
-      const float w = WBF16 ? __builtin_bit_cast(float, (uint32_t)((const uint16_t*)weights)[(int64_t)t * k + j] << 16)
-                            : ((const float*)weights)[(int64_t)t * k + j];
+      const float w = W16 ? lo16<F16>((uint32_t)((const uint16_t*)weights)[(int64_t)t * k + j])
+                          : ((const float*)weights)[(int64_t)t * k + j];
       const u32x4_t v = y[(int64_t)row * d8 + c];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        acc[2 * e] += w * bf16_lo(v[e]);
-        acc[2 * e + 1] += w * bf16_hi(v[e]);
+        acc[2 * e] += w * lo16<F16>(v[e]);
+        acc[2 * e + 1] += w * hi16<F16>(v[e]);
       }
     }
     u32x4_t o;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(acc[2 * e], acc[2 * e + 1]);
+    for (int e = 0; e < 4; ++e) o[e] = pack16x2<F16>(acc[2 * e], acc[2 * e + 1]);
     out[(int64_t)t * d8 + c] = o;
   }
 }
 
 }  // namespace
 
-hipError_t silu_and_mul_launch(const void* in, void* out, int64_t rows, int n, hipStream_t stream) {
+hipError_t silu_and_mul_launch(const void* in, void* out, int64_t rows, int n, bool fp16, hipStream_t stream) {
   if (rows == 0 || n == 0) return hipSuccess;
   const int64_t total = rows * (n / 8);
   const int blocks = (int)(total / 256 + 1 < 256 * 32 ? total / 256 + 1 : 256 * 32);
-  hipLaunchKernelGGL(silu_and_mul_kernel, dim3(blocks), dim3(256), 0, stream, (const u32x4_t*)in, (u32x4_t*)out, rows, n / 8);
+  if (fp16) hipLaunchKernelGGL(silu_and_mul_kernel<true>, dim3(blocks), dim3(256), 0, stream, (const u32x4_t*)in, (u32x4_t*)out, rows, n / 8);
+  else hipLaunchKernelGGL(silu_and_mul_kernel<false>, dim3(blocks), dim3(256), 0, stream, (const u32x4_t*)in, (u32x4_t*)out, rows, n / 8);
   return hipGetLastError();
 }
 
@@ -94,12 +108,15 @@ hipError_t invert_perm_launch(const int32_t* perm, int32_t* inv, int n, const in
   return hipGetLastError();
 }
 
-hipError_t combine_topk_launch(const void* y, const int32_t* inv, const void* weights, bool weights_bf16, void* out,
-                               int T, int k, int d, int n_rows, hipStream_t stream) {
+hipError_t combine_topk_launch(const void* y, const int32_t* inv, const void* weights, bool weights_16bit, bool fp16,
+                               void* out, int T, int k, int d, int n_rows, hipStream_t stream) {
   if (T == 0 || d == 0) return hipSuccess;
-  if (weights_bf16)
-    hipLaunchKernelGGL(combine_topk_kernel<true>, dim3(T), dim3(256), 0, stream, (const u32x4_t*)y, inv, weights, (u32x4_t*)out, k, d / 8, n_rows);
-  else
-    hipLaunchKernelGGL(combine_topk_kernel<false>, dim3(T), dim3(256), 0, stream, (const u32x4_t*)y, inv, weights, (u32x4_t*)out, k, d / 8, n_rows);
+  const u32x4_t* yp = (const u32x4_t*)y;
+  u32x4_t* op = (u32x4_t*)out;
+  const dim3 grid(T), block(256);
+  if (fp16 && weights_16bit) hipLaunchKernelGGL((combine_topk_kernel<true, true>), grid, block, 0, stream, yp, inv, weights, op, k, d / 8, n_rows);
+  else if (fp16) hipLaunchKernelGGL((combine_topk_kernel<false, true>), grid, block, 0, stream, yp, inv, weights, op, k, d / 8, n_rows);
+  else if (weights_16bit) hipLaunchKernelGGL((combine_topk_kernel<true, false>), grid, block, 0, stream, yp, inv, weights, op, k, d / 8, n_rows);
+  else hipLaunchKernelGGL((combine_topk_kernel<false, false>), grid, block, 0, stream, yp, inv, weights, op, k, d / 8, n_rows);
   return hipGetLastError();
 }

@@ -26,15 +26,17 @@ FUSED_SWIGLU_MIN_ROWS = 1024
 
 
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
-    """out = silu(x[:, :n]) * x[:, n:] for bf16 x [rows, 2n] (ops.silu_and_mul, v0_moe_fused.py:284)."""
-    if x.dim() != 2 or x.dtype != torch.bfloat16 or x.shape[1] % 2:
-        raise ValueError("x must be bf16 [rows, 2n]")
+    """out = silu(x[:, :n]) * x[:, n:] for bf16 or fp16 x [rows, 2n] (ops.silu_and_mul, v0_moe_fused.py:284)."""
+    if x.dim() != 2 or x.dtype not in (torch.bfloat16, torch.float16) or x.shape[1] % 2:
+        raise ValueError("x must be bf16 or fp16 [rows, 2n]")
     dev = _require_cuda(x)
     x = x.contiguous()
     rows, n = x.shape[0], x.shape[1] // 2
-    out = torch.empty((rows, n), dtype=torch.bfloat16, device=dev)
+    out = torch.empty((rows, n), dtype=x.dtype, device=dev)
     with torch.cuda.device(dev):
-        rc = _lib.lib().moe_gg_silu_and_mul(x.data_ptr(), out.data_ptr(), rows, n, _stream_ptr(dev))
+        L = _lib.lib()
+        fn = L.moe_gg_silu_and_mul_f16 if x.dtype == torch.float16 else L.moe_gg_silu_and_mul
+        rc = fn(x.data_ptr(), out.data_ptr(), rows, n, _stream_ptr(dev))
     _lib.check(rc, "moe_gg_silu_and_mul")
     return out
 
@@ -42,11 +44,12 @@ def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
 def combine_topk(y: torch.Tensor, perm: torch.Tensor, offsets: torch.Tensor, topk_weights: torch.Tensor,
                  out: torch.Tensor = None) -> torch.Tensor:
     """out[t] = sum_j topk_weights[t, j] * y[row of (t, j)], y in expert-sorted row order (perm as from
-    route_group / route_topk, offsets its [E + 1] prefix table); fp32 accumulation, bf16 result."""
-    if y.dim() != 2 or y.dtype != torch.bfloat16:
-        raise ValueError("y must be bf16 [rows, d]")
-    if topk_weights.dim() != 2 or topk_weights.dtype not in (torch.float32, torch.bfloat16):
-        raise ValueError("topk_weights must be fp32 or bf16 [T, k]")
+    route_group / route_topk, offsets its [E + 1] prefix table); fp32 accumulation, result in y's dtype (bf16 or
+    fp16; the weights are fp32 or have y's dtype)."""
+    if y.dim() != 2 or y.dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError("y must be bf16 or fp16 [rows, d]")
+    if topk_weights.dim() != 2 or topk_weights.dtype not in (torch.float32, y.dtype):
+        raise ValueError("topk_weights must be [T, k] in fp32 or in y's dtype")
     dev = _require_cuda(y, perm, offsets, topk_weights)
     y = y.contiguous()
     topk_weights = topk_weights.contiguous()
@@ -55,16 +58,18 @@ def combine_topk(y: torch.Tensor, perm: torch.Tensor, offsets: torch.Tensor, top
         raise ValueError("perm must have T * k entries")
     inv = torch.full((T * k,), -1, dtype=torch.int32, device=dev)
     if out is None:
-        out = torch.empty((T, y.shape[1]), dtype=torch.bfloat16, device=dev)
-    elif out.shape != (T, y.shape[1]) or out.dtype != torch.bfloat16 or not out.is_contiguous():
-        raise ValueError("out must be a contiguous bf16 [T, d] tensor")
-    wdt = 2 if topk_weights.dtype == torch.float32 else 0  # MOE_GG_DTYPE_FP32 / MOE_GG_DTYPE_BF16
+        out = torch.empty((T, y.shape[1]), dtype=y.dtype, device=dev)
+    elif out.shape != (T, y.shape[1]) or out.dtype != y.dtype or not out.is_contiguous():
+        raise ValueError("out must be a contiguous [T, d] tensor of y's dtype")
+    fp16 = y.dtype == torch.float16
+    wdt = 2 if topk_weights.dtype == torch.float32 else (1 if fp16 else 0)  # MOE_GG_DTYPE_FP32 / _FP16 / _BF16
     with torch.cuda.device(dev):
         L = _lib.lib()
         rc = L.moe_gg_invert_perm(perm.data_ptr(), inv.data_ptr(), T * k, offsets[-1:].data_ptr(), _stream_ptr(dev))
         _lib.check(rc, "moe_gg_invert_perm")
-        rc = L.moe_gg_combine_topk(y.data_ptr(), inv.data_ptr(), topk_weights.data_ptr(), wdt, out.data_ptr(), T, k,
-                                   y.shape[1], y.shape[0], _stream_ptr(dev))
+        fn = L.moe_gg_combine_topk_f16 if fp16 else L.moe_gg_combine_topk
+        rc = fn(y.data_ptr(), inv.data_ptr(), topk_weights.data_ptr(), wdt, out.data_ptr(), T, k,
+                y.shape[1], y.shape[0], _stream_ptr(dev))
     _lib.check(rc, "moe_gg_combine_topk")
     return out
 
@@ -136,15 +141,15 @@ def dequant_gemm_moe(hidden_states: torch.Tensor, qw1: torch.Tensor, qw2: torch.
                      scales_qw2: torch.Tensor, zeros_qw1: torch.Tensor, zeros_qw2: torch.Tensor, topk_ids: torch.Tensor,
                      topk_weights: torch.Tensor = None, zero_offset: int = 1) -> torch.Tensor:
     """MoE layer with int4 (GPTQ) expert weights; arguments as the reference's dequant_gemm_moe
-    (kernels/triton/inference/gptq/mixtral/w4a16_fused_dequant_gemm.py:255-318): hidden_states [M, K] bf16,
-    qw1 [E, K/8, 2n] / qw2 [E, n/8, d] int32, scales [E, K/g, 2n] / [E, n/g, d] bf16, zeros [E, K/g, 2n/8] /
+    (kernels/triton/inference/gptq/mixtral/w4a16_fused_dequant_gemm.py:255-318): hidden_states [M, K] bf16 or fp16,
+    qw1 [E, K/8, 2n] / qw2 [E, n/8, d] int32, scales [E, K/g, 2n] / [E, n/g, d] in that dtype, zeros [E, K/g, 2n/8] /
     [E, n/g, d/8] int32, topk_ids [M, k]. Like the reference, the k rows of a token are summed without routed
     weights (:316-317) unless topk_weights is given. Same pipeline as fused_moe with the two products done by
     the grouped W4A16 kernel (moe_gg_w4a16_grouped)."""
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
     assert qw1.is_contiguous(), "Expert weights1 must be contiguous"
     assert qw2.is_contiguous(), "Expert weights2 must be contiguous"
-    assert hidden_states.dtype == torch.bfloat16, "bf16 only"
+    assert hidden_states.dtype in (torch.bfloat16, torch.float16), "bf16 or fp16"
     _require_cuda(hidden_states, qw1, qw2, scales_qw1, scales_qw2, zeros_qw1, zeros_qw2, topk_ids)
     E = qw1.shape[0]
     assert hidden_states.shape[1] == qw1.shape[1] * 8, "Incompatible dimensions"
@@ -154,7 +159,7 @@ def dequant_gemm_moe(hidden_states: torch.Tensor, qw1: torch.Tensor, qw2: torch.
     if topk_weights is None:
         tw = torch.ones((T, k), dtype=torch.float32, device=hidden_states.device)
     else:
-        tw = topk_weights if topk_weights.dtype in (torch.float32, torch.bfloat16) else topk_weights.float()
+        tw = topk_weights if topk_weights.dtype in (torch.float32, hidden_states.dtype) else topk_weights.float()
 
     perm, m_sizes, offsets = route_group(ids, E)
     xs = gather_sorted(hidden_states, perm, k)

@@ -199,11 +199,16 @@ int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const
  *   out[t, :] = sum_j weights[t, j] * y[inv[t*k + j], :]   (fp32 accumulation, j ascending; inv entries
  *   outside [0, n_rows) contribute nothing). y device [n_rows, d], out device [T, d], d % 8 == 0;
  *   weights device [T, k], fp32 or bf16 (weights_dtype = MOE_GG_DTYPE_FP32 / MOE_GG_DTYPE_BF16).
+ * The _f16 forms are the same on IEEE half data (and half or fp32 weights): the reference's layers also take fp16,
+ * and its W4A16 MoE test runs in it (kernels/triton/inference/gptq/mixtral/test_dequant_moe_gemm.py:25-84).
  */
 int moe_gg_silu_and_mul(const void* in, void* out, int64_t rows, int n, void* stream);
+int moe_gg_silu_and_mul_f16(const void* in, void* out, int64_t rows, int n, void* stream);
 int moe_gg_invert_perm(const int32_t* perm, int32_t* inv, int64_t n, const int32_t* n_valid, void* stream);
 int moe_gg_combine_topk(const void* y, const int32_t* inv, const void* weights, int weights_dtype, void* out,
                         int64_t T, int k, int d, int64_t n_rows, void* stream);
+int moe_gg_combine_topk_f16(const void* y, const int32_t* inv, const void* weights, int weights_dtype, void* out,
+                            int64_t T, int k, int d, int64_t n_rows, void* stream);
 
 /*
  * 1 x 128 group-wise fp8 e4m3fn quantiser. Replaces float8_groupwise_quantize

@@ -75,6 +75,8 @@ def test_argument_errors_of_the_other_entry_points(lib):
     assert lib.moe_gg_align_block_size(None, None, 8, 4, 16, None, None, None, None) == -1   # null pointers
     assert lib.moe_gg_silu_and_mul(None, None, 4, 12, None) == -1                            # null pointers
     assert lib.moe_gg_silu_and_mul(None, None, 0, 12, None) == 0
+    assert lib.moe_gg_silu_and_mul_f16(None, None, 4, 12, None) == -1                        # null pointers
+    assert lib.moe_gg_combine_topk_f16(None, None, None, 0, None, 4, 2, 64, 8, None) == -1   # bf16 weights with fp16 data
     assert lib.moe_gg_invert_perm(None, None, -1, None, None) == -1
     assert lib.moe_gg_combine_topk(None, None, None, 1, None, 4, 2, 8, 8, None) == -1        # fp16 weights unsupported
     assert lib.moe_gg_combine_topk(None, None, None, 2, None, 4, 0, 8, 8, None) == -1        # k <= 0

@@ -209,3 +209,28 @@ def test_invoke_fused_moe_kernel_both_gemms_of_the_layer(M, k, E, N, K):
     A.invoke_fused_moe_kernel(h, w2.cuda(), c2, tw.cuda(), ids.cuda(), sorted_ids, expert_ids, post, True, 1, {})
     ref2 = torch.einsum("mjn,mjkn->mjk", c1.float().cpu(), w2.float()[ids]) * tw[:, :, None]
     assert torch.allclose(c2.float().cpu(), ref2, rtol=1e-2, atol=1e-2)
+
+
+def test_fp16_forms_of_silu_and_mul_and_combine():
+    """The glue kernels on IEEE half data (the int4 layer runs in it): SiLU-and-mul within one fp16 ulp of the fp32
+    formula (the exponential is the fast one), the combine within the bar of the layer."""
+    import applied_ai_amd as A
+
+    gen = torch.Generator().manual_seed(5)
+    x = (torch.randn(37, 2 * 64, generator=gen) * 3).half()
+    got = A.silu_and_mul(x.cuda()).cpu()
+    want = (torch.nn.functional.silu(x[:, :64].float()) * x[:, 64:].float())
+    assert got.dtype == torch.float16
+    ulp = torch.maximum(want.abs(), torch.tensor(2.0 ** -14)) * 2.0 ** -10
+    assert bool(((got.float() - want).abs() <= ulp).all())
+
+    T, k, E, d = 50, 3, 8, 64
+    ids = torch.stack([torch.randperm(E, generator=gen)[:k] for _ in range(T)]).to(torch.int32)
+    perm, m_sizes, offsets = A.route_group(ids.cuda(), E)
+    y = torch.randn(T * k, d, generator=gen).half()
+    for w in (torch.rand(T, k, generator=gen), torch.rand(T, k, generator=gen).half()):
+        out = A.combine_topk(y.cuda(), perm, offsets, w.cuda()).cpu()
+        inv = torch.empty(T * k, dtype=torch.long)
+        inv[perm.cpu().long()] = torch.arange(T * k)
+        want = (w.float()[:, :, None] * y.float()[inv].view(T, k, d)).sum(1)
+        assert out.dtype == torch.float16 and torch.allclose(out.float(), want, rtol=2e-3, atol=2e-3)
