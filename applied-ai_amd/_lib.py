@@ -26,6 +26,11 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_i64, _c_int,
          _c_void_p],
     ),
+    "moe_gg_grouped_gemm_f16": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_i64, _c_int,
+         _c_void_p],
+    ),
     "moe_gg_grouped_gemm_fp8": (
         _c_int,
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_i64, _c_int, _c_int,

@@ -93,8 +93,8 @@ int moe_gg_set_variant(int op, int variant) {
   return MOE_GG_OK;
 }
 
-int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
-                             int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream) {
+static int grouped_gemm_16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M, int N, int K,
+                           int64_t ldy, int out_layout, bool fp16, void* stream) {
   if (G < 0 || M < 0 || N < 0 || K < 0) return MOE_GG_EINVAL;
   if (out_layout != MOE_GG_OUT_MN && out_layout != MOE_GG_OUT_BLOCK) return MOE_GG_EINVAL;
   if (M > INT32_MAX || (int64_t)G * N > INT32_MAX || ldy > INT32_MAX) return MOE_GG_EUNSUPPORTED;
@@ -117,6 +117,7 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
   p.col_block = out_layout == MOE_GG_OUT_BLOCK ? N : 0;
   p.vec_store = vec_store_level(y, ldy, N);
   p.xcds = di->xcds;
+  p.fp16 = fp16 ? 1 : 0;
 
   hipStream_t s = (hipStream_t)stream;
   const bool tiled_ok = K % 64 == 0 && aligned(x, 16) && aligned(w, 16);
@@ -157,7 +158,7 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
       // Automatic choice only: few low tiles that would take a round of their own go to the small-M kernel
       // (moe_gg_tails_apart, decided on the device by both kernels). Its grid has N / 32 workgroups per expert,
       // most of which leave at once: only worth launching for a few experts.
-      const bool tails = automatic && decode_ok && G <= TAILS_APART_MAX_GROUPS && K >= TAILS_APART_MIN_K;
+      const bool tails = automatic && decode_ok && !fp16 && G <= TAILS_APART_MAX_GROUPS && K >= TAILS_APART_MIN_K;
       p.tails_apart = tails ? num_wg : 0;
       const hipError_t e = gg_bf16_pingpong_launch(p, num_wg, s);
       if (e != hipSuccess || !tails) return (int)e;
@@ -168,6 +169,16 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
     case MOE_GG_GG_TILED_64: return (int)gg_bf16_tiled_launch(p, 64, num_wg, s);
     default: return MOE_GG_EINVAL;
   }
+}
+
+int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
+                             int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream) {
+  return grouped_gemm_16(x, w, y, m_sizes, G, M, N, K, ldy, out_layout, false, stream);
+}
+
+int moe_gg_grouped_gemm_f16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
+                            int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream) {
+  return grouped_gemm_16(x, w, y, m_sizes, G, M, N, K, ldy, out_layout, true, stream);
 }
 
 int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* x_scale, const float* w_scale,

@@ -27,6 +27,25 @@ DEVINL uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
+// The same for IEEE half.
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+DEVINL uint32_t pack_f16x2(float a, float b) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)a) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)b) << 16);
+}
+// 16-bit float type of a kernel instantiation: F16 = IEEE half, else bf16. Both are 2 bytes, so the data movement of
+// the kernels is the same; only the MFMA instruction and the conversions of the epilogue differ.
+template <bool F16> DEVINL uint32_t pack_16x2(float a, float b) { return F16 ? pack_f16x2(a, b) : pack_bf16x2(a, b); }
+template <bool F16> DEVINL uint16_t cvt_16(float a) {
+  return F16 ? __builtin_bit_cast(uint16_t, (_Float16)a) : __builtin_bit_cast(uint16_t, (__bf16)a);
+}
+template <bool F16> DEVINL float f32_of_16(uint16_t h) {
+  return F16 ? (float)__builtin_bit_cast(_Float16, h) : __builtin_bit_cast(float, (uint32_t)h << 16);
+}
+template <bool F16> DEVINL f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c) {
+  if (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
 DEVINL int lane_id() { return threadIdx.x & 63; }
 DEVINL int wave_id() { return threadIdx.x >> 6; }
 

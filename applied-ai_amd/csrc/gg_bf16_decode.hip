@@ -26,7 +26,7 @@ namespace {
 
 // TAIL: the kernel computes the low tiles that the 256 x 256 ping-pong kernel of the same call leaves out
 // (p.tails_apart, moe_gg_tails_apart): of every expert the rows beyond its last full 256-row tile.
-template <int NF, int MF, int WAVES, int DEPTH, bool PAIR, bool TAIL = false>
+template <int NF, int MF, int WAVES, int DEPTH, bool PAIR, bool TAIL = false, bool F16 = false>
 __global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
   __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MF][256];
   __shared__ int s_row0, s_rows;
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
             for (int j = 0; j < NF; ++j)
 #pragma unroll
               for (int i = 0; i < MF; ++i)
-                acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[d][h][j], xb[d][h][i], acc[j][i], 0, 0, 0);
+                acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wb[d][h][j]), __builtin_bit_cast(u32x4_t, xb[d][h][i]), acc[j][i]);
           if (t0 + d + DP < steps) load(d, t0 + d + DP);
         }
       }
@@ -154,13 +154,13 @@ __global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
         bf16_t* yrow = (bf16_t*)p.y + (int64_t)(row0 + m) * p.ldy + (int64_t)g * p.col_block;
         if (p.vec_store && n + 3 < N) {
           u32x2_t o;
-          o[0] = pack_bf16x2(v[0], v[1]);
-          o[1] = pack_bf16x2(v[2], v[3]);
+          o[0] = pack_16x2<F16>(v[0], v[1]);
+          o[1] = pack_16x2<F16>(v[2], v[3]);
           *(u32x2_t*)(yrow + n) = o;
         } else {
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            if (n + r < N) yrow[n + r] = (bf16_t)v[r];
+            if (n + r < N) ((uint16_t*)yrow)[n + r] = cvt_16<F16>(v[r]);
         }
       }
     }
@@ -171,7 +171,10 @@ __global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
 template <int NF, int MF, int DEPTH>
 hipError_t launch(const GgParams& p, hipStream_t stream) {
   dim3 grid((p.N + 16 * NF - 1) / (16 * NF), p.G);
-  if (p.K % 256 == 0) hipLaunchKernelGGL((gg_bf16_decode<NF, MF, 4, DEPTH, true>), grid, dim3(256), 0, stream, p);
+  if (p.fp16) {
+    if (p.K % 256 == 0) hipLaunchKernelGGL((gg_bf16_decode<NF, MF, 4, DEPTH, true, false, true>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((gg_bf16_decode<NF, MF, 4, DEPTH, false, false, true>), grid, dim3(256), 0, stream, p);
+  } else if (p.K % 256 == 0) hipLaunchKernelGGL((gg_bf16_decode<NF, MF, 4, DEPTH, true>), grid, dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((gg_bf16_decode<NF, MF, 4, DEPTH, false>), grid, dim3(256), 0, stream, p);
   return hipGetLastError();
 }

@@ -60,7 +60,7 @@ DEVINL void wait_vmcnt() {
 // expert g in columns pad_off[g] .. pad_off[g] + roundup(m_g, 64) - 1 (zero padded), so the reduction of expert g
 // is a whole number of 64-wide steps. Every expert has the same ceil(N / BM) * ceil(K / BN) tiles; an expert
 // without rows gets zeros. p.N = rows of dW per expert (N), p.K = columns (K), p.M = ldm, p.y = dW [G * N, K].
-template <class C, bool WGRAD>
+template <class C, bool WGRAD, bool F16 = false>
 __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
   __shared__ __attribute__((aligned(1024))) char lds[2 * C::STAGE];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
       for (int j = 0; j < C::FN; ++j)
 #pragma unroll
         for (int i = 0; i < C::FM; ++i)
-          acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[i], acc[j][i], 0, 0, 0);
+          acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf[j]), __builtin_bit_cast(u32x4_t, xf[i]), acc[j][i]);
     };
     // Ask the scheduler to spread the fragment reads of the next half over the MFMAs of this one.
     auto interleave = [&]() {
@@ -221,13 +221,13 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
           const f32x4_t v = acc[j][i];
           if (vec_ok && n + 3 < cols_valid) {
             u32x2_t o;
-            o[0] = pack_bf16x2(v[0], v[1]);
-            o[1] = pack_bf16x2(v[2], v[3]);
+            o[0] = pack_16x2<F16>(v[0], v[1]);
+            o[1] = pack_16x2<F16>(v[2], v[3]);
             *(u32x2_t*)(yrow + n) = o;
           } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-              if (n + r < cols_valid) yrow[n + r] = (bf16_t)v[r];
+              if (n + r < cols_valid) ((uint16_t*)yrow)[n + r] = cvt_16<F16>(v[r]);
           }
         }
       }
@@ -237,7 +237,8 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
 
 template <class C, bool WGRAD = false>
 hipError_t launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  hipLaunchKernelGGL((gg_bf16_persistent<C, WGRAD>), dim3(num_wg), dim3(C::NT), 0, stream, p);
+  if (!WGRAD && p.fp16) hipLaunchKernelGGL((gg_bf16_persistent<C, false, true>), dim3(num_wg), dim3(C::NT), 0, stream, p);
+  else hipLaunchKernelGGL((gg_bf16_persistent<C, WGRAD>), dim3(num_wg), dim3(C::NT), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -27,11 +27,17 @@ __global__ __launch_bounds__(256) void gg_bf16_generic(GgParams p) {
   if (g < 0) return;  // row beyond sum(m_sizes): left untouched
   const int n = blockIdx.y * 256 + threadIdx.x;
   if (n >= p.N) return;
-  const bf16_t* xr = (const bf16_t*)p.x + (int64_t)m * p.K;
-  const bf16_t* wr = (const bf16_t*)p.w + ((int64_t)g * p.N + n) * p.K;
+  const uint16_t* xr = (const uint16_t*)p.x + (int64_t)m * p.K;
+  const uint16_t* wr = (const uint16_t*)p.w + ((int64_t)g * p.N + n) * p.K;
+  uint16_t* yo = (uint16_t*)p.y + (int64_t)m * p.ldy + (int64_t)g * p.col_block + n;
   float acc = 0.f;
-  for (int k = 0; k < p.K; ++k) acc = __builtin_fmaf((float)xr[k], (float)wr[k], acc);
-  ((bf16_t*)p.y)[(int64_t)m * p.ldy + (int64_t)g * p.col_block + n] = (bf16_t)acc;
+  if (p.fp16) {
+    for (int k = 0; k < p.K; ++k) acc = __builtin_fmaf(f32_of_16<true>(xr[k]), f32_of_16<true>(wr[k]), acc);
+    *yo = cvt_16<true>(acc);
+  } else {
+    for (int k = 0; k < p.K; ++k) acc = __builtin_fmaf(f32_of_16<false>(xr[k]), f32_of_16<false>(wr[k]), acc);
+    *yo = cvt_16<false>(acc);
+  }
 }
 
 }  // namespace

@@ -85,8 +85,9 @@ constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x
 // OP_BF16_NT and both fragment kinds come from transposing reads. A tile reduces over the rows of its expert:
 // max(1, ceil(m_g / 64)) K steps; rows beyond the expert's last one re-read that row (the loads stay inside the
 // tensors), and group 0 overwrites them with zeros in the dY slab once it has landed, so they add nothing.
+// OP_F16: OP_BF16 on IEEE half data (the same kernel with the f16 MFMA and half conversions in the epilogue).
 constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4, OP_BF16_NT = 5,
-              OP_BF16_WGRAD_DIRECT = 6;
+              OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7;
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
 // 64 lanes x 16 B (or 4 B) from global memory straight into LDS: lane l's bytes land at lds_addr + 16 l
@@ -156,6 +157,7 @@ struct Cursor {
 template <int GRP, int OP>
 DEVINL void run_group(const GgParams& p, const Shared& sh) {
   constexpr bool FP8 = OP == OP_FP8_ROW || OP == OP_FP8_BLOCK;
+  constexpr bool F16 = OP == OP_F16;
   constexpr bool BLOCK = OP == OP_FP8_BLOCK;
   constexpr bool WGRAD = OP == OP_BF16_WGRAD;
   constexpr bool SWIGLU = OP == OP_BF16_SWIGLU;
@@ -473,8 +475,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
         // bf16: one of the two MFMAs (K half kk) of fragment pair (j, i); fp8: its single MFMA.
         auto mma = [&](int j, int i, int kk) {
           if (!FP8) {
-            acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf[kk][j]),
-                                                               __builtin_bit_cast(bf16x8_t, xf[kk][i]), acc[j][i], 0, 0, 0);
+            acc[j][i] = mfma_16x16x32<F16>(wf[kk][j], xf[kk][i], acc[j][i]);
           } else {
             const i32x8_t a = {(int)wf[0][j][0], (int)wf[0][j][1], (int)wf[0][j][2], (int)wf[0][j][3],
                                (int)wf[1][j][0], (int)wf[1][j][1], (int)wf[1][j][2], (int)wf[1][j][3]};
@@ -598,8 +599,8 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
             for (int j = 0; j < FN; j += 2) {
               f32x4_t v0 = acc[j][i], v1 = acc[j + 1][i];
               if (OP == OP_FP8_ROW) { v0 = v0 * am * bs[j]; v1 = v1 * am * bs[j + 1]; }
-              const uint32_t a0 = pack_bf16x2(v0[0], v0[1]), a1 = pack_bf16x2(v0[2], v0[3]);
-              const uint32_t b0 = pack_bf16x2(v1[0], v1[1]), b1 = pack_bf16x2(v1[2], v1[3]);
+              const uint32_t a0 = pack_16x2<F16>(v0[0], v0[1]), a1 = pack_16x2<F16>(v0[2], v0[3]);
+              const uint32_t b0 = pack_16x2<F16>(v1[0], v1[1]), b1 = pack_16x2<F16>(v1[2], v1[3]);
               const bool odd = eq & 1;
               const uint32_t s0 = odd ? a0 : b0, s1 = odd ? a1 : b1;   // what the partner stores
               const uint32_t r0 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)s0, 0x401F);  // lane ^ 16
@@ -615,8 +616,8 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
               f32x4_t v = acc[j][i];
               if (OP == OP_FP8_ROW) v = v * am * bs[j];
               u32x2_t o;
-              o[0] = pack_bf16x2(v[0], v[1]);
-              o[1] = pack_bf16x2(v[2], v[3]);
+              o[0] = pack_16x2<F16>(v[0], v[1]);
+              o[1] = pack_16x2<F16>(v[2], v[3]);
               *(u32x2_t*)(ybase + voff + j * 16) = o;
             }
             }
@@ -639,7 +640,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
                 if (n + rr < cols_valid) {
                   float o = v[rr];
                   if (OP == OP_FP8_ROW) o = o * am * wcol_scale[n + rr];
-                  yrow[n + rr] = (bf16_t)o;
+                  ((uint16_t*)yrow)[n + rr] = cvt_16<F16>(o);
                 }
             }
           }
@@ -763,6 +764,7 @@ DEVINL void pingpong_body(const GgParams& p) {
 }
 
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_body<OP_BF16>(p); }
+__global__ __launch_bounds__(NT) void gg_f16_pingpong(GgParams p) { pingpong_body<OP_F16>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_nt(GgParams p) { pingpong_body<OP_BF16_NT>(p); }
@@ -773,7 +775,8 @@ __global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpo
 }  // namespace
 
 hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  hipLaunchKernelGGL(gg_bf16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
+  if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
+  else hipLaunchKernelGGL(gg_bf16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -24,6 +24,7 @@ struct GgParams {
   // gg_bf16_pingpong + gg_bf16_decode_tails pair: 0, or the ping-pong launch's workgroup count; the low tiles are
   // then computed by the small-M kernel whenever moe_gg_tails_apart() says so (both kernels evaluate it).
   int tails_apart;
+  int fp16;  // forward kernels: x, w and y are IEEE half instead of bf16 (same layouts)
 };
 
 // block_m in {256, 128, 64}; the matching tile width is gg_bf16_tiled_block_n(block_m).

@@ -26,7 +26,6 @@
 
 namespace {
 
-typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
 
 template <bool FP16>
 struct Elem;

@@ -82,13 +82,13 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, t
     (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:183-220, kernel :17-135): for every flat
     position p = token * k + j of topk_ids, C.view(-1, N)[p] = A[p // top_k] @ B[topk_ids[p]].T, times
     topk_weights.view(-1)[p] if mul_routed_weight (:122-126). A is [M, K] with top_k = k for the first GEMM and
-    [M * k, K] with top_k = 1 for the second; B [E, N, K]; C [M, k, N], written in place. bf16 only.
+    [M * k, K] with top_k = 1 for the second; B [E, N, K]; C [M, k, N], written in place. bf16 or fp16.
 
     The rows are grouped by expert from topk_ids itself (the grouping that sorted_token_ids / expert_ids /
     num_tokens_post_padded encode with padding; those arguments and config are accepted and not needed), gathered,
     multiplied by the grouped GEMM and scattered back; the routed weight multiplies the bf16 product."""
     assert A.is_contiguous() and B.is_contiguous() and C.is_contiguous(), "A, B and C must be contiguous"
-    assert A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and C.dtype == torch.bfloat16, "bf16 only"
+    assert A.dtype in (torch.bfloat16, torch.float16) and B.dtype == A.dtype and C.dtype == A.dtype, "bf16 or fp16"
     E, N, K = B.shape
     assert A.shape[1] == K, "Incompatible dimensions"
     n = topk_ids.numel()
@@ -99,7 +99,7 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, t
     xs = gather_sorted(A, perm, top_k)
     y = grouped_gemm(xs, B.view(E * N, K), m_sizes)
     if mul_routed_weight:
-        w = topk_weights if topk_weights.dtype in (torch.float32, torch.bfloat16) else topk_weights.float()
+        w = topk_weights if topk_weights.dtype in (torch.float32, A.dtype) else topk_weights.float()
         w = w.contiguous().view(n, 1)
     else:
         w = torch.ones((n, 1), dtype=torch.float32, device=A.device)
@@ -110,25 +110,25 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, t
               topk_ids: torch.Tensor, inplace: bool = False) -> torch.Tensor:
     """Mixture-of-experts layer with top-k gating; arguments as the reference's fused_moe
     (v0_moe_fused.py:222-227): hidden_states [M, K], w1 [E, 2n, K], w2 [E, d, n], topk_weights / topk_ids [M, k].
-    bf16 only (the reference also takes fp16). With inplace=True the result is written into hidden_states
-    (d must equal K), as the reference does (:291-294)."""
+    bf16 or fp16 (:216). With inplace=True the result is written into hidden_states (d must equal K), as the
+    reference does (:291-294)."""
     assert hidden_states.shape[1] == w1.shape[2], "Incompatible dimensions"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
     assert w1.is_contiguous(), "Expert weights1 must be contiguous"
     assert w2.is_contiguous(), "Expert weights2 must be contiguous"
-    assert hidden_states.dtype == torch.bfloat16 and w1.dtype == torch.bfloat16 and w2.dtype == torch.bfloat16, \
-        "bf16 only"
+    assert hidden_states.dtype in (torch.bfloat16, torch.float16), "Only float16 and bfloat16 are supported"
+    assert w1.dtype == hidden_states.dtype and w2.dtype == hidden_states.dtype, "weights must have the activations' dtype"
     _require_cuda(hidden_states, w1, w2, topk_weights, topk_ids)
     E, two_n, K = w1.shape
     assert two_n % 2 == 0 and w2.shape[0] == E and w2.shape[2] == two_n // 2, "Incompatible expert weights"
     k = topk_ids.shape[1]
     ids = topk_ids if topk_ids.dtype == torch.int32 else topk_ids.to(torch.int32)
-    tw = topk_weights if topk_weights.dtype in (torch.float32, torch.bfloat16) else topk_weights.float()
+    tw = topk_weights if topk_weights.dtype in (torch.float32, hidden_states.dtype) else topk_weights.float()
 
     perm, m_sizes, offsets = route_group(ids, E)
     xs = gather_sorted(hidden_states, perm, k)
     swiglu_tiles = (xs.shape[0] // 256 + E) * ((two_n // 2 + 127) // 128)   # bound of the fused kernel's tile table
-    if (xs.shape[0] >= FUSED_SWIGLU_MIN_ROWS and K % 64 == 0 and two_n % 8 == 0 and two_n * K < 2 ** 31
+    if (xs.dtype == torch.bfloat16 and xs.shape[0] >= FUSED_SWIGLU_MIN_ROWS and K % 64 == 0 and two_n % 8 == 0 and two_n * K < 2 ** 31
             and swiglu_tiles <= 1023 * 256):
         h2 = grouped_gemm_swiglu(xs, w1.view(E * two_n, K), m_sizes)
     else:

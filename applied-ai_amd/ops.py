@@ -45,15 +45,17 @@ def _grouped_gemm_bf16(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, 
         raise ValueError(f"w.shape[0]={w.shape[0]} is not a multiple of G={G}")
     N = w.shape[0] // G
     assert K == w.shape[1], f"K mismatch: x has {K}, w has {w.shape[1]}"
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise ValueError("grouped_gemm takes bf16 x and w")
+    if x.dtype not in (torch.bfloat16, torch.float16) or w.dtype != x.dtype:
+        raise ValueError("grouped_gemm takes bf16 (or fp16) x and w of the same dtype")
     if m_sizes.dtype != torch.int32:
         raise ValueError("m_sizes must be int32")
     dev = _require_cuda(x, w, m_sizes)
     cols = N * G if out_layout == OUT_BLOCK else N
-    y = torch.empty((M, cols), device=dev, dtype=torch.bfloat16)
+    y = torch.empty((M, cols), device=dev, dtype=x.dtype)
     with torch.cuda.device(dev):
-        rc = _lib.lib().moe_gg_grouped_gemm_bf16(
+        L = _lib.lib()
+        fn = L.moe_gg_grouped_gemm_f16 if x.dtype == torch.float16 else L.moe_gg_grouped_gemm_bf16
+        rc = fn(
             x.data_ptr(), w.data_ptr(), y.data_ptr(), m_sizes.data_ptr(), G, M, N, K, cols, out_layout,
             _stream_ptr(dev),
         )
@@ -62,7 +64,8 @@ def _grouped_gemm_bf16(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, 
 
 
 def grouped_gemm(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor) -> torch.Tensor:
-    """y[off_g:off_g+m_g] = x[off_g:off_g+m_g] @ w[g*N:(g+1)*N].T for every expert g; y is [M, N] bf16.
+    """y[off_g:off_g+m_g] = x[off_g:off_g+m_g] @ w[g*N:(g+1)*N].T for every expert g; y is [M, N] in the dtype of
+    x and w (bf16 as in the reference, or fp16).
 
     Drop-in for grouped_gemm (dev/triton_groupGEMM/groupgemm.py:518-521). Rows at or beyond
     sum(m_sizes) are left uninitialised, as in the reference (torch.empty, groupgemm.py:427).

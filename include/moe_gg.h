@@ -58,6 +58,11 @@ const char* moe_gg_strerror(int code);
  */
 int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
                              int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream);
+/* The same on IEEE half x, w and y (the reference's MoE layer and its test run in fp16 as well:
+ * kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:216, test_moe_gemm.py:33-60). Same kernels with the f16
+ * MFMA; the low tiles are never handed to a second kernel. */
+int moe_gg_grouped_gemm_f16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
+                            int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream);
 
 #define MOE_GG_SCALE_ROWWISE 0  /* x_scale [M], w_scale [G*N] */
 #define MOE_GG_SCALE_BLOCK128 1 /* x_scale [M, K/128], w_scale [G*N/128, K/128] */

@@ -184,3 +184,33 @@ def test_mixtral_prefill_shape_sampled_rows():
         xr = c["x_sorted"][rows].float().numpy()
         ref = O.grouped_gemm(xr, c["w"][g * N:(g + 1) * N].float().numpy(), [len(rows)])
         np.testing.assert_allclose(to_np(y[rows]), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5])
+def test_fp16_every_kernel_family(variant):
+    """IEEE half data through every kernel family (ping-pong, tiled 256 / 128 / 64, generic, small-M) and through the
+    automatic choice, against the oracle on the same half-rounded inputs."""
+    import applied_ai_amd as A
+
+    L = A._lib.lib()
+    cases = [(8, [300, 0, 517, 64, 1, 255, 256, 700], 512, 256), (4, [5, 0, 17, 9], 256, 512), (3, [20, 10, 20], 40, 72)]
+    try:
+        for G, ms, N, K in cases:
+            if variant == 5 and (K % 128 or sum(ms) > 24 * G):
+                continue
+            if variant in (0, 1, 2, 3) and K % 64:
+                continue
+            x, w, _ = bf16_inputs(G, sum(ms), N, K, seed=41, w_std=0.25)
+            x, w = x.half(), w.half()
+            L.moe_gg_set_variant(0, variant)
+            y = A.grouped_gemm(x.cuda(), w.cuda(), torch.tensor(ms, dtype=torch.int32, device="cuda"))
+            assert y.dtype == torch.float16
+            ref = O.grouped_gemm(to_np(x), to_np(w), ms)
+            np.testing.assert_allclose(to_np(y), ref, rtol=RTOL, atol=ATOL)
+            yb = A.grouped_gemm_forward(x.cuda(), w.cuda(), torch.tensor(ms, dtype=torch.int32, device="cuda"))
+            row = 0
+            for g, m in enumerate(ms):
+                assert torch.equal(yb[row:row + m, g * N:(g + 1) * N], y[row:row + m])
+                row += m
+    finally:
+        L.moe_gg_set_variant(0, -1)

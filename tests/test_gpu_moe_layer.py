@@ -234,3 +234,24 @@ def test_fp16_forms_of_silu_and_mul_and_combine():
         inv[perm.cpu().long()] = torch.arange(T * k)
         want = (w.float()[:, :, None] * y.float()[inv].view(T, k, d)).sum(1)
         assert out.dtype == torch.float16 and torch.allclose(out.float(), want, rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("m", [2, 33, 200, 1500])
+def test_fused_moe_fp16_as_the_reference_test_runs_it(m):
+    """fp16 data (kernels/triton/inference/col_major_moe_gemm/test_moe_gemm.py:33-60) against torch_moe restated in
+    fp32 (:16-30); the reference's bar: atol 1e-2, rtol 0 (:78-79)."""
+    import applied_ai_amd as A
+
+    n, k, e, topk = 128, 256, 8, 2
+    a, w1, w2, tw, ids = make(m, n, k, e, topk, seed=300 + m)
+    a, w1, w2 = a.half(), w1.half(), w2.half()
+    y = A.fused_moe(a.cuda(), w1.cuda(), w2.cuda(), tw.cuda(), ids.cuda())
+    assert y.dtype == torch.float16 and y.shape == (m, k)
+    ref = torch.zeros(m, k)
+    for t in range(m):
+        for j in range(topk):
+            ex = int(ids[t, j])
+            h = a[t].float() @ w1[ex].float().t()
+            h = torch.nn.functional.silu(h[:n]) * h[n:]
+            ref[t] += tw[t, j] * (h @ w2[ex].float().t())
+    assert torch.allclose(y.float().cpu(), ref, atol=1e-2, rtol=0), float((y.float().cpu() - ref).abs().max())
