@@ -158,7 +158,7 @@ static int grouped_gemm_16(const void* x, const void* w, void* y, const int32_t*
       // Automatic choice only: few low tiles that would take a round of their own go to the small-M kernel
       // (moe_gg_tails_apart, decided on the device by both kernels). Its grid has N / 32 workgroups per expert,
       // most of which leave at once: only worth launching for a few experts.
-      const bool tails = automatic && decode_ok && !fp16 && G <= TAILS_APART_MAX_GROUPS && K >= TAILS_APART_MIN_K;
+      const bool tails = automatic && decode_ok && G <= TAILS_APART_MAX_GROUPS && K >= TAILS_APART_MIN_K;
       p.tails_apart = tails ? num_wg : 0;
       const hipError_t e = gg_bf16_pingpong_launch(p, num_wg, s);
       if (e != hipSuccess || !tails) return (int)e;

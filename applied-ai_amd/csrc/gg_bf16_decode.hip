@@ -185,7 +185,10 @@ hipError_t launch(const GgParams& p, hipStream_t stream) {
 hipError_t gg_bf16_decode_tails_launch(const GgParams& p, hipStream_t stream) {
   static_assert(MOE_GG_TAIL_PASS_ROWS == 32, "two activation fragments per pass");
   dim3 grid((p.N + 31) / 32, p.G);
-  if (p.K % 256 == 0) hipLaunchKernelGGL((gg_bf16_decode<2, 2, 4, 8, true, true>), grid, dim3(256), 0, stream, p);
+  if (p.fp16) {
+    if (p.K % 256 == 0) hipLaunchKernelGGL((gg_bf16_decode<2, 2, 4, 8, true, true, true>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((gg_bf16_decode<2, 2, 4, 8, false, true, true>), grid, dim3(256), 0, stream, p);
+  } else if (p.K % 256 == 0) hipLaunchKernelGGL((gg_bf16_decode<2, 2, 4, 8, true, true>), grid, dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((gg_bf16_decode<2, 2, 4, 8, false, true>), grid, dim3(256), 0, stream, p);
   return hipGetLastError();
 }

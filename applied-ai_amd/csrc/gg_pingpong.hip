@@ -679,7 +679,7 @@ DEVINL void pingpong_body(const GgParams& p) {
     build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
     total_low = uni(part_off[p.G]);
     total = uni(tile_off[p.G]);
-    if (OP == OP_BF16 && p.tails_apart) {
+    if ((OP == OP_BF16 || OP == OP_F16) && p.tails_apart) {
       // Few low tiles that would open a round of their own are computed by the small-M kernel of the same call.
       build_tile_prefix(row_off, p.G, seq_tab, [&](int rows) { return moe_gg_low_passes(rows, BM) * ntn; });
       if (moe_gg_tails_apart(total, total_low, uni(seq_tab[p.G]), p.tails_apart)) total_low = 0;

@@ -60,7 +60,7 @@ int moe_gg_grouped_gemm_bf16(const void* x, const void* w, void* y, const int32_
                              int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream);
 /* The same on IEEE half x, w and y (the reference's MoE layer and its test run in fp16 as well:
  * kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:216, test_moe_gemm.py:33-60). Same kernels with the f16
- * MFMA; the low tiles are never handed to a second kernel. */
+ * MFMA. */
 int moe_gg_grouped_gemm_f16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G,
                             int64_t M, int N, int K, int64_t ldy, int out_layout, void* stream);
 

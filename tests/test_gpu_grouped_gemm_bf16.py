@@ -62,6 +62,7 @@ def test_edge_cases(G, M, N, K, m_sizes):
     check(x, w, m_sizes)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("K", [8192, 8320])
 @pytest.mark.parametrize("m_sizes", [
     [1012, 1039, 1048, 1036, 998, 1023, 1040, 996],   # the Mixtral routing of the benchmark: tails of 12-24 rows
@@ -69,7 +70,7 @@ def test_edge_cases(G, M, N, K, m_sizes):
     [40, 2008, 2000, 2000, 2048, 0, 48, 48],           # experts that are one low tile, an empty one
     [1151, 1024, 1024, 1024, 1024, 1024, 1024, 897],   # a tail of 127 rows (four passes)
 ])
-def test_low_tiles_left_to_the_small_m_kernel(m_sizes, K):
+def test_low_tiles_left_to_the_small_m_kernel(m_sizes, K, dtype):
     """One full round of 256 x 256 tiles on 256 workgroups plus a few low tiles: the automatic choice computes the
     low tiles with the small-M kernel behind the ping-pong kernel (moe_gg_host_tails_apart mirrors the decision)."""
     import ctypes
@@ -82,7 +83,7 @@ def test_low_tiles_left_to_the_small_m_kernel(m_sizes, K):
     arr = (ctypes.c_int32 * G)(*m_sizes)
     assert A._lib.lib().moe_gg_host_tails_apart(arr, G, M, N, K, cus - cus % 8) == (1 if cus == 256 else 0)
     x, w, _ = bf16_inputs(G, M, N, K, seed=21, w_std=0.05)
-    check(x, w, m_sizes)
+    check(x.to(dtype), w.to(dtype), m_sizes)
 
 
 def test_large_two_groups():
