@@ -311,8 +311,8 @@ int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int
   return (int)gather_rows_launch(x, perm, k, out, (int)n, row_bytes, (hipStream_t)stream);
 }
 
-int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M,
-                                    int n, int K, int64_t ldy, void* stream) {
+static int grouped_gemm_swiglu_16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M, int n,
+                                  int K, int64_t ldy, bool fp16, void* stream) {
   if (G < 0 || M < 0 || n < 0 || K < 0) return MOE_GG_EINVAL;
   if (ldy < n) return MOE_GG_ESHAPE;
   if (G == 0 || M == 0 || n == 0) return MOE_GG_OK;
@@ -334,7 +334,18 @@ int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
   if (!moe_gg_two_list_fits(M, G, 256, (n + 127) / 128, num_wg)) return MOE_GG_EUNSUPPORTED;
+  p.fp16 = fp16 ? 1 : 0;
   return (int)gg_bf16_pingpong_swiglu_launch(p, num_wg, (hipStream_t)stream);
+}
+
+int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M,
+                                    int n, int K, int64_t ldy, void* stream) {
+  return grouped_gemm_swiglu_16(x, w, y, m_sizes, G, M, n, K, ldy, false, stream);
+}
+
+int moe_gg_grouped_gemm_swiglu_f16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M,
+                                   int n, int K, int64_t ldy, void* stream) {
+  return grouped_gemm_swiglu_16(x, w, y, m_sizes, G, M, n, K, ldy, true, stream);
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }

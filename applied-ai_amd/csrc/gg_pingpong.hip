@@ -85,9 +85,10 @@ constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x
 // OP_BF16_NT and both fragment kinds come from transposing reads. A tile reduces over the rows of its expert:
 // max(1, ceil(m_g / 64)) K steps; rows beyond the expert's last one re-read that row (the loads stay inside the
 // tensors), and group 0 overwrites them with zeros in the dY slab once it has landed, so they add nothing.
-// OP_F16: OP_BF16 on IEEE half data (the same kernel with the f16 MFMA and half conversions in the epilogue).
+// OP_F16, OP_F16_SWIGLU: OP_BF16 / OP_BF16_SWIGLU on IEEE half data (the same kernels with the f16 MFMA and half
+// conversions in the epilogue).
 constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4, OP_BF16_NT = 5,
-              OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7;
+              OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7, OP_F16_SWIGLU = 8;
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
 // 64 lanes x 16 B (or 4 B) from global memory straight into LDS: lane l's bytes land at lds_addr + 16 l
@@ -157,10 +158,10 @@ struct Cursor {
 template <int GRP, int OP>
 DEVINL void run_group(const GgParams& p, const Shared& sh) {
   constexpr bool FP8 = OP == OP_FP8_ROW || OP == OP_FP8_BLOCK;
-  constexpr bool F16 = OP == OP_F16;
+  constexpr bool F16 = OP == OP_F16 || OP == OP_F16_SWIGLU;
   constexpr bool BLOCK = OP == OP_FP8_BLOCK;
   constexpr bool WGRAD = OP == OP_BF16_WGRAD;
-  constexpr bool SWIGLU = OP == OP_BF16_SWIGLU;
+  constexpr bool SWIGLU = OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU;
   constexpr bool WG2 = OP == OP_BF16_WGRAD_DIRECT;
   constexpr bool WNT = OP == OP_BF16_NT || WG2;  // weight slab: 64 reduction rows by 256 columns (transposing reads)
   constexpr int TILE_COLS = SWIGLU ? BN / 2 : BN;  // output columns of a tile
@@ -540,17 +541,18 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
               const f32x4_t gv = acc[j][i], uv = acc[j + 2][i];
-              const uint32_t g01 = pack_bf16x2(gv[0], gv[1]), g23 = pack_bf16x2(gv[2], gv[3]);
-              const uint32_t u01 = pack_bf16x2(uv[0], uv[1]), u23 = pack_bf16x2(uv[2], uv[3]);
-              const float g[4] = {__builtin_bit_cast(float, g01 << 16), __builtin_bit_cast(float, g01 & 0xFFFF0000u),
-                                  __builtin_bit_cast(float, g23 << 16), __builtin_bit_cast(float, g23 & 0xFFFF0000u)};
-              const float u[4] = {__builtin_bit_cast(float, u01 << 16), __builtin_bit_cast(float, u01 & 0xFFFF0000u),
-                                  __builtin_bit_cast(float, u23 << 16), __builtin_bit_cast(float, u23 & 0xFFFF0000u)};
+              // both products rounded to the 16-bit type first, as they are when the GEMM output is stored
+              const uint32_t g01 = pack_16x2<F16>(gv[0], gv[1]), g23 = pack_16x2<F16>(gv[2], gv[3]);
+              const uint32_t u01 = pack_16x2<F16>(uv[0], uv[1]), u23 = pack_16x2<F16>(uv[2], uv[3]);
+              const float g[4] = {f32_of_16<F16>((uint16_t)g01), f32_of_16<F16>((uint16_t)(g01 >> 16)),
+                                  f32_of_16<F16>((uint16_t)g23), f32_of_16<F16>((uint16_t)(g23 >> 16))};
+              const float u[4] = {f32_of_16<F16>((uint16_t)u01), f32_of_16<F16>((uint16_t)(u01 >> 16)),
+                                  f32_of_16<F16>((uint16_t)u23), f32_of_16<F16>((uint16_t)(u23 >> 16))};
               float o[4];
 #pragma unroll
               for (int rr = 0; rr < 4; ++rr) o[rr] = g[rr] / (1.f + __expf(-g[rr])) * u[rr];
-              q[j][0] = pack_bf16x2(o[0], o[1]);
-              q[j][1] = pack_bf16x2(o[2], o[3]);
+              q[j][0] = pack_16x2<F16>(o[0], o[1]);
+              q[j][1] = pack_16x2<F16>(o[2], o[3]);
             }
             if (p.vec_store == 2 && cols_valid == TILE_COLS) {
               // 16-byte stores: lanes l and l ^ 16 trade halves as in the plain epilogue below.
@@ -672,7 +674,7 @@ DEVINL void pingpong_body(const GgParams& p) {
     build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
     total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
   } else {
-    const int ntn = OP == OP_BF16_SWIGLU ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
+    const int ntn = (OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU) ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
     const int skip = p.skip_rows;
     build_row_offsets(p.m_sizes, p.G, p.M, row_off);
     build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
@@ -707,7 +709,7 @@ DEVINL void pingpong_body(const GgParams& p) {
   const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
   for (int i = threadIdx.x; i < n_my; i += NT) {
     int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
-    constexpr int TC = OP == OP_BF16_SWIGLU ? BN / 2 : BN;  // output columns of a tile
+    constexpr int TC = (OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU) ? BN / 2 : BN;  // output columns of a tile
     int g, m0, h, n0, nc = TC;  // group, first row inside the group, rows, first column, columns
     if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
       // Tiles of an expert in bands of four column tiles, column tile fastest inside a band: the 32 tiles an XCD
@@ -767,6 +769,7 @@ __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_bo
 __global__ __launch_bounds__(NT) void gg_f16_pingpong(GgParams p) { pingpong_body<OP_F16>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
+__global__ __launch_bounds__(NT) void gg_f16_pingpong_swiglu(GgParams p) { pingpong_body<OP_F16_SWIGLU>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_nt(GgParams p) { pingpong_body<OP_BF16_NT>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad_direct(GgParams p) { pingpong_body<OP_BF16_WGRAD_DIRECT>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise(GgParams p) { pingpong_body<OP_FP8_ROW>(p); }
@@ -786,7 +789,8 @@ hipError_t gg_bf16_pingpong_wgrad_launch(const GgParams& p, int num_wg, hipStrea
 }
 
 hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  hipLaunchKernelGGL(gg_bf16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
+  if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
+  else hipLaunchKernelGGL(gg_bf16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -128,7 +128,7 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, t
     perm, m_sizes, offsets = route_group(ids, E)
     xs = gather_sorted(hidden_states, perm, k)
     swiglu_tiles = (xs.shape[0] // 256 + E) * ((two_n // 2 + 127) // 128)   # bound of the fused kernel's tile table
-    if (xs.dtype == torch.bfloat16 and xs.shape[0] >= FUSED_SWIGLU_MIN_ROWS and K % 64 == 0 and two_n % 8 == 0 and two_n * K < 2 ** 31
+    if (xs.shape[0] >= FUSED_SWIGLU_MIN_ROWS and K % 64 == 0 and two_n % 8 == 0 and two_n * K < 2 ** 31
             and swiglu_tiles <= 1023 * 256):
         h2 = grouped_gemm_swiglu(xs, w1.view(E * two_n, K), m_sizes)
     else:

@@ -98,15 +98,16 @@ def grouped_gemm_swiglu(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor)
         raise ValueError(f"w.shape[0]={w.shape[0]} is not a multiple of 2*G={2 * G}")
     n = w.shape[0] // (2 * G)
     assert K == w.shape[1], f"K mismatch: x has {K}, w has {w.shape[1]}"
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise ValueError("grouped_gemm_swiglu takes bf16 x and w")
+    if x.dtype not in (torch.bfloat16, torch.float16) or w.dtype != x.dtype:
+        raise ValueError("grouped_gemm_swiglu takes bf16 (or fp16) x and w of the same dtype")
     if m_sizes.dtype != torch.int32:
         raise ValueError("m_sizes must be int32")
     dev = _require_cuda(x, w, m_sizes)
-    y = torch.empty((M, n), device=dev, dtype=torch.bfloat16)
+    y = torch.empty((M, n), device=dev, dtype=x.dtype)
     with torch.cuda.device(dev):
-        rc = _lib.lib().moe_gg_grouped_gemm_swiglu_bf16(
-            x.data_ptr(), w.data_ptr(), y.data_ptr(), m_sizes.data_ptr(), G, M, n, K, n, _stream_ptr(dev))
+        L = _lib.lib()
+        fn = L.moe_gg_grouped_gemm_swiglu_f16 if x.dtype == torch.float16 else L.moe_gg_grouped_gemm_swiglu_bf16
+        rc = fn(x.data_ptr(), w.data_ptr(), y.data_ptr(), m_sizes.data_ptr(), G, M, n, K, n, _stream_ptr(dev))
     _lib.check(rc, "moe_gg_grouped_gemm_swiglu_bf16")
     return y
 

@@ -189,6 +189,9 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
  */
 int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M,
                                     int n, int K, int64_t ldy, void* stream);
+/* The same on IEEE half data. */
+int moe_gg_grouped_gemm_swiglu_f16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M,
+                                   int n, int K, int64_t ldy, void* stream);
 
 /*
  * Glue between the two grouped GEMMs of a whole MoE layer, as in the reference's fused_moe

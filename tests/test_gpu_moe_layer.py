@@ -255,3 +255,20 @@ def test_fused_moe_fp16_as_the_reference_test_runs_it(m):
             h = torch.nn.functional.silu(h[:n]) * h[n:]
             ref[t] += tw[t, j] * (h @ w2[ex].float().t())
     assert torch.allclose(y.float().cpu(), ref, atol=1e-2, rtol=0), float((y.float().cpu() - ref).abs().max())
+
+
+@pytest.mark.parametrize("sizes,n,K", [([300, 0, 41, 700], 256, 128), ([513, 64, 1], 1032, 256)])
+def test_swiglu_gemm_fp16_equals_gemm_then_silu_and_mul(sizes, n, K):
+    """The fp16 form of the fused kernel: bit-identical to the fp16 GEMM followed by the fp16 activation kernel."""
+    import applied_ai_amd as A
+
+    G, M = len(sizes), sum(sizes) + 5
+    gen = torch.Generator().manual_seed(78)
+    x = torch.randn(M, K, generator=gen).half()
+    w = (torch.randn(G * 2 * n, K, generator=gen) / 8).half()
+    m = torch.tensor(sizes, dtype=torch.int32)
+    fused = A.grouped_gemm_swiglu(x.cuda(), w.cuda(), m.cuda())
+    two = A.silu_and_mul(A.grouped_gemm(x.cuda(), w.cuda(), m.cuda()))
+    R = sum(sizes)
+    assert fused.dtype == torch.float16 and fused.shape == (M, n)
+    assert torch.equal(fused[:R].view(torch.int16), two[:R].view(torch.int16))
