@@ -51,6 +51,8 @@ def test_argument_errors_are_rejected_before_any_launch(lib):
 
 def test_argument_errors_of_the_other_entry_points(lib):
     """Every entry point validates sizes, enums and null pointers before it touches a device."""
+    one = ctypes.c_void_p(16)  # never dereferenced: the expert count is refused first
+    assert lib.moe_gg_grouped_gemm_bf16(one, one, one, one, 1025, 8, 128, 128, 128, 0, None) == -4   # more than 1024 experts
     assert lib.moe_gg_grouped_gemm_f16(None, None, None, None, 2, 8, 128, 128, 64, 0, None) == -2    # ldy < N
     assert lib.moe_gg_grouped_gemm_f16(None, None, None, None, 2, 8, 128, 128, 128, 0, None) == -1   # null pointers
     f8 = lib.moe_gg_grouped_gemm_fp8

@@ -214,3 +214,26 @@ def test_fp16_every_kernel_family(variant):
                 row += m
     finally:
         L.moe_gg_set_variant(0, -1)
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 2, 4, 5])
+def test_largest_expert_count(variant):
+    """G = 1024, the largest expert count the grouped kernels take (their in-LDS offset tables): many empty experts,
+    a few rows each otherwise; every kernel family against the oracle."""
+    import applied_ai_amd as A
+
+    L = A._lib.lib()
+    G, N, K = 1024, 128, 128
+    rng = np.random.default_rng(5)
+    ms = rng.integers(0, 9, size=G)
+    ms[rng.integers(0, G, size=300)] = 0
+    ms[[0, 511, 1023]] = [300, 260, 17]   # some row tiles at the first, a middle and the last expert
+    ms = [int(v) for v in ms]
+    x, w, _ = bf16_inputs(G, sum(ms), N, K, seed=6, w_std=0.25)
+    try:
+        L.moe_gg_set_variant(0, variant)
+        y = A.grouped_gemm(x.cuda(), w.cuda(), torch.tensor(ms, dtype=torch.int32, device="cuda"))
+    finally:
+        L.moe_gg_set_variant(0, -1)
+    ref = O.grouped_gemm(to_np(x), to_np(w), ms)
+    np.testing.assert_allclose(to_np(y), ref, rtol=RTOL, atol=ATOL)
