@@ -237,3 +237,38 @@ def test_largest_expert_count(variant):
         L.moe_gg_set_variant(0, -1)
     ref = O.grouped_gemm(to_np(x), to_np(w), ms)
     np.testing.assert_allclose(to_np(y), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("which", ["y", "x", "w"])
+def test_tensors_beyond_two_to_the_31_elements(which):
+    """Each operand in turn is larger than 2^31 elements (4 GB of bf16), so every row, column and expert offset of
+    that operand is exercised beyond 32 bits; sampled rows (the last ones among them) against an fp32 product."""
+    import applied_ai_amd as A
+
+    L = A._lib.lib()
+    if which == "y":      # output [70000, 32768]
+        G, ms, N, K, variants = 2, [35000, 35000], 32768, 64, (-1, 2)
+    elif which == "x":    # activations [40000, 65536]
+        G, ms, N, K, variants = 1, [40000], 64, 65536, (-1, 0)
+    else:                 # weights [64 * 1024, 32768 + 128]
+        G, ms, N, K, variants = 64, [4] * 64, 1024, 32768 + 128, (-1, 0)
+    M = sum(ms)
+    assert max(M * N, M * K, G * N * K) > 2 ** 31
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.empty((M, K), dtype=torch.bfloat16, device="cuda").normal_(generator=gen)
+    w = torch.empty((G * N, K), dtype=torch.bfloat16, device="cuda").normal_(std=0.05, generator=gen)
+    m = torch.tensor(ms, dtype=torch.int32, device="cuda")
+    rows = sorted(set([0, 1, M // 2, M - 2, M - 1] + torch.randint(0, M, (40,)).tolist()))
+    bounds = np.cumsum([0] + ms)
+    try:
+        for variant in variants:
+            L.moe_gg_set_variant(0, variant)
+            y = A.grouped_gemm(x, w, m)
+            torch.cuda.synchronize()
+            for r in rows:
+                g = int(np.searchsorted(bounds, r, side="right") - 1)
+                ref = x[r].float() @ w[g * N:(g + 1) * N].float().t()
+                assert torch.allclose(y[r].float(), ref, rtol=RTOL, atol=ATOL * 4), (which, variant, r)
+            del y
+    finally:
+        L.moe_gg_set_variant(0, -1)
