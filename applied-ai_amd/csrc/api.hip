@@ -137,7 +137,9 @@ static int grouped_gemm_16(const void* x, const void* w, void* y, const int32_t*
     const int64_t avg = (M + G - 1) / G;
     const int mf = avg <= 10 ? 1 : (avg <= 24 ? 2 : 4);
     int nf = ((int64_t)(N / 64) * G >= 4 * (int64_t)di->cus) ? 4 : 2;
-    if (mf == 4) nf = 2;
+    // One activation fragment per pass (up to 10 rows per expert on average): the narrow workgroups are 2-20 %
+    // faster on every shape measured (8-256 experts, N and K of 2048-14336), also when there are many of them.
+    if (mf == 4 || mf == 1) nf = 2;
     return (int)gg_bf16_decode_launch(p, nf, mf, s);
   }
   if (variant < 0) {
