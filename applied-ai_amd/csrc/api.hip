@@ -415,7 +415,7 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
     const int64_t ntn256 = (K + 255) / 256;
     const int64_t t256 = (M / 256 + (G + 1) / 2) * ntn256;
     const bool nt_ok = direct_shapes && N % 64 == 0 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg) &&
-                       t256 * 4 >= (int64_t)num_wg * 3;
+                       t256 * 5 >= (int64_t)num_wg * 2;
     if (nt_ok) {
       GgParams q{};
       q.x = grad_out; q.w = w; q.y = grad_x; q.m_sizes = m_sizes;
