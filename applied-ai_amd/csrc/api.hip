@@ -405,7 +405,8 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   const int v = g_variant[MOE_GG_OP_GG_BF16].load();
   const int x_col_block = grad_layout == MOE_GG_OUT_BLOCK ? N : 0;
   // Both gradients can be computed from the operands as stored (ping-pong kernels with transposing LDS reads)
-  // when there are enough 256 x 256 tiles and the row pitches allow 16-byte pieces; no workspace is touched then.
+  // when there are enough 256 x 256 tiles (see below) and the row pitches allow 16-byte pieces; no workspace is
+  // touched then.
   // Otherwise, or when a kernel variant is pinned, the operands are transposed into the workspace first.
   const bool direct_shapes = v < 0 && N % 8 == 0 && K % 8 == 0 && ld_go % 8 == 0 &&
                              ld_go < PINGPONG_MAX_ROW_BYTES / 2 && (int64_t)K < PINGPONG_MAX_ROW_BYTES / 2 &&
@@ -414,8 +415,10 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
     // grad_x = dY [M, N] times w[g] [N, K].
     const int64_t ntn256 = (K + 255) / 256;
     const int64_t t256 = (M / 256 + (G + 1) / 2) * ntn256;
+    // Almost always: the other way transposes all the weights first (254 -> 143 us at 8 experts x 32 rows,
+    // N = K = 4096); only calls of a few tiles are as fast or faster through the small-tile forward kernels.
     const bool nt_ok = direct_shapes && N % 64 == 0 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg) &&
-                       t256 * 5 >= (int64_t)num_wg * 2;
+                       t256 * 8 >= (int64_t)num_wg;
     if (nt_ok) {
       GgParams q{};
       q.x = grad_out; q.w = w; q.y = grad_x; q.m_sizes = m_sizes;
