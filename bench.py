@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # 1.94 GB fetched + 0.235 GB written.
 PREFILL_TRAFFIC_BYTES = 2.18e9
 # The same for the other workloads (profiles/bench_all_kernels_traffic.md): fetched + written bytes per launch.
-DECODE_TRAFFIC_BYTES = {"up": 0.951e9 + 1.8e6, "down": 0.957e9 + 0.5e6}
+DECODE_TRAFFIC_BYTES = {"up": 0.946e9 + 1.8e6, "down": 0.957e9 + 0.5e6}
 W4A16_TRAFFIC_BYTES = {1: 32.3e6 + 0.03e6, 16: 32.3e6 + 0.46e6, 64: 48.0e6 + 1.8e6}
 W4A16_GROUPED_TRAFFIC_BYTES = 254.2e6 + 1.8e6
 FP8_BLOCK_TRAFFIC_BYTES = 9.04e9 + 0.27e9
