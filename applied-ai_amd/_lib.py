@@ -46,6 +46,11 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int,
          _c_int, _c_void_p],
     ),
+    "moe_gg_w4a16_grouped_fp8out": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int,
+         _c_int, _c_int, _c_int, _c_void_p],
+    ),
     "moe_gg_route_topk": (_c_int, [_c_void_p, _c_i64, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "moe_gg_route_group": (_c_int, [_c_void_p, _c_i64, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "moe_gg_gather_rows": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_i64, _c_i64, _c_void_p]),

@@ -258,24 +258,43 @@ int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scale
   return (int)w4a16_splitk_launch(p, dtype == MOE_GG_DTYPE_FP16, (hipStream_t)stream);
 }
 
-int moe_gg_w4a16_grouped(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros, void* c,
-                         const int32_t* m_sizes, int G, int64_t M, int N, int K, int group_size, int zero_offset,
-                         int dtype, void* stream) {
+static int w4a16_grouped_any(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros, void* c,
+                            void* c_q, float* c_scale, bool fp8out, const int32_t* m_sizes, int G, int64_t M, int N,
+                            int K, int group_size, int zero_offset, int dtype, void* stream) {
   if (G < 0 || M < 0 || N < 0 || K < 0 || group_size <= 0) return MOE_GG_EINVAL;
   if (zero_offset != 0 && zero_offset != 1) return MOE_GG_EINVAL;
   if (dtype != MOE_GG_DTYPE_BF16 && dtype != MOE_GG_DTYPE_FP16) return MOE_GG_EINVAL;
   if (G == 0 || M == 0 || N == 0) return MOE_GG_OK;
-  if (!a || !qweight || !scales || !qzeros || !c || !m_sizes) return MOE_GG_EINVAL;
+  if (!a || !qweight || !scales || !qzeros || !m_sizes) return MOE_GG_EINVAL;
+  if (fp8out ? (!c_q || !c_scale) : !c) return MOE_GG_EINVAL;
   if (K == 0 || K % group_size != 0 || K % 8 != 0 || N % 8 != 0) return MOE_GG_ESHAPE;
-  if (group_size % 32 != 0 || N % 64 != 0 || G > 65535 || M > INT32_MAX) return MOE_GG_EUNSUPPORTED;
-  if (!aligned(a, 16) || !aligned(qweight, 16) || !aligned(scales, 16) || !aligned(qzeros, 8) || !aligned(c, 2) ||
-      !aligned(m_sizes, 4))
+  if (group_size % 32 != 0 || N % (fp8out ? 128 : 64) != 0 || G > 65535 || M > INT32_MAX) return MOE_GG_EUNSUPPORTED;
+  if (!aligned(a, 16) || !aligned(qweight, 16) || !aligned(scales, 16) || !aligned(qzeros, 8) || !aligned(m_sizes, 4))
     return MOE_GG_EALIGN;
+  if (fp8out ? !aligned(c_scale, 4) : !aligned(c, 2)) return MOE_GG_EALIGN;
   const DeviceInfo* di = nullptr;
   int rc = current_device_info(&di);
   if (rc != MOE_GG_OK) return rc;
-  W4Params p{a, qweight, scales, qzeros, c, (int)M, N, K, group_size, zero_offset, m_sizes, G};
+  W4Params p{a, qweight, scales, qzeros, fp8out ? nullptr : c, (int)M, N, K, group_size, zero_offset, m_sizes, G};
+  if (fp8out) {
+    p.cq = c_q;
+    p.cscale = c_scale;
+  }
   return (int)w4a16_splitk_launch(p, dtype == MOE_GG_DTYPE_FP16, (hipStream_t)stream);
+}
+
+int moe_gg_w4a16_grouped(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros, void* c,
+                         const int32_t* m_sizes, int G, int64_t M, int N, int K, int group_size, int zero_offset,
+                         int dtype, void* stream) {
+  return w4a16_grouped_any(a, qweight, scales, qzeros, c, nullptr, nullptr, false, m_sizes, G, M, N, K, group_size,
+                           zero_offset, dtype, stream);
+}
+
+int moe_gg_w4a16_grouped_fp8out(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                                void* c_q, float* c_scale, const int32_t* m_sizes, int G, int64_t M, int N, int K,
+                                int group_size, int zero_offset, int dtype, void* stream) {
+  return w4a16_grouped_any(a, qweight, scales, qzeros, nullptr, c_q, c_scale, true, m_sizes, G, M, N, K, group_size,
+                           zero_offset, dtype, stream);
 }
 
 int moe_gg_route_topk(const float* logits, int64_t T, int E, int k, int32_t* ids, int32_t* perm, int32_t* m_sizes,

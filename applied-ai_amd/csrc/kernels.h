@@ -57,6 +57,10 @@ struct W4Params {
   // qweight [G, K/8, N], scales [G, K/group_size, N], qzeros [G, K/group_size, N/8]; M is the total row count.
   const int32_t* m_sizes;
   int G;
+  // fp8 output instead of c (c may be nullptr then): cq [M, N] e4m3fn and cscale [M, N/128] fp32, the 1 x 128
+  // group-wise quantisation of the 16-bit result; needs N % 128 == 0.
+  void* cq = nullptr;
+  float* cscale = nullptr;
 };
 hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream);
 

@@ -21,6 +21,11 @@
 //   total += s * (acc_group - (BIAS + z + zero_offset) * S).
 // With the four words of a lane feeding four MFMAs, a lane ends up with 16 consecutive output
 // columns of one output row.
+//
+// Quantised output (QOUT kernels, W4Params::cq != nullptr): a workgroup does two adjacent 64-column blocks one
+// after the other and, instead of storing 16-bit values, quantises each row's 128 results to fp8 e4m3fn with one
+// fp32 scale - float8_groupwise_quantize (kernels/triton/inference/fp8/float8_groupwise_quant.py:20-50) applied to
+// the 16-bit result, bit for bit, without the round trip of that result through memory.
 #include "common.h"
 #include "kernels.h"
 
@@ -61,11 +66,13 @@ struct W4View {
   const int32_t* qzeros;
   uint16_t* c;
   int M;
+  uint8_t* cq;    // QOUT: [M, N] e4m3fn
+  float* cscale;  // QOUT: [M, N/128]
 };
 
 // Must be called by every thread of the workgroup (it contains a barrier in grouped mode).
 DEVINL W4View w4_view(const W4Params& p) {
-  W4View v{(const uint16_t*)p.a, p.qweight, (const uint16_t*)p.scales, p.qzeros, (uint16_t*)p.c, p.M};
+  W4View v{(const uint16_t*)p.a, p.qweight, (const uint16_t*)p.scales, p.qzeros, (uint16_t*)p.c, p.M, (uint8_t*)p.cq, p.cscale};
   if (p.m_sizes == nullptr) return v;
   __shared__ int s_row0, s_rows;
   const int g = blockIdx.y;
@@ -90,18 +97,63 @@ DEVINL W4View w4_view(const W4Params& p) {
   const int ngroups = p.K / p.group_size;
   v.M = s_rows;
   v.a += (int64_t)row0 * p.K;
-  v.c += (int64_t)row0 * p.N;
+  if (v.c) v.c += (int64_t)row0 * p.N;
+  if (v.cq) {
+    v.cq += (int64_t)row0 * p.N;
+    v.cscale += (int64_t)row0 * (p.N / 128);
+  }
   v.qweight += (int64_t)g * (p.K / 8) * p.N;
   v.scales += (int64_t)g * ngroups * p.N;
   v.qzeros += (int64_t)g * ngroups * (p.N / 8);
   return v;
 }
 
+// Sum the waves' partial results of rows mb .. mb + 16 MF - 1 x columns n0 .. n0 + 63 (red[wave][i][m_local * 64 +
+// col]) in a fixed order and store them. A wave takes one row per pass, a lane one column. QOUT: column block 0
+// (cb = 0) only keeps its values, rounded to the 16-bit type; column block 1 then has each row's 128 values in one
+// wave (two per lane) and quantises them as fp8_groupwise_quant_kernel (quant.hip) does.
+template <bool FP16, bool QOUT, int MF, int NW>
+DEVINL void w4_reduce_store(const float (&red)[NW][MF][16 * 64], const W4View& v, int N, int mb, int n0, int cb,
+                            float (&keep)[2 * MF]) {
+  using E = Elem<FP16>;
+  static_assert(NW == 8, "one row per wave and pass: 16 MF rows in 2 MF passes");
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rows_here = min(v.M - mb, 16 * MF);
+#pragma unroll
+  for (int k = 0; k < 2 * MF; ++k) {
+    const int ml = wave + NW * k;
+    if (ml >= rows_here) continue;  // the same for all lanes of a wave
+    const int i = ml / 16, rem = (ml % 16) * 64 + lane;
+    float sum = red[0][i][rem];
+#pragma unroll
+    for (int w2 = 1; w2 < NW; ++w2) sum += red[w2][i][rem];
+    const uint16_t h = E::from_f32(sum);
+    if (!QOUT) {
+      if (n0 + lane < N) v.c[(int64_t)(mb + ml) * N + n0 + lane] = h;
+    } else if (cb == 0) {
+      keep[k] = E::to_f32(h);
+    } else {
+      const float a = keep[k], b = E::to_f32(h);
+      float amax = fmaxf(fabsf(a), fabsf(b));
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d, 64));
+      const float s = fmaxf(amax, 1e-12f) / 448.0f;
+      const float ya = fminf(fmaxf(a / s, -448.0f), 448.0f);
+      const float yb = fminf(fmaxf(b / s, -448.0f), 448.0f);
+      const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(ya, yb, 0, false);
+      uint8_t* q = v.cq + (int64_t)(mb + ml) * N + (n0 - 64) + lane;
+      q[0] = (uint8_t)(packed & 0xFF);
+      q[64] = (uint8_t)((packed >> 8) & 0xFF);
+      if (lane == 0) v.cscale[(int64_t)(mb + ml) * (N / 128) + (n0 - 64) / 128] = s;
+    }
+  }
+}
+
 constexpr int WAVES = 8;
 constexpr int DEPTH = 8;  // K steps of qweight loads in flight per wave
 
 // Any group size that is a multiple of 32; scales / zeros are loaded where they are used.
-template <bool FP16, int MF>
+template <bool FP16, int MF, bool QOUT>
 __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) {
   using E = Elem<FP16>;
   __shared__ __attribute__((aligned(16))) float red[WAVES][MF][64 * 16];
@@ -112,7 +164,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
   const int fr = lane & 15, fq = lane >> 4;
   const W4View v = w4_view(p);
   const int N = p.N, K = p.K, M = v.M;
-  const int n0 = blockIdx.x * 64;
+  constexpr int CB = QOUT ? 2 : 1;                 // 64-column blocks per workgroup
   const int spg = p.group_size / 32;               // K steps per quantisation group
   const int ngroups = K / p.group_size;
   const int my_groups = ngroups > wave ? (ngroups - wave + WAVES - 1) / WAVES : 0;
@@ -121,14 +173,16 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
   // step t of this wave -> absolute K step
   auto kstep = [&](int t) { return ((t / spg) * WAVES + wave) * spg + t % spg; };
 
-  // qweight: lane reads words of columns n0 + 4*fr .. + 3 (clamped at the right edge), k-word row 4*step + fq
-  const int wcol = min(n0 + 4 * fr, N - 4);
-  const int32_t* qw = v.qweight + wcol;
-  // output / scale columns of this lane: n0 + 16*fq + 0..15
-  const int ocol = n0 + 16 * fq;
-  const int ocol_c = min(ocol, N - 16 >= 0 ? N - 16 : 0);
-
-  for (int mb = 0; mb < M; mb += 16 * MF) {
+  float keep[2 * MF];
+  for (int mb = 0; mb < M; mb += 16 * MF)
+  for (int cb = 0; cb < CB; ++cb) {
+    const int n0 = (blockIdx.x * CB + cb) * 64;
+    // qweight: lane reads words of columns n0 + 4*fr .. + 3 (clamped at the right edge), k-word row 4*step + fq
+    const int wcol = min(n0 + 4 * fr, N - 4);
+    const int32_t* qw = v.qweight + wcol;
+    // output / scale columns of this lane: n0 + 16*fq + 0..15
+    const int ocol = n0 + 16 * fq;
+    const int ocol_c = min(ocol, N - 16 >= 0 ? N - 16 : 0);
     const uint16_t* arow[MF];
 #pragma unroll
     for (int i = 0; i < MF; ++i) arow[i] = v.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
@@ -215,14 +269,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
 #pragma unroll
         for (int ii = 0; ii < 4; ++ii) red[wave][i][fr * 64 + 16 * fq + 4 * ii + j] = total[i][j][ii];
     __syncthreads();
-    for (int o = tid; o < MF * 16 * 64; o += 64 * WAVES) {
-      const int i = o / 1024, rem = o % 1024;
-      const int m = mb + i * 16 + rem / 64, n = n0 + rem % 64;
-      float sum = red[0][i][rem];
-#pragma unroll
-      for (int w2 = 1; w2 < WAVES; ++w2) sum += red[w2][i][rem];
-      if (m < M && n < N) v.c[(int64_t)m * N + n] = E::from_f32(sum);
-    }
+    w4_reduce_store<FP16, QOUT, MF, WAVES>(red, v, N, mb, n0, cb, keep);
     __syncthreads();
   }
 }
@@ -236,7 +283,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
 // 4 * (lane / 16) + r of the four adjacent columns n0 + 4 * (lane % 16) + j of its own qweight words. It
 // then needs just four scales and four zero points per group (one 8-byte and one 4-byte load), and the
 // fold costs a quarter of the vector instructions of the 16-columns-per-lane layout.
-template <bool FP16, int MF, int GA, int NWAVES>  // GA = groups kept in flight
+template <bool FP16, int MF, int GA, int NWAVES, bool QOUT>  // GA = groups kept in flight
 __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
   using E = Elem<FP16>;
   constexpr int SPG = 4, D = SPG * GA;
@@ -248,42 +295,45 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
   const int fr = lane & 15, fq = lane >> 4;
   const W4View v = w4_view(p);
   const int N = p.N, K = p.K, M = v.M;
-  const int n0 = blockIdx.x * 64;
+  constexpr int CB = QOUT ? 2 : 1;                      // 64-column blocks per workgroup
   const int ngroups = K / 128;
   const int my_groups = ngroups > wave ? (ngroups - wave + NWAVES - 1) / NWAVES : 0;
   const int steps = my_groups * SPG;
   auto kstep = [&](int t) { return ((t / SPG) * NWAVES + wave) * SPG + t % SPG; };
 
-  const int32_t* qw = v.qweight + n0 + 4 * fr;          // k-word row 4 * step + fq, columns n0 + 4 fr .. + 3
-  const uint16_t* sc = v.scales + n0 + 4 * fr;
-  const int32_t* zp = v.qzeros + (n0 + 4 * fr) / 8;
   const int zshift = 16 * (fr & 1);                     // the lane's four zero nibbles inside the word
 
-  for (int mb = 0; mb < M; mb += 16 * MF) {
-    const uint16_t* arow[MF];
+  // One pass = 16 MF rows x one 64-column block over the whole K. The first loads of the next pass are issued
+  // before the cross-wave reduction of the current one, so the load queue does not run dry between passes.
+  const int passes = (M + 16 * MF - 1) / (16 * MF) * CB;
+  if (passes == 0) return;  // an expert without rows (the same for the whole workgroup)
+  const int32_t* qw;        // k-word row 4 * step + fq, columns n0 + 4 fr .. + 3
+  const uint16_t* sc;
+  const int32_t* zp;
+  const uint16_t* arow[MF];
+  auto setup = [&](int pass) {
+    const int mb = pass / CB * (16 * MF), n0 = (blockIdx.x * CB + pass % CB) * 64;
+    qw = v.qweight + n0 + 4 * fr;
+    sc = v.scales + n0 + 4 * fr;
+    zp = v.qzeros + (n0 + 4 * fr) / 8;
 #pragma unroll
     for (int i = 0; i < MF; ++i) arow[i] = v.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
-
-    f32x4_t total[MF][4];  // [row fragment i][column j]: rows mb + 16 i + 4 fq + r
+  };
+  u32x4_t wb[D], xr[D][MF];
+  u32x2_t sg[GA];
+  uint32_t zg[GA];
+  auto load_step = [&](int d, int t) {
+    const int ks = kstep(t);
+    wb[d] = *(const u32x4_t*)(qw + (int64_t)(ks * 4 + fq) * N);
 #pragma unroll
-    for (int i = 0; i < MF; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) total[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-    u32x4_t wb[D], xr[D][MF];
-    u32x2_t sg[GA];
-    uint32_t zg[GA];
-    auto load_step = [&](int d, int t) {
-      const int ks = kstep(t);
-      wb[d] = *(const u32x4_t*)(qw + (int64_t)(ks * 4 + fq) * N);
-#pragma unroll
-      for (int i = 0; i < MF; ++i) xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
-    };
-    auto load_group = [&](int q, int gi) {  // gi = index among this wave's groups
-      const int64_t g = (int64_t)gi * NWAVES + wave;
-      sg[q] = *(const u32x2_t*)(sc + g * N);
-      zg[q] = (uint32_t)zp[g * (N / 8)];
-    };
+    for (int i = 0; i < MF; ++i) xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
+  };
+  auto load_group = [&](int q, int gi) {  // gi = index among this wave's groups
+    const int64_t g = (int64_t)gi * NWAVES + wave;
+    sg[q] = *(const u32x2_t*)(sc + g * N);
+    zg[q] = (uint32_t)zp[g * (N / 8)];
+  };
+  auto first_loads = [&]() {
 #pragma unroll
     for (int q = 0; q < GA; ++q) {
 #pragma unroll
@@ -291,6 +341,18 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
         if (q * SPG + e < steps) load_step(q * SPG + e, q * SPG + e);
       if (q < my_groups) load_group(q, q);
     }
+  };
+  setup(0);
+  first_loads();
+
+  float keep[2 * MF];
+  for (int pass = 0; pass < passes; ++pass) {
+    const int mb = pass / CB * (16 * MF), cb = pass % CB, n0 = (blockIdx.x * CB + cb) * 64;
+    f32x4_t total[MF][4];  // [row fragment i][column j]: rows mb + 16 i + 4 fq + r
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) total[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     for (int g0 = 0; g0 < my_groups; g0 += GA) {
 #pragma unroll
@@ -349,6 +411,10 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
       }
     }
 
+    if (pass + 1 < passes) {
+      setup(pass + 1);
+      first_loads();
+    }
     // Cross-wave (split-K) reduction in a fixed order: red[wave][i][m_local * 64 + col_local].
 #pragma unroll
     for (int i = 0; i < MF; ++i)
@@ -356,38 +422,33 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
       for (int r = 0; r < 4; ++r)
         *(f32x4_t*)&red[wave][i][(4 * fq + r) * 64 + 4 * fr] = f32x4_t{total[i][0][r], total[i][1][r], total[i][2][r], total[i][3][r]};
     __syncthreads();
-    const int rows_here = min(M - mb, 16 * MF);
-    for (int o = tid; o < rows_here * 64; o += 64 * NWAVES) {
-      const int ml = o / 64, col = o % 64;
-      const int i = ml / 16, rem = (ml % 16) * 64 + col;
-      float sum = red[0][i][rem];
-#pragma unroll
-      for (int w2 = 1; w2 < NWAVES; ++w2) sum += red[w2][i][rem];
-      if (n0 + col < N) v.c[(int64_t)(mb + ml) * N + n0 + col] = E::from_f32(sum);
-    }
+    w4_reduce_store<FP16, QOUT, MF, NWAVES>(red, v, N, mb, n0, cb, keep);
     __syncthreads();
   }
 }
 
-template <bool FP16>
+template <bool FP16, bool QOUT>
 hipError_t launch(const W4Params& p, hipStream_t stream) {
   // Grouped call: one grid row per expert; the kernel variant follows the average rows per expert (an
   // expert with more rows than one pass covers is done in several passes over its weights).
-  dim3 grid((p.N + 63) / 64, p.m_sizes ? p.G : 1), block(64 * WAVES);
+  // (fp8 output: 128 columns per workgroup, N % 128 == 0 checked by the caller.)
+  dim3 grid(QOUT ? p.N / 128 : (p.N + 63) / 64, p.m_sizes ? p.G : 1), block(64 * WAVES);
   const int M = p.m_sizes ? (p.M + p.G - 1) / p.G : p.M;
   // Group size 128: one activation fragment per pass for M <= 16, two for more rows (32 rows per pass over the
   // weights; four fragments do not fit the registers), all loads issued one group ahead (deeper queues and
-  // more waves measured slower). Other group sizes: up to four activation fragments per pass.
-  if (M <= 16 && p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES>), grid, block, 0, stream, p);
-  else if (p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 2, 1, WAVES>), grid, block, 0, stream, p);
-  else if (M <= 16) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 1>), grid, block, 0, stream, p);
-  else if (M <= 32) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 2>), grid, block, 0, stream, p);
-  else hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 4>), grid, block, 0, stream, p);
+  // more waves measured slower). Other group sizes: up to four activation fragments per pass (two with fp8
+  // output, whose kept values of the first column block need registers too).
+  if (M <= 16 && p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES, QOUT>), grid, block, 0, stream, p);
+  else if (p.group_size == 128) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 2, 1, WAVES, QOUT>), grid, block, 0, stream, p);
+  else if (M <= 16) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 1, QOUT>), grid, block, 0, stream, p);
+  else if (M <= 32 || QOUT) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 2, QOUT>), grid, block, 0, stream, p);
+  else if constexpr (!QOUT) hipLaunchKernelGGL((w4a16_splitk_anygroup<FP16, 4, false>), grid, block, 0, stream, p);
   return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream) {
-  return fp16 ? launch<true>(p, stream) : launch<false>(p, stream);
+  if (p.cq) return fp16 ? launch<true, true>(p, stream) : launch<false, true>(p, stream);
+  return fp16 ? launch<true, false>(p, stream) : launch<false, false>(p, stream);
 }

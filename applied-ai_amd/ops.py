@@ -204,8 +204,13 @@ small_qlinear = a100_qlinear
 
 
 def matmul_split_k_grouped(a: torch.Tensor, b: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
-                           m_sizes: torch.Tensor, zero_offset: int = 1, groupsize: Optional[int] = None) -> torch.Tensor:
+                           m_sizes: torch.Tensor, zero_offset: int = 1, groupsize: Optional[int] = None,
+                           quantize_output: bool = False):
     """W4A16 grouped GEMM over expert-sorted rows: c[rows of expert g] = a[rows of g] @ dequant(b[g], scales[g], zeros[g]).
+
+    quantize_output=True returns float8_groupwise_quantize(c)
+    (kernels/triton/inference/fp8/float8_groupwise_quant.py:53-91) instead of c - (q [M, N] float8_e4m3fn, scales
+    [M, N/128] fp32), computed in the GEMM's epilogue; needs N % 128 == 0. Rows beyond sum(m_sizes) are zero then.
 
     The GEMM of the reference's W4A16 fused MoE kernel
     (kernels/triton/inference/gptq/mixtral/w4a16_fused_dequant_gemm.py:49-149) without its padded token lists:
@@ -226,6 +231,18 @@ def matmul_split_k_grouped(a: torch.Tensor, b: torch.Tensor, scales: torch.Tenso
         raise ValueError("scales must be [E, K/g, N], zeros [E, K/g, N/8], m_sizes [E]")
     dev = _require_cuda(a, b, scales, zeros, m_sizes)
     a, b, scales, zeros, m_sizes = a.contiguous(), b.contiguous(), scales.contiguous(), zeros.contiguous(), m_sizes.contiguous()
+    if quantize_output:
+        if n % 128 != 0:
+            raise ValueError(f"quantize_output needs N % 128 == 0, got N = {n}")
+        q = torch.zeros((m, n), device=dev, dtype=torch.float8_e4m3fn)
+        qs = torch.zeros((m, n // 128), device=dev, dtype=torch.float32)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().moe_gg_w4a16_grouped_fp8out(
+                a.data_ptr(), b.data_ptr(), scales.data_ptr(), zeros.data_ptr(), q.data_ptr(), qs.data_ptr(),
+                m_sizes.data_ptr(), e, m, n, k, g, zero_offset, 1 if a.dtype == torch.float16 else 0, _stream_ptr(dev),
+            )
+        _lib.check(rc, "moe_gg_w4a16_grouped_fp8out")
+        return q, qs
     c = torch.empty((m, n), device=dev, dtype=a.dtype)
     with torch.cuda.device(dev):
         rc = _lib.lib().moe_gg_w4a16_grouped(

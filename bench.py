@@ -179,6 +179,30 @@ def secondary_workloads(torch, A, dev):
                 "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128 (grid.y = experts)", "achieved": round(byt / ms / 1e6, 1),
                              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
                              "traffic": W4A16_GROUPED_TRAFFIC_BYTES}})
+
+    # the same call with the 1 x 128 fp8 quantiser as its epilogue, beside the two launches it replaces
+    cq = torch.empty(64, N, device=dev, dtype=torch.uint8)
+    cs = torch.empty(64, N // 128, device=dev, dtype=torch.float32)
+
+    def call_q():
+        q = qwe[state["i"] & 1]
+        state["i"] += 1
+        lib.moe_gg_w4a16_grouped_fp8out(a.data_ptr(), q.data_ptr(), sce.data_ptr(), qze.data_ptr(), cq.data_ptr(),
+                                        cs.data_ptr(), ms3.data_ptr(), E, 64, N, K, 128, 0, 0, stream)
+
+    def call_two():
+        call()
+        lib.moe_gg_fp8_groupwise_quant(c.data_ptr(), 0, cq.data_ptr(), cs.data_ptr(), 64 * N, stream)
+
+    ms_q = event_time_ms(torch, call_q, 40, 6)
+    ms_two = event_time_ms(torch, call_two, 40, 6)
+    byt_q = byt - 64 * N * 2 + 64 * N + 64 * (N // 128) * 4
+    out.append({"workload": f"W4A16 grouped GEMM with the fp8 1x128 quantiser as epilogue, same shape (fp8 codes + scales out)",
+                "us_per_launch": round(ms_q * 1e3, 2), "gemm_then_quantiser_us": round(ms_two * 1e3, 2),
+                "value": round(byt_q / ms_q / 1e6, 1), "unit": "GB/s",
+                "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128 (fp8 output)", "achieved": round(byt_q / ms_q / 1e6, 1),
+                             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt_q / ms_q / 1e6 / PEAK_HBM_GBS, 4),
+                             "traffic": None}})
     del qwe
 
     # ---- config 5: DeepSeek-V3-style fp8 block-scaled, 256 experts top-8, Zipf(1.1) routing ----

@@ -120,6 +120,20 @@ int moe_gg_w4a16_grouped(const void* a, const int32_t* qweight, const void* scal
                          const int32_t* m_sizes, int G, int64_t M, int N, int K, int group_size, int zero_offset,
                          int dtype, void* stream);
 
+/*
+ * The same grouped W4A16 GEMM with the 1 x 128 fp8 activation quantiser as its epilogue: instead of the 16-bit
+ * result c it stores float8_groupwise_quantize(c) (kernels/triton/inference/fp8/float8_groupwise_quant.py:20-50,
+ * 53-91), ready to be the x / x_scale of moe_gg_grouped_gemm_fp8 with MOE_GG_SCALE_BLOCK128. The reference runs
+ * the quantiser as a kernel of its own on a result read back from memory (float8_groupwise_quant.py:53-91); here
+ * the 16-bit result never leaves the chip. Bit-identical to moe_gg_w4a16_grouped followed by
+ * moe_gg_fp8_groupwise_quant.
+ *   c_q device [M, N] e4m3fn; c_scale device fp32 [M, N/128]; everything else as for moe_gg_w4a16_grouped,
+ *   and N % 128 == 0. Rows >= sum(m_sizes) of c_q and c_scale are not written.
+ */
+int moe_gg_w4a16_grouped_fp8out(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                                void* c_q, float* c_scale, const int32_t* m_sizes, int G, int64_t M, int N, int K,
+                                int group_size, int zero_offset, int dtype, void* stream);
+
 #define MOE_GG_MAX_ROUTE_EXPERTS 768
 
 /*

@@ -70,6 +70,11 @@ def test_argument_errors_of_the_other_entry_points(lib):
     assert w4g(None, None, None, None, None, None, -1, 4, 64, 128, 128, 1, 0, None) == -1
     assert w4g(None, None, None, None, None, None, 2, 4, 64, 128, 128, 1, 0, None) == -1    # null pointers
     assert w4g(None, None, None, None, None, None, 2, 0, 64, 128, 128, 1, 0, None) == 0     # no rows
+    w4q = lib.moe_gg_w4a16_grouped_fp8out
+    assert w4q(None, None, None, None, None, None, None, 2, 4, 128, 128, 128, 1, 2, None) == -1   # fp32 is no W4A16 dtype
+    assert w4q(None, None, None, None, None, None, None, 2, 4, 128, 128, 128, 1, 0, None) == -1   # null pointers
+    assert w4q(None, None, None, None, None, None, None, 2, 0, 128, 128, 128, 1, 0, None) == 0    # no rows
+    assert w4q(one, one, one, one, one, one, one, 2, 4, 192, 128, 128, 1, 0, None) == -4          # N % 128 != 0
     assert lib.moe_gg_route_topk(None, 4, 8, 9, None, None, None, None, None) == -1         # k > E
     assert lib.moe_gg_route_topk(None, 4, 1000, 2, None, None, None, None, None) == -4      # E too large
     assert lib.moe_gg_route_group(None, 4, 0, None, None, None, None) == -1

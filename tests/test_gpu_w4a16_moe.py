@@ -48,6 +48,75 @@ def test_grouped_against_oracle(dtype, E, K, N, gs, zo, m_sizes):
     assert rel_fro(to_np(c)[:R], ref[:R]) <= TOL
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("E,K,N,gs,zo,m_sizes", [
+    (4, 256, 128, 128, 1, [3, 0, 16, 1]),
+    (8, 512, 256, 128, 0, [9, 7, 10, 6, 4, 6, 11, 11]),
+    (3, 256, 384, 64, 1, [17, 40, 2]),
+    (2, 1152, 128, 128, 1, [70, 5]),
+    (5, 256, 128, 32, 0, [0, 0, 33, 0, 1]),
+    (8, 4096, 1024, 128, 1, [1, 2, 0, 3, 1, 0, 0, 1]),
+])
+def test_grouped_fp8_output(dtype, E, K, N, gs, zo, m_sizes):
+    """The quantiser as the GEMM's epilogue: (1) bit-identical to the GEMM followed by float8_groupwise_quantize,
+    the two launches it replaces; (2) against the oracle chain (W4A16 product, rounded to the 16-bit type, 1 x 128
+    quantiser): the GPU's fp32 summation order differs, so a few results land on the other side of a rounding
+    boundary - dequantised values within the fp8 / W4A16 bar (relative Frobenius 2e-2) of the oracle chain's;
+    (3) against the unquantised oracle product the error is that of e4m3 itself (3 mantissa bits: 2^-4 / sqrt(3) =
+    3.6 % rms), bound 5e-2 here."""
+    import applied_ai_amd as A
+
+    print(f"case {dtype} E={E} K={K} N={N} group={gs} zero_offset={zo} m_sizes={m_sizes}", flush=True)
+    rng = np.random.default_rng(E * 37 + K + N)
+    qw, qz, sc = make_experts(rng, E, K, N, gs)
+    scales = torch.from_numpy(sc).to(dtype)
+    R = sum(m_sizes)
+    M = R + 3
+    a = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    args = (a.cuda(), torch.from_numpy(qw).cuda(), scales.cuda(), torch.from_numpy(qz).cuda(),
+            torch.tensor(m_sizes, dtype=torch.int32).cuda())
+    q, s = A.matmul_split_k_grouped(*args, zero_offset=zo, groupsize=gs, quantize_output=True)
+    c = A.matmul_split_k_grouped(*args, zero_offset=zo, groupsize=gs)
+    q2, s2 = A.float8_groupwise_quantize(c[:R] if dtype == torch.bfloat16 else c[:R].float())
+    torch.cuda.synchronize()
+    assert q.dtype == torch.float8_e4m3fn and q.shape == (M, N) and s.shape == (M, N // 128) and s.dtype == torch.float32
+    assert torch.equal(q.view(torch.uint8)[:R], q2.view(torch.uint8))
+    assert torch.equal(s[:R], s2)
+    assert int(q.view(torch.uint8)[R:].max()) == 0 and float(s[R:].abs().max()) == 0.0  # rows of no expert: not written
+
+    ref = O.w4a16_grouped(to_np(a), qw, to_np(scales), qz, m_sizes, gs, zo)[:R]
+    ref16 = O.round_bf16(ref) if dtype == torch.bfloat16 else ref.astype(np.float16).astype(np.float32)
+    oq, osc = O.fp8_groupwise_quant(ref16)
+    deq = O.e4m3_to_f32(q.view(torch.uint8)[:R].cpu().numpy()) * np.repeat(s[:R].cpu().numpy(), 128, axis=1)
+    odeq = O.e4m3_to_f32(oq) * np.repeat(osc, 128, axis=1)
+    assert rel_fro(deq, odeq) <= TOL
+    np.testing.assert_allclose(s[:R].cpu().numpy(), osc, rtol=1e-2)
+    assert rel_fro(deq, ref) <= 5e-2
+
+
+def test_grouped_fp8_output_feeds_the_fp8_grouped_gemm():
+    """What the epilogue is for: its (q, scales) are the x / x_scale of the block-scaled fp8 grouped GEMM."""
+    import applied_ai_amd as A
+
+    rng = np.random.default_rng(77)
+    E, K, N, N2, gs = 4, 512, 256, 128, 128
+    m_sizes = [5, 0, 20, 7]
+    R = sum(m_sizes)
+    qw, qz, sc = make_experts(rng, E, K, N, gs)
+    scales = torch.from_numpy(sc).to(torch.bfloat16)
+    a = torch.from_numpy(rng.standard_normal((R, K)).astype(np.float32)).to(torch.bfloat16)
+    ms = torch.tensor(m_sizes, dtype=torch.int32).cuda()
+    q, s = A.matmul_split_k_grouped(a.cuda(), torch.from_numpy(qw).cuda(), scales.cuda(), torch.from_numpy(qz).cuda(), ms,
+                                    zero_offset=1, quantize_output=True)
+    w2 = torch.from_numpy((rng.standard_normal((E * N2, N)) * 0.05).astype(np.float32))
+    w2q, w2s = A.float8_blockwise_quantize_weight(w2)
+    y = A.grouped_gemm_fp8_blockwise(q, w2q.cuda(), ms, s, w2s.cuda())
+    torch.cuda.synchronize()
+    ref = O.grouped_gemm_fp8(q.view(torch.uint8).cpu().numpy(), w2q.view(torch.uint8).numpy(), s.cpu().numpy(), w2s.numpy(),
+                             m_sizes, 1)
+    assert rel_fro(to_np(y), ref) <= TOL
+
+
 def test_grouped_equals_dense_call_per_expert_bitwise():
     """One expert of a grouped call must give exactly what the dense entry point gives for the same rows."""
     import applied_ai_amd as A
