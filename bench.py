@@ -147,9 +147,15 @@ def secondary_workloads(torch, A, dev):
             lib.moe_gg_w4a16_splitk(a.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), c.data_ptr(), M, N, K, 128, 0, 0, stream)
 
         ms = event_time_ms(torch, call, 120, 24)
+
+        def call_hot():  # always the same 29 MB of weights: they stay in the 256 MB last-level cache
+            lib.moe_gg_w4a16_splitk(a.data_ptr(), qws[0].data_ptr(), sc.data_ptr(), qz.data_ptr(), c.data_ptr(), M, N, K, 128, 0, 0, stream)
+
+        ms_hot = event_time_ms(torch, call_hot, 120, 24)
         byt = K * N // 2 + (K // 128) * N * 2 + (K // 128) * N // 2 + M * K * 2 + M * N * 2
         out.append({"workload": f"W4A16 split-K M={M} K=4096 N=14336 group 128",
-                    "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
+                    "us_per_launch": round(ms * 1e3, 2), "cache_hot_us_per_launch": round(ms_hot * 1e3, 2),
+                    "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
                     "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128", "achieved": round(byt / ms / 1e6, 1),
                                  "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
                                  "traffic": W4A16_TRAFFIC_BYTES.get(M)}})
