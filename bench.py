@@ -27,8 +27,9 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 PREFILL_TRAFFIC_BYTES = 2.18e9
 # The same for the other workloads (profiles/bench_all_kernels_traffic.md): fetched + written bytes per launch.
 DECODE_TRAFFIC_BYTES = {"up": 0.946e9 + 1.8e6, "down": 0.957e9 + 0.5e6}
-W4A16_TRAFFIC_BYTES = {1: 32.3e6 + 0.03e6, 16: 32.3e6 + 0.46e6, 64: 48.0e6 + 1.8e6}
+W4A16_TRAFFIC_BYTES = {1: 32.3e6 + 0.03e6, 16: 32.3e6 + 0.46e6, 64: 44.9e6 + 1.8e6}
 W4A16_GROUPED_TRAFFIC_BYTES = 254.2e6 + 1.8e6
+W4A16_GROUPED_FP8OUT_TRAFFIC_BYTES = 254.4e6 + 1.15e6
 FP8_BLOCK_TRAFFIC_BYTES = 9.04e9 + 0.27e9
 
 
@@ -208,7 +209,7 @@ def secondary_workloads(torch, A, dev):
                 "value": round(byt_q / ms_q / 1e6, 1), "unit": "GB/s",
                 "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128 (fp8 output)", "achieved": round(byt_q / ms_q / 1e6, 1),
                              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt_q / ms_q / 1e6 / PEAK_HBM_GBS, 4),
-                             "traffic": None}})
+                             "traffic": W4A16_GROUPED_FP8OUT_TRAFFIC_BYTES}})
     del qwe
 
     # ---- config 5: DeepSeek-V3-style fp8 block-scaled, 256 experts top-8, Zipf(1.1) routing ----
