@@ -29,22 +29,26 @@ namespace {
 template <int NF, int MF, int WAVES, int DEPTH, bool PAIR, bool TAIL = false, bool F16 = false>
 __global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
   __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MF][256];
-  __shared__ int s_row0, s_rows;
-  __shared__ int32_t tail_row_off[TAIL ? MOE_GG_MAX_GROUPS + 1 : 1];
+  __shared__ int s_g, s_row0, s_rows;
+  __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int g = blockIdx.y;
   const int K = p.K, N = p.N;
 
-  if (TAIL) {
-    // The ping-pong kernel's own tables and counts, so that both take the same decision.
-    build_row_offsets(p.m_sizes, p.G, p.M, tail_row_off);
-    if (wave == 0) {
+  // Grid row blockIdx.y takes the blockIdx.y-th expert that has rows to compute, not expert blockIdx.y: the
+  // workgroups without work are then the last ones of the launch. Scattered among the others they leave at once
+  // and the dispatcher fills their places unevenly: with every second expert empty the working workgroups ended
+  // up on part of the CUs only (123 us against 88 us for the same four experts next to each other).
+  build_row_offsets(p.m_sizes, p.G, p.M, row_off);
+  if (wave == 0) {
+    bool apart = false;
+    if (TAIL) {
+      // The ping-pong kernel's own tables and counts, so that both take the same decision.
       long long n_long = 0, n_low = 0, passes = 0;
       for (int i = lane; i < p.G; i += 64) {
-        const int r = tail_row_off[i + 1] - tail_row_off[i];
+        const int r = row_off[i + 1] - row_off[i];
         n_long += moe_gg_long_row_tiles(r, 256);
         n_low += moe_gg_low_row_tiles(r, 256);
         passes += moe_gg_low_passes(r, 256);
@@ -55,33 +59,23 @@ __global__ __launch_bounds__(64 * WAVES) void gg_bf16_decode(GgParams p) {
         n_low += __shfl_xor(n_low, d, 64);
         passes += __shfl_xor(passes, d, 64);
       }
-      if (lane == 0) {
-        const int ntn = moe_gg_cdiv(N, 256);
-        const int r = tail_row_off[g + 1] - tail_row_off[g];
-        const bool mine = moe_gg_low_row_tiles(r, 256) > 0 &&
-                          moe_gg_tails_apart((int)(n_long * ntn), (int)(n_low * ntn), passes * ntn, p.tails_apart);
-        s_row0 = tail_row_off[g] + r / 256 * 256;
-        s_rows = mine ? r % 256 : 0;
-      }
+      const int ntn = moe_gg_cdiv(N, 256);
+      apart = moe_gg_tails_apart((int)(n_long * ntn), (int)(n_low * ntn), passes * ntn, p.tails_apart);
     }
-  } else if (wave == 0) {
-    // Row range of expert g: prefix sum of m_sizes[0 .. g) (clamped like tile_sched.h does).
-    long long s = 0;
-    for (int i = lane; i < g; i += 64) {
-      int m = p.m_sizes[i];
-      s += m < 0 ? 0 : (m > p.M ? p.M : m);
-    }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
+    const int g = nth_group(p.G, blockIdx.y, [&](int i) {
+      const int r = row_off[i + 1] - row_off[i];
+      return TAIL ? apart && moe_gg_low_row_tiles(r, 256) > 0 : r > 0;
+    });
     if (lane == 0) {
-      const long long r0 = s > p.M ? p.M : s;
-      s_row0 = (int)r0;
-      s_rows = moe_gg_clamp_rows(p.m_sizes[g], r0, p.M);
+      const int r = g < 0 ? 0 : row_off[g + 1] - row_off[g];
+      s_g = g;
+      s_row0 = g < 0 ? 0 : row_off[g] + (TAIL ? r / 256 * 256 : 0);
+      s_rows = TAIL ? r % 256 : r;
     }
   }
   __syncthreads();
-  const int row0 = s_row0, rows = s_rows;
-  if (rows == 0) return;
+  const int g = s_g, row0 = s_row0, rows = s_rows;
+  if (g < 0 || rows == 0) return;
 
   const int n0 = blockIdx.x * (16 * NF);
   const int fr = lane & 15, fq = lane >> 4;

@@ -17,7 +17,7 @@
 // kernel, launched beside this one, skips exactly the experts handled here.
 #include "common.h"
 #include "kernels.h"
-#include "tile_sched.h"
+#include "gg_tables.h"
 
 namespace {
 
@@ -29,33 +29,34 @@ __global__ __launch_bounds__(256) void gg_fp8_stream(GgParams p, int max_rows) {
   constexpr int RP = MF >= 2 ? 2 : 1;          // the reduction runs in RP passes over MF / RP activation fragments,
   constexpr int MFP = MF / RP;                 // which keeps the LDS footprint at 32 KB and three workgroups per CU
   __shared__ __attribute__((aligned(16))) float red[WAVES][NF * MFP][256];
-  __shared__ int s_row0, s_rows;
+  __shared__ int s_g, s_row0, s_rows;
+  __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int g = blockIdx.y;
   const int K = p.K, N = p.N;
   const int KB = K / 128;
 
+  // Grid row blockIdx.y takes the blockIdx.y-th expert with 1 .. max_rows rows: the workgroups without work are
+  // then the last ones of the launch (scattered among the others they make the dispatcher fill the CUs unevenly).
+  build_row_offsets(p.m_sizes, p.G, p.M, row_off);
   if (wave == 0) {
-    long long s = 0;
-    for (int i = lane; i < g; i += 64) {
-      int m = p.m_sizes[i];
-      s += m < 0 ? 0 : (m > p.M ? p.M : m);
-    }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
+    const int gi = nth_group(p.G, blockIdx.y, [&](int i) {
+      const int r = row_off[i + 1] - row_off[i];
+      return r > 0 && r <= max_rows;
+    });
     if (lane == 0) {
-      const long long r0 = s > p.M ? p.M : s;
-      s_row0 = (int)r0;
-      s_rows = moe_gg_clamp_rows(p.m_sizes[g], r0, p.M);
+      s_g = gi;
+      s_row0 = gi < 0 ? 0 : row_off[gi];
+      s_rows = gi < 0 ? 0 : row_off[gi + 1] - row_off[gi];
     }
   }
   __syncthreads();
+  const int g = __builtin_amdgcn_readfirstlane(s_g);
   const int row0 = __builtin_amdgcn_readfirstlane(s_row0);
   const int rows = __builtin_amdgcn_readfirstlane(s_rows);
-  if (rows == 0 || rows > max_rows) return;
+  if (g < 0 || rows == 0) return;
   const int nmf = (rows + 15) >> 4;  // activation fragments in use (<= MF)
 
   const int n0 = blockIdx.x * (16 * NF);

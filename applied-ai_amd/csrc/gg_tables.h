@@ -15,6 +15,31 @@ DEVINL long long wave_incl_scan_i64(long long x) {
   return x;
 }
 
+// The n-th group (counted from 0) for which has_work(g) holds, or -1 if there are fewer. Called by all 64 lanes of
+// one wave; every lane gets the answer.
+template <class F>
+DEVINL int nth_group(int G, int n, F has_work) {
+  const int l = lane_id(), per = (G + 63) >> 6, g0 = l * per;
+  int c = 0;
+  for (int i = 0; i < per; ++i)
+    if (g0 + i < G && has_work(g0 + i)) ++c;
+  int incl = c;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int v = __shfl_up(incl, d, 64);
+    if (l >= d) incl += v;
+  }
+  int found = -1;
+  if (n >= incl - c && n < incl) {
+    int k = n - (incl - c);
+    for (int i = 0; i < per && found < 0; ++i)
+      if (g0 + i < G && has_work(g0 + i) && k-- == 0) found = g0 + i;
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) found = max(found, __shfl_xor(found, d, 64));
+  return found;
+}
+
 // Must be called by every thread of the workgroup (it ends with a barrier).
 // row_off: LDS array of G + 1 entries, G <= MOE_GG_MAX_GROUPS: row_off[g] = min(sum of the clamped sizes before g, M).
 DEVINL void build_row_offsets(const int32_t* __restrict__ m_sizes, int G, int M, int32_t* row_off) {

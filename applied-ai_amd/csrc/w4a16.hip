@@ -27,10 +27,10 @@
 // fp32 scale - float8_groupwise_quantize (kernels/triton/inference/fp8/float8_groupwise_quant.py:20-50) applied to
 // the 16-bit result, bit for bit, without the round trip of that result through memory.
 #include "common.h"
+#include "gg_tables.h"
 #include "kernels.h"
 
 namespace {
-
 
 template <bool FP16>
 struct Elem;
@@ -74,25 +74,54 @@ struct W4View {
 DEVINL W4View w4_view(const W4Params& p) {
   W4View v{(const uint16_t*)p.a, p.qweight, (const uint16_t*)p.scales, p.qzeros, (uint16_t*)p.c, p.M, (uint8_t*)p.cq, p.cscale};
   if (p.m_sizes == nullptr) return v;
-  __shared__ int s_row0, s_rows;
-  const int g = blockIdx.y;
+  // Grid row blockIdx.y takes the blockIdx.y-th expert that has rows (the workgroups without work are then the last
+  // ones of the launch; scattered among the others they make the dispatcher fill the CUs unevenly).
+  __shared__ int s_g, s_row0, s_rows;
   if (threadIdx.x < 64) {
-    long long s = 0;
-    for (int i = threadIdx.x; i < g; i += 64) {
+    const int l = threadIdx.x, per = (p.G + 63) >> 6, g0 = l * per, want = blockIdx.y;
+    auto rows_of = [&](int i) {
       const int m = p.m_sizes[i];
-      s += m < 0 ? 0 : (m > p.M ? p.M : m);
-    }
+      return m < 0 ? 0 : (m > p.M ? p.M : m);
+    };
+    long long s = 0;
+    int c = 0;
+    for (int i = 0; i < per; ++i)
+      if (g0 + i < p.G) {
+        const int m = rows_of(g0 + i);
+        s += m;
+        c += m > 0;
+      }
+    long long run = wave_incl_scan_i64(s) - s;
+    int incl = c;
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
-    if (threadIdx.x == 0) {
-      const long long r0 = s > p.M ? p.M : s;
-      int m = p.m_sizes[g];
-      m = m < 0 ? 0 : m;
-      s_row0 = (int)r0;
-      s_rows = (long long)m > p.M - r0 ? (int)(p.M - r0) : m;
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (l >= d) incl += up;
+    }
+    const bool here = want >= incl - c && want < incl;  // true in one lane at most
+    if (__ballot(here) == 0) {
+      if (l == 0) s_g = -1;
+    } else if (here) {
+      int k = want - (incl - c);
+      for (int i = 0; i < per; ++i) {
+        const int m = g0 + i < p.G ? rows_of(g0 + i) : 0;
+        if (m > 0 && k-- == 0) {
+          const long long r0 = run > p.M ? p.M : run;
+          s_g = g0 + i;
+          s_row0 = (int)r0;
+          s_rows = (long long)m > p.M - r0 ? (int)(p.M - r0) : m;
+          break;
+        }
+        run += m;
+      }
     }
   }
   __syncthreads();
+  const int g = s_g;
+  if (g < 0) {
+    v.M = 0;
+    return v;
+  }
   const int row0 = s_row0;
   const int ngroups = p.K / p.group_size;
   v.M = s_rows;
