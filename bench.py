@@ -263,6 +263,7 @@ def secondary_workloads(torch, A, dev):
     ms = event_time_ms(torch, lambda: A.fused_moe(h, w1, w2, tw, ids), 10, 3)
     flop = 2.0 * T * topk * (2 * n * K + K * n)
     out.append({"workload": "Mixtral 8x7B MoE layer (fused_moe: group, gather, w1 GEMM, SiLU-and-mul, w2 GEMM, top-2 combine), T=4096, bf16",
+                "m_sizes": torch.bincount(ids.flatten().long(), minlength=E).tolist(),
                 "ms_per_launch": round(ms, 3), "value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
                 "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong (two launches) + glue kernels", "achieved": round(flop / ms / 1e9, 1),
                              "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
