@@ -163,6 +163,32 @@ def test_every_kernel_variant_against_oracle(variant, mode):
     assert rel_fro(to_np(y), ref) <= TOL
 
 
+@pytest.mark.parametrize("variant", [-1, 1, 2])
+def test_many_experts_most_of_them_empty(variant):
+    """200 experts, most without rows, a few beyond the streaming kernel's 64 rows: its grid rows are taken by the
+    n-th expert within its row range, found by one wave over more experts than it has lanes."""
+    import applied_ai_amd as A
+
+    G, N, K = 200, 128, 256
+    rng = np.random.default_rng(200)
+    m_sizes = rng.integers(1, 9, size=G)
+    m_sizes[rng.permutation(G)[:140]] = 0
+    m_sizes[[0, 77, 199]] = [70, 130, 5]
+    m_sizes = [int(v) for v in m_sizes]
+    M = sum(m_sizes)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((G * N, K)) * 0.05).astype(np.float32)
+    xq, xs = O.fp8_groupwise_quant(x); wq, ws = O.fp8_block_quant_weight(w)
+    lib = A._lib.lib()
+    assert lib.moe_gg_set_variant(1, variant) == 0
+    try:
+        y = run(xq, wq, xs, ws, m_sizes, 1)
+    finally:
+        lib.moe_gg_set_variant(1, -1)
+    ref = O.grouped_gemm_fp8(xq, wq, xs, ws, m_sizes, 1)
+    assert rel_fro(to_np(y), ref) <= TOL
+
+
 def test_rowwise_block_layout_of_the_training_copy():
     """grouped_gemm_fp8_rowwise_forward writes [M, N*G]: expert g's rows in columns [g*N, (g+1)*N), the same values
     as the [M, N] entry point (kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:468-480)."""

@@ -117,6 +117,33 @@ def test_grouped_fp8_output_feeds_the_fp8_grouped_gemm():
     assert rel_fro(to_np(y), ref) <= TOL
 
 
+@pytest.mark.parametrize("quantize_output", [False, True])
+def test_grouped_many_experts_most_of_them_empty(quantize_output):
+    """130 experts, two thirds without rows: a grid row is taken by the n-th expert that has rows, found by one wave
+    over more experts than it has lanes."""
+    import applied_ai_amd as A
+
+    rng = np.random.default_rng(130)
+    E, K, N, gs = 130, 256, 128, 128
+    m_sizes = rng.integers(1, 6, size=E)
+    m_sizes[rng.permutation(E)[:87]] = 0
+    m_sizes[[0, 64, 129]] = [3, 0, 18]
+    m_sizes = [int(v) for v in m_sizes]
+    R = sum(m_sizes)
+    qw, qz, sc = make_experts(rng, E, K, N, gs)
+    scales = torch.from_numpy(sc).to(torch.bfloat16)
+    a = torch.from_numpy(rng.standard_normal((R, K)).astype(np.float32)).to(torch.bfloat16)
+    args = (a.cuda(), torch.from_numpy(qw).cuda(), scales.cuda(), torch.from_numpy(qz).cuda(),
+            torch.tensor(m_sizes, dtype=torch.int32).cuda())
+    c = A.matmul_split_k_grouped(*args, zero_offset=1)
+    ref = O.w4a16_grouped(to_np(a), qw, to_np(scales), qz, m_sizes, gs, 1)
+    assert rel_fro(to_np(c), ref) <= TOL
+    if quantize_output:
+        q, s = A.matmul_split_k_grouped(*args, zero_offset=1, quantize_output=True)
+        q2, s2 = A.float8_groupwise_quantize(c)
+        assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
+
+
 def test_grouped_equals_dense_call_per_expert_bitwise():
     """One expert of a grouped call must give exactly what the dense entry point gives for the same rows."""
     import applied_ai_amd as A
