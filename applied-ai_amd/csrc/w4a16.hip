@@ -84,10 +84,11 @@ DEVINL W4View w4_view(const W4Params& p) {
       return m < 0 ? 0 : (m > p.M ? p.M : m);
     };
     long long s = 0;
-    int c = 0;
+    int c = 0, m_first = 0;  // m_first: rows of the lane's first expert (its only one when G <= 64)
     for (int i = 0; i < per; ++i)
       if (g0 + i < p.G) {
         const int m = rows_of(g0 + i);
+        if (i == 0) m_first = m;
         s += m;
         c += m > 0;
       }
@@ -104,7 +105,7 @@ DEVINL W4View w4_view(const W4Params& p) {
     } else if (here) {
       int k = want - (incl - c);
       for (int i = 0; i < per; ++i) {
-        const int m = g0 + i < p.G ? rows_of(g0 + i) : 0;
+        const int m = i == 0 ? m_first : (g0 + i < p.G ? rows_of(g0 + i) : 0);
         if (m > 0 && k-- == 0) {
           const long long r0 = run > p.M ? p.M : run;
           s_g = g0 + i;
