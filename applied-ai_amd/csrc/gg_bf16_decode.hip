@@ -15,8 +15,9 @@
 // 32 KB vector L1 (the waves of a CU keep far more lines in flight than that) and fetches it again, which
 // costs 15-20 % of the streaming rate. The fragments are multiplied with the activation fragments
 // ("B" operand, L2-resident) by v_mfma_f32_16x16x32_bf16, and the four partial accumulators are
-// summed through LDS (fixed order: deterministic) before the bf16 store. Experts with m_g = 0 exit
-// at once, so their weights are never touched.
+// summed through LDS (fixed order: deterministic) before the bf16 store. Grid row y works on the y-th
+// expert with m_g > 0; the rows of the grid beyond the number of such experts exit at once, so the
+// weights of an expert without rows are never touched.
 #include "common.h"
 #include "kernels.h"
 #include "tile_sched.h"

@@ -57,7 +57,7 @@ struct Elem<true> {  // fp16
   static DEVINL uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
 };
 
-// What one workgroup works on: the whole problem (dense call), or expert blockIdx.y of a grouped call
+// What one workgroup works on: the whole problem (dense call), or one expert of a grouped call
 // (rows row0 .. row0 + M - 1 of a and c, and that expert's slice of the stacked weights).
 struct W4View {
   const uint16_t* a;
