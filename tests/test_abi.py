@@ -286,3 +286,15 @@ def test_there_is_no_cpu_path():
             A._lib.lib()
     finally:
         A._lib.LIB_PATH, A._lib._lib = saved
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it exits with a message that says so, before touching any device."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
