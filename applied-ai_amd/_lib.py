@@ -53,7 +53,7 @@ SIGNATURES = {
     ),
     "moe_gg_route_topk": (_c_int, [_c_void_p, _c_i64, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "moe_gg_route_group": (_c_int, [_c_void_p, _c_i64, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
-    "moe_gg_gather_rows": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_i64, _c_i64, _c_void_p]),
+    "moe_gg_gather_rows": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_i64, _c_i64, _c_i64, _c_void_p, _c_void_p]),
     "moe_gg_grouped_gemm_backward_workspace": (ctypes.c_size_t, [_c_int, _c_i64, _c_int, _c_int, _c_int]),
     "moe_gg_grouped_gemm_backward_bf16": (
         _c_int,
@@ -70,6 +70,7 @@ SIGNATURES = {
     "moe_gg_combine_topk": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_i64, _c_int, _c_int, _c_i64, _c_void_p]),
     "moe_gg_combine_topk_f16": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_i64, _c_int, _c_int, _c_i64, _c_void_p]),
     "moe_gg_fp8_groupwise_quant": (_c_int, [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_i64, _c_void_p]),
+    "moe_gg_fp8_block128_quant": (_c_int, [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "moe_gg_align_block_size": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p]),
     "moe_gg_host_enumerate_tiles": (
         _c_int,

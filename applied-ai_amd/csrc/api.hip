@@ -326,13 +326,14 @@ int moe_gg_align_block_size(const int32_t* perm, const int32_t* m_sizes, int E, 
 }
 
 int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int64_t n, int64_t row_bytes,
-                       void* stream) {
-  if (n < 0 || k <= 0 || row_bytes < 0) return MOE_GG_EINVAL;
+                       int64_t src_rows, const int32_t* n_valid, void* stream) {
+  if (n < 0 || k <= 0 || row_bytes < 0 || src_rows < 0) return MOE_GG_EINVAL;
   if (n == 0 || row_bytes == 0) return MOE_GG_OK;
-  if (!x || !perm || !out) return MOE_GG_EINVAL;
+  if (!perm || !out || (src_rows > 0 && !x)) return MOE_GG_EINVAL;
   if (n > INT32_MAX) return MOE_GG_EUNSUPPORTED;
   if (row_bytes % 16 != 0 || !aligned(x, 16) || !aligned(out, 16)) return MOE_GG_EALIGN;
-  return (int)gather_rows_launch(x, perm, k, out, (int)n, row_bytes, (hipStream_t)stream);
+  if (n_valid && !aligned(n_valid, 4)) return MOE_GG_EALIGN;
+  return (int)gather_rows_launch(x, perm, k, out, (int)n, row_bytes, src_rows, n_valid, (hipStream_t)stream);
 }
 
 static int grouped_gemm_swiglu_16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M, int n,
@@ -475,13 +476,12 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
     q.xcds = xcds;
     return (int)gg_bf16_pingpong_wgrad_direct_launch(q, num_wg, s);
   }
-  if (M > 0) {
-    // dY^T and x^T with every expert padded to whole 64-row blocks.
-    e = transpose_padded_launch(grad_out, dyt, m_sizes, G, (int)M, N, ld_go, x_col_block, ldm, s);
-    if (e != hipSuccess) return (int)e;
-    e = transpose_padded_launch(x, xt, m_sizes, G, (int)M, K, K, 0, ldm, s);
-    if (e != hipSuccess) return (int)e;
-  }
+  // dY^T and x^T with every expert padded to whole 64-row blocks. Also without any row (M = 0): nothing is read
+  // then and every expert gets its one block of zeros, which makes grad_w all zeros below.
+  e = transpose_padded_launch(grad_out, dyt, m_sizes, G, (int)M, N, ld_go, x_col_block, ldm, s);
+  if (e != hipSuccess) return (int)e;
+  e = transpose_padded_launch(x, xt, m_sizes, G, (int)M, K, K, 0, ldm, s);
+  if (e != hipSuccess) return (int)e;
   GgParams p{};
   p.x = dyt; p.w = xt; p.y = grad_w; p.m_sizes = m_sizes;
   p.G = G; p.M = (int)ldm; p.N = N; p.K = K;
@@ -556,6 +556,17 @@ int moe_gg_fp8_groupwise_quant(const void* in, int dtype, void* out, float* scal
   if (!in || !out || !scales) return MOE_GG_EINVAL;
   if (!aligned(in, 8) || !aligned(out, 2) || !aligned(scales, 4)) return MOE_GG_EALIGN;
   return (int)fp8_groupwise_quant_launch(in, dtype == MOE_GG_DTYPE_BF16, out, scales, numel / 128, (hipStream_t)stream);
+}
+
+int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scales, int64_t rows, int K, void* stream) {
+  if (rows < 0 || K < 0) return MOE_GG_EINVAL;
+  if (dtype != MOE_GG_DTYPE_BF16 && dtype != MOE_GG_DTYPE_FP32) return MOE_GG_EINVAL;
+  if (rows % 128 != 0 || K % 128 != 0) return MOE_GG_ESHAPE;
+  if (rows == 0 || K == 0) return MOE_GG_OK;
+  if (!in || !out || !scales) return MOE_GG_EINVAL;
+  if (rows / 128 > 65535) return MOE_GG_EUNSUPPORTED;
+  if (!aligned(in, 16) || !aligned(out, 16) || !aligned(scales, 4)) return MOE_GG_EALIGN;
+  return (int)fp8_block128_quant_launch(in, dtype == MOE_GG_DTYPE_BF16, out, scales, rows, K, (hipStream_t)stream);
 }
 
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,

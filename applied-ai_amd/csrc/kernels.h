@@ -81,10 +81,14 @@ hipError_t align_block_size_launch(const int32_t* perm, const int32_t* m_sizes, 
                                    int32_t* sorted_ids, int32_t* expert_ids, int32_t* num_post_pad,
                                    hipStream_t stream);
 hipError_t gather_rows_launch(const void* x, const int32_t* perm, int k, void* out, int n, int64_t row_bytes,
-                              hipStream_t stream);
+                              int64_t src_rows, const int32_t* n_valid, hipStream_t stream);
 // 1 x 128 fp8 quantiser (quant.hip); `groups` groups of 128 consecutive elements.
 hipError_t fp8_groupwise_quant_launch(const void* in, bool bf16_in, void* out, float* scales, int64_t groups,
                                       hipStream_t stream);
+
+// 128 x 128 block quantiser of a [rows, K] matrix (quant.hip); rows % 128 == 0, K % 128 == 0; scales [rows/128, K/128].
+hipError_t fp8_block128_quant_launch(const void* in, bool bf16_in, void* out, float* scales, int64_t rows, int K,
+                                     hipStream_t stream);
 
 // MoE layer glue (moe_layer.hip). bf16 data; n and d multiples of 8; 16-byte aligned pointers.
 hipError_t silu_and_mul_launch(const void* in, void* out, int64_t rows, int n, bool fp16, hipStream_t stream);

@@ -130,16 +130,28 @@ __global__ __launch_bounds__(64 * GROUP_WAVES) void route_group_kernel(const int
       perm[off[e] + start + rank] = p;
     }
   }
+  // Dropped ids leave sum(m_sizes) < n: the unused tail of perm is -1, never stale memory.
+  for (int i = off[E] + tid; i < n; i += blockDim.x) perm[i] = -1;
 }
 
 // ---- gather: out[i] = x[perm[i] / k], rows of row_bytes (multiple of 16) ----------------------------
+// Positions at or beyond *n_valid (when given) and entries of perm that name no row of x (negative, or
+// perm[i] / k >= src_rows) read nothing: their output row is zeros.
 __global__ __launch_bounds__(256) void gather_rows_kernel(const char* __restrict__ x, const int32_t* __restrict__ perm,
-                                                          int k, char* __restrict__ out, int n, int64_t row_bytes) {
+                                                          int k, char* __restrict__ out, int n, int64_t row_bytes,
+                                                          int64_t src_rows, const int32_t* __restrict__ n_valid) {
   const int i = blockIdx.x;
   if (i >= n) return;
-  const int64_t src = perm[i] / k;
-  const u32x4_t* s = (const u32x4_t*)(x + src * row_bytes);
+  const int32_t pi = perm[i];
+  const int64_t src = pi / k;
+  const bool ok = pi >= 0 && src < src_rows && (!n_valid || i < *n_valid);
   u32x4_t* d = (u32x4_t*)(out + (int64_t)i * row_bytes);
+  if (!ok) {
+    const u32x4_t z = {0u, 0u, 0u, 0u};
+    for (int64_t c = threadIdx.x; c < row_bytes / 16; c += blockDim.x) d[c] = z;
+    return;
+  }
+  const u32x4_t* s = (const u32x4_t*)(x + src * row_bytes);
   for (int64_t c = threadIdx.x; c < row_bytes / 16; c += blockDim.x) d[c] = s[c];
 }
 
@@ -189,9 +201,10 @@ hipError_t route_group_launch(const int32_t* flat, int n, int E, int32_t* perm, 
 }
 
 hipError_t gather_rows_launch(const void* x, const int32_t* perm, int k, void* out, int n, int64_t row_bytes,
-                              hipStream_t stream) {
+                              int64_t src_rows, const int32_t* n_valid, hipStream_t stream) {
   if (n == 0) return hipSuccess;
-  hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, stream, (const char*)x, perm, k, (char*)out, n, row_bytes);
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, stream, (const char*)x, perm, k, (char*)out, n, row_bytes,
+                     src_rows, n_valid);
   return hipGetLastError();
 }
 

@@ -96,7 +96,7 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, t
     _require_cuda(A, B, C, topk_ids)
     ids = topk_ids if topk_ids.dtype == torch.int32 else topk_ids.to(torch.int32)
     perm, m_sizes, offsets = route_group(ids, E)
-    xs = gather_sorted(A, perm, top_k)
+    xs = gather_sorted(A, perm, top_k, offsets)
     y = grouped_gemm(xs, B.view(E * N, K), m_sizes)
     if mul_routed_weight:
         w = topk_weights if topk_weights.dtype in (torch.float32, A.dtype) else topk_weights.float()
@@ -126,7 +126,7 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, t
     tw = topk_weights if topk_weights.dtype in (torch.float32, hidden_states.dtype) else topk_weights.float()
 
     perm, m_sizes, offsets = route_group(ids, E)
-    xs = gather_sorted(hidden_states, perm, k)
+    xs = gather_sorted(hidden_states, perm, k, offsets)
     swiglu_tiles = (xs.shape[0] // 256 + E) * ((two_n // 2 + 127) // 128)   # bound of the fused kernel's tile table
     if (xs.shape[0] >= FUSED_SWIGLU_MIN_ROWS and K % 64 == 0 and two_n % 8 == 0 and two_n * K < 2 ** 31
             and swiglu_tiles <= 1023 * 256):
@@ -162,7 +162,7 @@ def dequant_gemm_moe(hidden_states: torch.Tensor, qw1: torch.Tensor, qw2: torch.
         tw = topk_weights if topk_weights.dtype in (torch.float32, hidden_states.dtype) else topk_weights.float()
 
     perm, m_sizes, offsets = route_group(ids, E)
-    xs = gather_sorted(hidden_states, perm, k)
+    xs = gather_sorted(hidden_states, perm, k, offsets)
     h1 = matmul_split_k_grouped(xs, qw1, scales_qw1, zeros_qw1, m_sizes, zero_offset=zero_offset)
     h2 = silu_and_mul(h1)
     y2 = matmul_split_k_grouped(h2, qw2, scales_qw2, zeros_qw2, m_sizes, zero_offset=zero_offset)

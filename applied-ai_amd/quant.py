@@ -28,12 +28,24 @@ def float8_groupwise_quantize(x: torch.Tensor, block_size: int = 128) -> Tuple[t
 
 
 def float8_blockwise_quantize_weight(w: torch.Tensor, block: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
-    """128 x 128 block quantisation of a [rows, K] weight matrix with the same scale and clamp rule as the
-    1 x 128 quantiser (one scale per block). Weight preparation, off the hot path: plain torch ops on whatever
-    device w lives on. The reference has no in-tree definition of this quantiser (it calls an un-vendored
-    FBGEMM routine, kernels/needs_perf_help/fp8_gemm_bench.py:16-21)."""
-    rows, K = w.shape
-    t = w.float().reshape(rows // block, block, K // block, block)
-    s = t.abs().amax(dim=(1, 3)).clamp_min(1e-12) / 448.0
-    q = (t / s[:, None, :, None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).reshape(rows, K)
-    return q, s.contiguous()
+    """128 x 128 block quantisation of a [rows, K] weight matrix (or a stack [G, N, K], taken as [G*N, K]) with the
+    scale and clamp rule of the 1 x 128 quantiser, one scale per block: returns (q like w as float8_e4m3fn, scales
+    [rows/128, K/128] fp32), the w / w_scale of grouped_gemm_fp8_blockwise. The reference takes this step from an
+    un-vendored package (quantize_fp8_block, kernels/needs_perf_help/fp8_gemm_bench.py:16-21)."""
+    if block != 128:
+        raise ValueError("only block = 128 is implemented")
+    if w.dim() not in (2, 3) or w.size(-1) % block != 0 or w.size(-2) % block != 0:
+        raise ValueError(f"w must be [rows, K] or [G, N, K] with N (rows) and K multiples of {block}")
+    if w.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("w must be fp32 or bf16")
+    dev = _require_cuda(w)
+    w = w.contiguous()
+    K = w.size(-1)
+    rows = w.numel() // K
+    out = torch.empty_like(w, dtype=torch.float8_e4m3fn)
+    scales = torch.empty(rows // block, K // block, dtype=torch.float32, device=w.device)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_fp8_block128_quant(w.data_ptr(), 0 if w.dtype == torch.bfloat16 else 2, out.data_ptr(),
+                                                  scales.data_ptr(), rows, K, _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_fp8_block128_quant")
+    return out, scales

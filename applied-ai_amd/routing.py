@@ -74,16 +74,21 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int,
     return sorted_ids, expert_ids, num_post_pad
 
 
-def gather_sorted(x: torch.Tensor, perm: torch.Tensor, k: int) -> torch.Tensor:
-    """x_sorted[i] = x[perm[i] // k]: the token rows in expert-sorted order."""
+def gather_sorted(x: torch.Tensor, perm: torch.Tensor, k: int, offsets: torch.Tensor = None) -> torch.Tensor:
+    """x_sorted[i] = x[perm[i] // k]: the token rows in expert-sorted order. With offsets (the [E + 1] table of
+    route_group / route_topk) only its last entry's worth of perm is in use (ids outside [0, E) were dropped); the
+    rows behind it, and rows whose perm entry names no row of x, come back as zeros."""
     if x.dim() != 2 or perm.dtype != torch.int32:
         raise ValueError("x must be 2-D and perm int32")
     dev = _require_cuda(x, perm)
+    if offsets is not None and (offsets.dtype != torch.int32 or offsets.device != dev or not offsets.is_contiguous()):
+        raise ValueError("offsets must be a contiguous int32 tensor on x's device")
     x = x.contiguous()
     n = perm.shape[0]
     out = torch.empty((n, x.shape[1]), dtype=x.dtype, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().moe_gg_gather_rows(x.data_ptr(), perm.data_ptr(), k, out.data_ptr(), n,
-                                           x.shape[1] * x.element_size(), _stream_ptr(dev))
+                                           x.shape[1] * x.element_size(), x.shape[0],
+                                           offsets[-1:].data_ptr() if offsets is not None else None, _stream_ptr(dev))
     _lib.check(rc, "moe_gg_gather_rows")
     return out

@@ -166,9 +166,14 @@ int moe_gg_route_group(const int32_t* flat_ids, int64_t n, int E, int32_t* perm,
  *   num_post_pad device out, int32 [1]: the padded total */
 int moe_gg_align_block_size(const int32_t* perm, const int32_t* m_sizes, int E, int64_t n, int block_size,
                             int32_t* sorted_ids, int32_t* expert_ids, int32_t* num_post_pad, void* stream);
-/* out[i, :] = x[perm[i] / k, :] for i < n; rows of row_bytes bytes (multiple of 16), x and out 16-byte aligned. */
+/* out[i, :] = x[perm[i] / k, :] for i < n; rows of row_bytes bytes (multiple of 16), x and out 16-byte aligned;
+ * x has src_rows rows. n_valid (device, int32 [1], may be null) is the number of leading entries of perm that are in
+ * use, e.g. offsets + E of moe_gg_route_group when ids were dropped. An output row whose position is at or beyond
+ * *n_valid, or whose perm entry names no row of x (negative, or perm[i] / k >= src_rows), is written as zeros and
+ * nothing is read for it. (The x[sorted_token_ids // top_k] gather of the reference's kernel,
+ * kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:63-69, with its token_mask.) */
 int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int64_t n, int64_t row_bytes,
-                       void* stream);
+                       int64_t src_rows, const int32_t* n_valid, void* stream);
 
 /*
  * Backward pass of the bf16 grouped GEMM. Replaces grouped_gemm_backward
@@ -240,6 +245,17 @@ int moe_gg_combine_topk_f16(const void* y, const int32_t* inv, const void* weigh
  *   scales device out, fp32 [numel / 128].
  */
 int moe_gg_fp8_groupwise_quant(const void* in, int dtype, void* out, float* scales, int64_t numel, void* stream);
+
+/*
+ * 128 x 128 block fp8 e4m3fn quantiser for weight matrices: the weight side of the block-scaled grouped GEMM
+ * (w / w_scale of moe_gg_grouped_gemm_fp8 with MOE_GG_SCALE_BLOCK128). Stands where the reference calls
+ * quantize_fp8_block of the FBGEMM package (kernels/needs_perf_help/fp8_gemm_bench.py:16-21, not vendored);
+ * the rule is the one of the in-tree 1 x 128 quantiser (float8_groupwise_quant.py:36-50) applied to a whole block:
+ * s = max(amax|block|, 1e-12) / 448, q = clamp(w / s, -448, 448) -> e4m3fn (RNE).
+ *   in  device [rows, K] row-major, bf16 or fp32 (dtype), rows % 128 == 0, K % 128 == 0, 16-byte aligned;
+ *   out device [rows, K] bytes, 16-byte aligned;  scales device out, fp32 [rows / 128, K / 128].
+ */
+int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scales, int64_t rows, int K, void* stream);
 
 /*
  * Test / tuning hooks (no counterpart in the reference).

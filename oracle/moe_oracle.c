@@ -12,10 +12,14 @@
  * Parity status:
  *   orc_offsets, orc_grouped_gemm, orc_route, orc_moe_align_block_size, orc_topk,
  *   orc_w4_dequant, orc_e4m3_*, orc_fp8_groupwise_quant, orc_grouped_gemm_fp8 (rowwise),
- *   orc_silu_and_mul, orc_fused_moe, orc_grouped_gemm_backward: pinned.
- *   orc_fp8_block_quant_weight (128x128 weight quantiser): PARITY UNPINNED - the reference calls an
- *   un-vendored FBGEMM routine for it (kernels/needs_perf_help/fp8_gemm_bench.py:16-21); this file
- *   defines it by analogy with the 1x128 quantiser and only its GEMM consumer is checked.
+ *   orc_silu_and_mul, orc_fused_moe, orc_grouped_gemm_backward, orc_fp8_block_quant_weight: pinned.
+ *   For orc_fp8_block_quant_weight (128x128 weight quantiser) the reference calls quantize_fp8_block of
+ *   the FBGEMM package, which is not vendored and pinned to no version
+ *   (kernels/needs_perf_help/fp8_gemm_bench.py:16-21); its published rule is per-block
+ *   max(amax, 1e-12) against the e4m3 maximum 448 with a clamp to +-448, the rule of the in-tree
+ *   1x128 quantiser, which this file applies to a whole block (scale stored as amax/448, codes from
+ *   w / scale). Pinned by constructed blocks, index order, numpy/torch routines and agreement with
+ *   the 1x128 quantiser where both must coincide.
  */
 #include <math.h>
 #include <stdint.h>
@@ -132,18 +136,25 @@ void orc_topk(const float* logits, int64_t T, int E, int k, int32_t* ids) {
  * loop (test_moe_gemm.py:24-29) and of moe_align_block_size
  * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:141-166).
  * Outputs: perm[n] (flat indices in sorted order; the source token is perm[i] / k), m_sizes[E].
+ * An id outside [0, E) (a masked slot, e.g. -1) belongs to no expert: it is counted nowhere, its
+ * position appears nowhere in perm, and the sum(m_sizes) .. n-1 tail of perm is -1 (the reference's
+ * kernel masks such slots out through token_mask, v0_moe_fused.py:63-66).
  * Pinned by: the docstring known answer of v0_moe_fused.py:157-165 (through
- * orc_moe_align_block_size below), numpy stable argsort and bincount. */
+ * orc_moe_align_block_size below), numpy stable argsort and bincount (over the valid positions
+ * when ids are masked). */
 void orc_route(const int32_t* flat_ids, int64_t n, int E, int32_t* perm, int32_t* m_sizes) {
   int64_t* cursor = (int64_t*)calloc((size_t)E + 1, sizeof(int64_t));
   memset(m_sizes, 0, sizeof(int32_t) * (size_t)E);
-  for (int64_t i = 0; i < n; ++i) m_sizes[flat_ids[i]]++;
+  for (int64_t i = 0; i < n; ++i)
+    if (flat_ids[i] >= 0 && flat_ids[i] < E) m_sizes[flat_ids[i]]++;
   int64_t run = 0;
   for (int e = 0; e < E; ++e) {
     cursor[e] = run;
     run += m_sizes[e];
   }
-  for (int64_t i = 0; i < n; ++i) perm[cursor[flat_ids[i]]++] = (int32_t)i;
+  for (int64_t i = 0; i < n; ++i)
+    if (flat_ids[i] >= 0 && flat_ids[i] < E) perm[cursor[flat_ids[i]]++] = (int32_t)i;
+  for (int64_t i = run; i < n; ++i) perm[i] = -1;
   free(cursor);
 }
 
@@ -269,7 +280,11 @@ void orc_fp8_groupwise_quant(const float* x, int64_t numel, int block, uint8_t* 
 }
 
 /* 128 x 128 block quantiser for a [rows, K] weight matrix: one scale per (rows/128, K/128) block,
- * same scale and clamp rule as above. PARITY UNPINNED (defined here, see file header). */
+ * same scale and clamp rule as above (see the file header for its source).
+ * Pinned by: a spike per block on a 2 x 3 grid of blocks (scale = |spike|/448 at [row block, K block],
+ * code 0x7E / 0xFE at the spike, all-zero block -> 1e-12/448 and zero codes), numpy
+ * reshape(rb,128,kb,128).max for the scales with torch's e4m3 cast for the codes, equality with
+ * orc_fp8_groupwise_quant when every row of a block holds the block's amax, power-of-two equivariance. */
 void orc_fp8_block_quant_weight(const float* w, int64_t rows, int K, int block, uint8_t* q, float* scales) {
   int64_t rb = rows / block;
   int kb = K / block;

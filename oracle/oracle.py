@@ -160,7 +160,7 @@ def fp8_groupwise_quant(x, block=128):
 
 
 def fp8_block_quant_weight(w, block=128):
-    """128x128 block quantiser for [rows, K] weights (defined by this oracle; parity unpinned)."""
+    """128x128 block quantiser for [rows, K] weights (rule of float8_groupwise_quant.py:36-50 per block)."""
     w = _f32(w)
     rows, K = w.shape
     q = np.empty(w.shape, dtype=np.uint8)

@@ -78,7 +78,7 @@ def test_argument_errors_of_the_other_entry_points(lib):
     assert lib.moe_gg_route_topk(None, 4, 8, 9, None, None, None, None, None) == -1         # k > E
     assert lib.moe_gg_route_topk(None, 4, 1000, 2, None, None, None, None, None) == -4      # E too large
     assert lib.moe_gg_route_group(None, 4, 0, None, None, None, None) == -1
-    assert lib.moe_gg_gather_rows(None, None, 0, None, 4, 16, None) == -1                    # k <= 0
+    assert lib.moe_gg_gather_rows(None, None, 0, None, 4, 16, 4, None, None) == -1                    # k <= 0
     assert lib.moe_gg_align_block_size(None, None, 8, 4, 0, None, None, None, None) == -1    # block_size <= 0
     assert lib.moe_gg_align_block_size(None, None, 1000, 4, 16, None, None, None, None) == -4  # E too large
     assert lib.moe_gg_align_block_size(None, None, 8, 4, 16, None, None, None, None) == -1   # null pointers

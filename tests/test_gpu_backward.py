@@ -38,6 +38,31 @@ def run_case(sizes, M, N, K, seed, block_layout=True, scale=1.0):
     return to_np(gx), to_np(gw)
 
 
+def test_empty_batch_gives_zero_weight_gradient():
+    """M = 0 (no row at all): grad_x is empty and grad_w is written as zeros, never left as it was."""
+    import applied_ai_amd as A
+
+    G, N, K = 3, 128, 192
+    w = bf(torch.randn(G * N, K))
+    for cols in (N * G, N):
+        gx, gw = A.grouped_gemm_backward(torch.empty(0, cols, dtype=torch.bfloat16, device="cuda"),
+                                         torch.empty(0, K, dtype=torch.bfloat16, device="cuda"), w.cuda(),
+                                         torch.zeros(G, dtype=torch.int32, device="cuda"))
+        assert gx.shape == (0, K) and gw.shape == (G * N, K)
+        assert not gw.any()
+    # straight through the C ABI, with grad_w and the workspace full of NaN beforehand
+    lib = A._lib.lib()
+    gw = torch.full((G * N, K), float("nan"), dtype=torch.bfloat16, device="cuda")
+    nbytes = lib.moe_gg_grouped_gemm_backward_workspace(G, 1, N, K, 0)
+    ws = torch.full((nbytes // 2,), float("nan"), dtype=torch.bfloat16, device="cuda")
+    m = torch.zeros(G, dtype=torch.int32, device="cuda")
+    rc = lib.moe_gg_grouped_gemm_backward_bf16(None, N, 0, None, w.cuda().data_ptr(), m.data_ptr(), G, 0, N, K, None,
+                                               gw.data_ptr(), ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert not gw.isnan().any() and not gw.any()
+
+
 def test_fast_verification_case():
     # G = 20, M = 1024, N = 512, K = 256, randn data (fast_verification.py:31-40)
     run_case(even_split(1024, 20), 1024, 512, 256, seed=1)

@@ -99,6 +99,100 @@ def test_quantiser_bit_exact(dtype):
         A.float8_groupwise_quantize(torch.zeros(4, 100, device="cuda"))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_quantiser_bit_exact(dtype):
+    """float8_blockwise_quantize_weight (128 x 128 blocks) against the oracle: codes and scales bit for bit, on a
+    3 x 5 grid of blocks with an all-zero block, a dominant outlier and a block of tiny values; also a [G, N, K]
+    stack, which is quantised as [G*N, K]."""
+    import applied_ai_amd as A
+
+    gen = torch.Generator().manual_seed(44)
+    w = (torch.randn(384, 640, generator=gen) * 0.02).to(dtype)
+    w[128:256, 256:384] = 0          # all-zero block: scale 1e-12 / 448, codes 0
+    w[300, 17] = 50.0                # outlier dominates block (2, 0)
+    w[0:128, 512:640] *= 1e-6        # tiny block
+    q, s = A.float8_blockwise_quantize_weight(w.cuda())
+    torch.cuda.synchronize()
+    oq, os_ = O.fp8_block_quant_weight(w.float().numpy())
+    assert q.dtype == F8 and q.shape == w.shape and s.shape == (3, 5) and s.dtype == torch.float32
+    assert np.array_equal(q.view(torch.uint8).cpu().numpy(), oq)
+    assert np.array_equal(s.cpu().numpy(), os_)
+    q3, s3 = A.float8_blockwise_quantize_weight(w.reshape(3, 128, 640).cuda())
+    assert q3.shape == (3, 128, 640) and torch.equal(q3.view(torch.uint8).reshape(384, 640), q.view(torch.uint8))
+    assert torch.equal(s3, s)
+    with pytest.raises(ValueError):
+        A.float8_blockwise_quantize_weight(torch.zeros(100, 128, device="cuda"))
+
+
+def test_config5_full_size():
+    """BASELINE config 5 as one launch: 256 experts, T = 4096 tokens top-8 -> 32768 rows with Zipf(1.1) routing,
+    x ~ N(0,1) [32768, 7168] through the 1 x 128 quantiser, fused gate+up weights ~ N(0, 0.02) [256, 4096, 7168]
+    through the 128 x 128 block quantiser (drawn and quantised expert by expert to bound memory), bf16 out.
+    Checked against the dequantise-then-matmul oracle (the recipe of dev/triton_groupGEMM/testing/
+    base_testing.py:83-90 with block scales) on rows of the largest expert, a mid-sized one, eight experts with at
+    most 16 rows, expert 0 and the last expert, at the first, a middle and the last 128 columns; plus bitwise
+    determinism, and rows at or beyond sum(m_sizes) staying untouched."""
+    import applied_ai_amd as A
+    from applied_ai_amd import configs
+
+    _, _, _, m_all = configs.cfg5_routing()
+    m_np = m_all.numpy()
+    G, N, K = 256, 4096, 7168
+    R = int(m_np.sum())
+    assert R == 32768 and len(m_np) == G
+    PAD = 64                                        # rows beyond sum(m_sizes): must stay as they were
+    M = R + PAD
+    gen = torch.Generator(device="cuda").manual_seed(1005)
+    x = torch.randn(M, K, generator=gen, device="cuda")
+    xq, xs = A.float8_groupwise_quantize(x)
+    del x
+    wq = torch.empty(G * N, K, dtype=F8, device="cuda")
+    ws = torch.empty(G * N // 128, K // 128, dtype=torch.float32, device="cuda")
+    for g in range(G):
+        wg = torch.randn(N, K, generator=gen, device="cuda") * 0.02
+        q, s = A.float8_blockwise_quantize_weight(wg)
+        wq[g * N:(g + 1) * N] = q
+        ws[g * N // 128:(g + 1) * N // 128] = s
+    m_dev = m_all.to(torch.int32).cuda()
+    SENT = 12345.0
+    lib = A._lib.lib()
+
+    def launch():
+        y = torch.full((M, N), SENT, dtype=torch.bfloat16, device="cuda")
+        rc = lib.moe_gg_grouped_gemm_fp8(xq.data_ptr(), wq.data_ptr(), y.data_ptr(), xs.data_ptr(), ws.data_ptr(), 1,
+                                         m_dev.data_ptr(), G, M, N, K, N, 0, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        return y
+
+    print(f"cfg5 full size: G={G} rows={R} (+{PAD} pad) N={N} K={K} max m={m_np.max()} empty={(m_np == 0).sum()}", flush=True)
+    y = launch()
+    y2 = launch()
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+    assert bool((y[R:] == SENT).all())
+    assert not bool((y[:R] == SENT).all(dim=1).any())   # every routed row was written
+
+    order = np.argsort(-m_np, kind="stable")
+    small = [int(g) for g in np.nonzero((m_np > 0) & (m_np <= 16))[0]]
+    step = max(1, len(small) // 8)
+    pick = [int(order[0]), int(order[G // 4]), 0, G - 1] + small[::step][:8]
+    pick = [g for g in dict.fromkeys(pick) if m_np[g] > 0]
+    off = O.offsets(m_np)
+    for g in pick:
+        m = int(m_np[g])
+        idx = sorted(set(list(range(min(m, 24))) + list(range(max(0, m - 24), m)) + [m // 2]))
+        rows = torch.tensor([int(off[g]) + i for i in idx], device="cuda")
+        xq_h = xq.view(torch.uint8)[rows].cpu().numpy(); xs_h = xs[rows].cpu().numpy()
+        for c0 in (0, 1920, N - 128):
+            wr = slice(g * N + c0, g * N + c0 + 128)
+            ref = O.grouped_gemm_fp8(xq_h, wq.view(torch.uint8)[wr].cpu().numpy(), xs_h,
+                                     ws[(g * N + c0) // 128:(g * N + c0) // 128 + 1].cpu().numpy(), [len(idx)], 1)
+            got = to_np(y[rows, c0:c0 + 128])
+            err = rel_fro(got, ref)
+            assert err <= TOL, f"expert {g} ({m} rows) columns {c0}: {err}"
+    print(f"cfg5 full size: checked experts {pick}", flush=True)
+
+
 def test_config5_shape_sampled_experts():
     """BASELINE config 5 at full K and N (7168, 4096) with its Zipf routing, on a sample of experts (largest,
     smallest, two in between): activations quantised by the GPU quantiser, weights by the block quantiser,

@@ -87,6 +87,38 @@ def test_fused_moe_top1_and_many_experts_with_empty_ones():
     assert ok, worst
 
 
+@pytest.mark.parametrize("m,frac", [(40, 0.3), (700, 0.1), (8, 1.0)])
+def test_fused_moe_with_masked_slots(m, frac):
+    """Slots whose expert id is -1 (or beyond the last expert) contribute nothing, as in the reference's torch_moe
+    (test_moe_gemm.py:24-29: no mask matches them, their rows stay zero); frac = 1: every slot masked, result zero."""
+    import applied_ai_amd as A
+
+    n, k, e, topk = 128, 256, 8, 2
+    a, w1, w2, tw, ids = make(m, n, k, e, topk, seed=500 + m)
+    gen = torch.Generator().manual_seed(m)
+    drop = torch.rand(ids.shape, generator=gen) < frac
+    ids = torch.where(drop, torch.full_like(ids, -1), ids)
+    if m > 8:
+        ids[0, 0] = e + 3
+    print(f"fused_moe masked m={m} dropped={int(drop.sum())}", flush=True)
+    y = to_np(A.fused_moe(a.cuda(), w1.cuda(), w2.cuda(), tw.cuda(), ids.cuda()))
+    ref = O.fused_moe(a.float().numpy(), w1.float().numpy(), w2.float().numpy(), tw.numpy(), ids.numpy())
+    ok, worst = close(y, ref)
+    assert ok, worst
+    if frac == 1.0:
+        assert not y.any()
+    out = torch.full((m, topk, 2 * n), 7.0, dtype=torch.bfloat16, device="cuda")
+    A.invoke_fused_moe_kernel(a.cuda(), w1.cuda(), out, tw.cuda(), ids.cuda(), top_k=topk)
+    flat = ids.reshape(-1)
+    ref1 = np.zeros((m * topk, 2 * n), dtype=np.float32)
+    for p in range(m * topk):
+        ex = int(flat[p])
+        if 0 <= ex < e:
+            ref1[p] = a[p // topk].float().numpy() @ w1[ex].float().numpy().T
+    ok, worst = close(to_np(out).reshape(m * topk, 2 * n), ref1)
+    assert ok, worst
+
+
 def test_fused_moe_inplace_and_int32_ids_and_bf16_weights():
     import applied_ai_amd as A
 

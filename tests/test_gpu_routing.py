@@ -80,6 +80,38 @@ def test_grouping_known_answer_and_gather():
     assert torch.equal(xs.cpu(), x[(perm.cpu() // 3).long()])
 
 
+def test_masked_ids_are_dropped_and_never_gathered():
+    """Ids outside [0, E) (masked slots): perm, m_sizes and offsets bit-exact against the oracle, the unused tail of
+    perm is -1, and the gather writes zeros for it instead of reading through it."""
+    import applied_ai_amd as A
+
+    rng = np.random.default_rng(17)
+    T, k, E = 150, 4, 12
+    ids = rng.integers(0, E, size=(T, k)).astype(np.int32)
+    ids.reshape(-1)[rng.permutation(T * k)[:90]] = -1
+    ids[5, 1] = E
+    ids[149, 3] = 2 ** 30
+    operm, om = O.route(ids, E)
+    perm, m_sizes, offsets = A.route_group(torch.from_numpy(ids).cuda(), E)
+    torch.cuda.synchronize()
+    assert np.array_equal(perm.cpu().numpy(), operm)
+    assert np.array_equal(m_sizes.cpu().numpy(), om)
+    assert np.array_equal(offsets.cpu().numpy(), O.offsets(om))
+    nv = int(om.sum())
+    assert nv == int(((ids >= 0) & (ids < E)).sum()) and nv < T * k - 80
+    x = torch.randn(T, 64).to(torch.bfloat16)
+    xs = A.gather_sorted(x.cuda(), perm, k, offsets).cpu()
+    assert torch.equal(xs[:nv], x[torch.from_numpy(operm[:nv] // k).long()])
+    assert bool((xs[nv:] == 0).all())
+    # without the count the -1 entries themselves are the guard; so is an entry naming a row x does not have
+    xs2 = A.gather_sorted(x.cuda(), perm, k).cpu()
+    assert torch.equal(xs2, xs)
+    bad = perm.clone()
+    bad[0] = T * k + 5
+    xs3 = A.gather_sorted(x.cuda(), bad, k).cpu()
+    assert bool((xs3[0] == 0).all()) and torch.equal(xs3[1:], xs[1:])
+
+
 def test_routed_pipeline_end_to_end():
     """logits -> route_topk -> gather_sorted -> grouped_gemm, against the oracle run on the same bits."""
     import applied_ai_amd as A

@@ -109,10 +109,10 @@ def test_grouped_fp8_output_feeds_the_fp8_grouped_gemm():
     q, s = A.matmul_split_k_grouped(a.cuda(), torch.from_numpy(qw).cuda(), scales.cuda(), torch.from_numpy(qz).cuda(), ms,
                                     zero_offset=1, quantize_output=True)
     w2 = torch.from_numpy((rng.standard_normal((E * N2, N)) * 0.05).astype(np.float32))
-    w2q, w2s = A.float8_blockwise_quantize_weight(w2)
-    y = A.grouped_gemm_fp8_blockwise(q, w2q.cuda(), ms, s, w2s.cuda())
+    w2q, w2s = A.float8_blockwise_quantize_weight(w2.cuda())
+    y = A.grouped_gemm_fp8_blockwise(q, w2q, ms, s, w2s)
     torch.cuda.synchronize()
-    ref = O.grouped_gemm_fp8(q.view(torch.uint8).cpu().numpy(), w2q.view(torch.uint8).numpy(), s.cpu().numpy(), w2s.numpy(),
+    ref = O.grouped_gemm_fp8(q.view(torch.uint8).cpu().numpy(), w2q.view(torch.uint8).cpu().numpy(), s.cpu().numpy(), w2s.cpu().numpy(),
                              m_sizes, 1)
     assert rel_fro(to_np(y), ref) <= TOL
 

@@ -52,6 +52,21 @@ def test_route_equals_stable_argsort_and_bincount():
         assert m.tolist() == np.bincount(flat, minlength=E).tolist()
 
 
+def test_route_drops_masked_ids_and_marks_the_tail():
+    # ids outside [0, E) belong to no expert: stable argsort over the valid positions, then a tail of -1.
+    rng = np.random.default_rng(5)
+    E, n = 6, 200
+    flat = rng.integers(0, E, size=n).astype(np.int32)
+    flat[rng.permutation(n)[:37]] = -1
+    flat[[3, 77]] = [E, E + 9]
+    perm, m = O.route(flat, E)
+    valid = np.nonzero((flat >= 0) & (flat < E))[0]
+    expect = valid[np.argsort(flat[valid], kind="stable")]
+    assert perm[:len(valid)].tolist() == expect.tolist()
+    assert (perm[len(valid):] == -1).all() and len(valid) == n - 39
+    assert m.tolist() == np.bincount(flat[valid], minlength=E).tolist()
+
+
 def test_route_matches_mask_loop_grouping():
     # The reference oracle groups rows with `mask = topk_ids == i` (test_moe_gemm.py:24-29): rows of
     # expert i in increasing flat order.
@@ -229,6 +244,77 @@ def test_fp8_groupwise_quant_closed_form():
     assert (q[1, 128:] == 0xFE).all()                       # -448
     deq = O.e4m3_to_f32(q) * np.repeat(s, 128, axis=1)
     assert np.abs(deq - x).max() <= 7.0 / 448.0 * 16        # half a spacing at the top binade
+
+
+# ---- 128 x 128 weight block quantiser ------------------------------------------------------------
+# The reference takes this step from an un-vendored package, so it is pinned by what the rule fixes: constructed
+# blocks with known scale and codes, the block -> (row block, K block) index order on a non-square grid of blocks,
+# agreement with the pinned 1 x 128 quantiser where the two must coincide, and independent library routines
+# (numpy reshape / max for the scales, torch's e4m3 cast for the codes).
+def test_fp8_block_quant_weight_spikes_and_zero_block():
+    rows, K = 256, 384                                       # 2 x 3 blocks: a transposed scale index would show
+    w = np.zeros((rows, K), dtype=np.float32)
+    spikes = {(0, 0): (5, 17, 3.0), (0, 1): (127, 128 + 0, -0.75), (0, 2): (64, 256 + 127, 1e-3),
+              (1, 0): (128 + 1, 99, 448.0), (1, 2): (255, 383, -1e4)}   # block (1, 1) stays all zero
+    rng = np.random.default_rng(21)
+    for (bi, bj), (r, c, v) in spikes.items():
+        blk = w[bi * 128:(bi + 1) * 128, bj * 128:(bj + 1) * 128]
+        blk[:] = rng.uniform(-0.5, 0.5, blk.shape).astype(np.float32) * np.float32(abs(v))
+        w[r, c] = v
+    q, s = O.fp8_block_quant_weight(w, 128)
+    assert q.shape == (rows, K) and q.dtype == np.uint8 and s.shape == (2, 3) and s.dtype == np.float32
+    for (bi, bj), (r, c, v) in spikes.items():
+        assert s[bi, bj] == np.float32(abs(v)) / np.float32(448.0)
+        assert q[r, c] == (0x7E if v > 0 else 0xFE)          # the block's amax maps to +-448
+    assert s[1, 1] == np.float32(1e-12) / np.float32(448.0)
+    assert (q[128:, 128:256] == 0).all()
+    # every other element of a block is below the spike, so no other code reaches the top binade's last step
+    assert ((q & 0x7F) == 0x7E).sum() == len(spikes)
+    deq = O.e4m3_to_f32(q) * np.kron(s, np.ones((128, 128), dtype=np.float32))
+    err = np.abs(deq - w)
+    bound = np.kron(s, np.ones((128, 128), dtype=np.float32)) * 16   # half a spacing of the top binade (32 / 2)
+    assert (err <= bound).all()
+
+
+def test_fp8_block_quant_weight_vs_numpy_and_torch_cast():
+    rng = np.random.default_rng(22)
+    rows, K = 384, 256
+    w = (rng.standard_normal((rows, K)) * 0.02).astype(np.float32)
+    w[130, 7] = 0.9                                          # one dominant block
+    q, s = O.fp8_block_quant_weight(w, 128)
+    amax = np.abs(w).reshape(rows // 128, 128, K // 128, 128).max(axis=(1, 3))
+    s_np = np.maximum(amax, np.float32(1e-12)).astype(np.float32) / np.float32(448.0)
+    assert s_np.dtype == np.float32 and np.array_equal(s, s_np)
+    y = np.clip(w / np.repeat(np.repeat(s_np, 128, axis=0), 128, axis=1), -448, 448).astype(np.float32)
+    codes = torch.from_numpy(y).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(q, codes)
+
+
+def test_fp8_block_quant_weight_equals_groupwise_when_rows_share_amax():
+    # Every row of every block holds its block's largest magnitude, so the 1 x 128 groups of the (pinned)
+    # activation quantiser see the same amax as the 128 x 128 block: codes and scales must coincide.
+    rng = np.random.default_rng(23)
+    rows, K = 128, 256
+    w = rng.uniform(-1.0, 1.0, (rows, K)).astype(np.float32)
+    for bj, top in enumerate([1.5, 0.031]):
+        w[:, bj * 128:(bj + 1) * 128] *= np.float32(top) * np.float32(0.99)
+        w[np.arange(rows), bj * 128 + rng.integers(0, 128, rows)] = np.float32(top) * rng.choice([-1.0, 1.0], rows)
+    qb, sb = O.fp8_block_quant_weight(w, 128)
+    qg, sg = O.fp8_groupwise_quant(w, 128)
+    assert np.array_equal(qb, qg)
+    assert np.array_equal(sg, np.repeat(sb, rows, axis=0))
+
+
+def test_fp8_block_quant_weight_scale_equivariance():
+    # Scaling a block by a power of two scales its scale and leaves its codes alone; other blocks do not move.
+    rng = np.random.default_rng(24)
+    w = (rng.standard_normal((128, 256)) * 0.02).astype(np.float32)
+    q0, s0 = O.fp8_block_quant_weight(w, 128)
+    w2 = w.copy()
+    w2[:, 128:] *= np.float32(8.0)
+    q1, s1 = O.fp8_block_quant_weight(w2, 128)
+    assert np.array_equal(q0, q1)
+    assert s1[0, 0] == s0[0, 0] and s1[0, 1] == s0[0, 1] * np.float32(8.0)
 
 
 def test_fp8_gemm_unit_scales_reduces_to_plain_gemm():
