@@ -60,6 +60,11 @@ SIGNATURES = {
         [_c_void_p, _c_i64, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_void_p, _c_void_p,
          _c_void_p, ctypes.c_size_t, _c_void_p],
     ),
+    "moe_gg_grouped_gemm_backward_bf16_static": (
+        _c_int,
+        [_c_void_p, _c_i64, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_void_p, _c_void_p,
+         _c_void_p],
+    ),
     "moe_gg_grouped_gemm_swiglu_bf16": (
         _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_i64, _c_void_p]),
     "moe_gg_grouped_gemm_swiglu_f16": (

@@ -385,9 +385,39 @@ size_t moe_gg_grouped_gemm_backward_workspace(int G, int64_t M, int N, int K, in
   return b;
 }
 
-int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int grad_layout, const void* x, const void* w,
-                                      const int32_t* m_sizes, int G, int64_t M, int N, int K, void* grad_x, void* grad_w,
-                                      void* workspace, size_t workspace_bytes, void* stream) {
+// Scratch memory of moe_gg_grouped_gemm_backward_bf16_static: one array per device in the library's own image, so
+// that entry point never allocates. Host code must not use the array's name as an address: the per-device address
+// comes from hipGetSymbolAddress (static_scratch_ptr below).
+static __device__ __align__(256) unsigned char scratch[MOE_GG_STATIC_SCRATCH_BYTES];
+
+namespace {
+void* g_scratch_ptr[kMaxDevices];
+std::once_flag g_scratch_once[kMaxDevices];
+hipError_t g_scratch_err[kMaxDevices];
+
+// Address of `scratch` on the current device; looked up once per device with that device current.
+int static_scratch_ptr(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return MOE_GG_EDEVICE;
+  std::call_once(g_scratch_once[dev], [dev]() {
+    void* p = nullptr;
+    g_scratch_err[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    g_scratch_ptr[dev] = g_scratch_err[dev] == hipSuccess ? p : nullptr;
+  });
+  if (g_scratch_err[dev] != hipSuccess) return (int)g_scratch_err[dev];
+  if (!g_scratch_ptr[dev]) return MOE_GG_EDEVICE;
+  *out = g_scratch_ptr[dev];
+  return MOE_GG_OK;
+}
+}  // namespace
+
+// static_scratch: the workspace is the library's own array, looked up only when the call needs it, and a call
+// whose transposed copies would not fit into it is refused.
+static int backward_bf16_impl(const void* grad_out, int64_t ld_go, int grad_layout, const void* x, const void* w,
+                              const int32_t* m_sizes, int G, int64_t M, int N, int K, void* grad_x, void* grad_w,
+                              void* workspace, size_t workspace_bytes, bool static_scratch, void* stream) {
   if (G < 0 || M < 0 || N < 0 || K < 0) return MOE_GG_EINVAL;
   if (grad_layout != MOE_GG_OUT_MN && grad_layout != MOE_GG_OUT_BLOCK) return MOE_GG_EINVAL;
   const int64_t min_ld = grad_layout == MOE_GG_OUT_BLOCK ? (int64_t)N * G : (int64_t)N;
@@ -401,8 +431,8 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   // 32-bit byte offsets inside a 256-row operand tile of pitch 2 * ldm
   if (backward_ldm(G, M > 0 ? M : 1) > (1 << 22)) return MOE_GG_EUNSUPPORTED;
   if (grad_layout == MOE_GG_OUT_MN && ld_go != N) return MOE_GG_EUNSUPPORTED;
-  if (!workspace || workspace_bytes < moe_gg_grouped_gemm_backward_workspace(G, M > 0 ? M : 1, N, K, grad_layout))
-    return MOE_GG_EINVAL;
+  const size_t ws_need = moe_gg_grouped_gemm_backward_workspace(G, M > 0 ? M : 1, N, K, grad_layout);
+  if (!static_scratch && (!workspace || workspace_bytes < ws_need)) return MOE_GG_EINVAL;
   if (!aligned(grad_out, 16) || !aligned(x, 16) || !aligned(w, 16) || !aligned(grad_x, 16) || !aligned(grad_w, 16) ||
       !aligned(workspace, 256) || !aligned(m_sizes, 4))
     return MOE_GG_EALIGN;
@@ -412,11 +442,6 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   hipStream_t s = (hipStream_t)stream;
   const int64_t Mw = M > 0 ? M : 1;
   const int64_t ldm = backward_ldm(G, Mw);
-  char* ws = (char*)workspace;
-  void* wt = ws;                      ws += align256((size_t)G * N * K * 2);
-  void* dyt = ws;                     ws += align256((size_t)N * ldm * 2);
-  void* xt = ws;                      ws += align256((size_t)K * ldm * 2);
-  void* dyc = ws;
 
   hipError_t e;
   int num_wg = di->cus - di->cus % di->xcds;
@@ -431,14 +456,29 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
   const bool direct_shapes = v < 0 && N % 8 == 0 && K % 8 == 0 && ld_go % 8 == 0 &&
                              ld_go < PINGPONG_MAX_ROW_BYTES / 2 && (int64_t)K < PINGPONG_MAX_ROW_BYTES / 2 &&
                              (int64_t)N < PINGPONG_MAX_ROW_BYTES / 2;
+  // grad_x = dY [M, N] times w[g] [N, K]: from the operands as stored almost always: the other way transposes all
+  // the weights first (254 -> 143 us at 8 experts x 32 rows, N = K = 4096); only calls of a few tiles are as fast
+  // or faster through the small-tile forward kernels.
+  const int64_t gx_ntn256 = (K + 255) / 256;
+  const int64_t gx_t256 = (M / 256 + (G + 1) / 2) * gx_ntn256;
+  const bool nt_ok = direct_shapes && N % 64 == 0 && moe_gg_two_list_fits(M, G, 256, (int)gx_ntn256, num_wg) &&
+                     gx_t256 * 8 >= (int64_t)num_wg;
+  // grad_w[g] = dY_g^T X_g.
+  const int64_t t256 = (int64_t)G * ((N + 255) / 256) * ((K + 255) / 256);
+  const bool pingpong_ok = t256 <= (int64_t)(MOE_GG_SEQ_CAP - 1) * num_wg;  // its per-workgroup tile table
+  const bool gw_direct = M > 0 && direct_shapes && pingpong_ok && t256 * 4 >= (int64_t)num_wg * 3;
+  if (static_scratch && !((nt_ok || M == 0) && gw_direct)) {
+    // The call goes through transposed copies: they live in the library's own array.
+    if (ws_need > (size_t)MOE_GG_STATIC_SCRATCH_BYTES) return MOE_GG_EUNSUPPORTED;
+    rc = static_scratch_ptr(&workspace);
+    if (rc != MOE_GG_OK) return rc;
+  }
+  char* ws = (char*)workspace;
+  void* wt = ws;                      ws += align256((size_t)G * N * K * 2);
+  void* dyt = ws;                     ws += align256((size_t)N * ldm * 2);
+  void* xt = ws;                      ws += align256((size_t)K * ldm * 2);
+  void* dyc = ws;
   if (M > 0) {
-    // grad_x = dY [M, N] times w[g] [N, K].
-    const int64_t ntn256 = (K + 255) / 256;
-    const int64_t t256 = (M / 256 + (G + 1) / 2) * ntn256;
-    // Almost always: the other way transposes all the weights first (254 -> 143 us at 8 experts x 32 rows,
-    // N = K = 4096); only calls of a few tiles are as fast or faster through the small-tile forward kernels.
-    const bool nt_ok = direct_shapes && N % 64 == 0 && moe_gg_two_list_fits(M, G, 256, (int)ntn256, num_wg) &&
-                       t256 * 8 >= (int64_t)num_wg;
     if (nt_ok) {
       GgParams q{};
       q.x = grad_out; q.w = w; q.y = grad_x; q.m_sizes = m_sizes;
@@ -463,10 +503,7 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
       if (rc != MOE_GG_OK) return rc;
     }
   }
-  // grad_w[g] = dY_g^T X_g.
-  const int64_t t256 = (int64_t)G * ((N + 255) / 256) * ((K + 255) / 256);
-  const bool pingpong_ok = t256 <= (int64_t)(MOE_GG_SEQ_CAP - 1) * num_wg;  // its per-workgroup tile table
-  if (M > 0 && direct_shapes && pingpong_ok && t256 * 4 >= (int64_t)num_wg * 3) {
+  if (gw_direct) {
     GgParams q{};
     q.x = grad_out; q.w = x; q.y = grad_w; q.m_sizes = m_sizes;
     q.G = G; q.M = (int)M; q.N = N; q.K = K;
@@ -497,6 +534,20 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
     return (int)gg_bf16_pingpong_wgrad_launch(p, num_wg, s);
   if (v < 0 && t256 >= num_wg) return (int)gg_bf16_wgrad_launch(p, 256, num_wg, s);
   return (int)gg_bf16_wgrad_launch(p, 128, num_wg, s);
+}
+
+int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int grad_layout, const void* x, const void* w,
+                                      const int32_t* m_sizes, int G, int64_t M, int N, int K, void* grad_x, void* grad_w,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  return backward_bf16_impl(grad_out, ld_go, grad_layout, x, w, m_sizes, G, M, N, K, grad_x, grad_w, workspace,
+                            workspace_bytes, false, stream);
+}
+
+int moe_gg_grouped_gemm_backward_bf16_static(const void* grad_out, int64_t ld_go, int grad_layout, const void* x,
+                                             const void* w, const int32_t* m_sizes, int G, int64_t M, int N, int K,
+                                             void* grad_x, void* grad_w, void* stream) {
+  return backward_bf16_impl(grad_out, ld_go, grad_layout, x, w, m_sizes, G, M, N, K, grad_x, grad_w, nullptr, 0, true,
+                            stream);
 }
 
 static int silu_and_mul_any(const void* in, void* out, int64_t rows, int n, bool fp16, void* stream) {

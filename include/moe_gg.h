@@ -197,6 +197,24 @@ int moe_gg_grouped_gemm_backward_bf16(const void* grad_out, int64_t ld_go, int g
                                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The same backward pass for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. It takes no workspace: the
+ * transposed copies go into an array of MOE_GG_STATIC_SCRATCH_BYTES bytes that is part of the library's device
+ * image (every GPU the library runs on holds its own copy until the process ends), and the call allocates and frees
+ * nothing. Same arguments, results (bit for bit) and return codes as moe_gg_grouped_gemm_backward_bf16, plus
+ * MOE_GG_EUNSUPPORTED when the call needs transposed copies and
+ * moe_gg_grouped_gemm_backward_workspace(G, M, N, K, grad_layout) exceeds MOE_GG_STATIC_SCRATCH_BYTES (calls large
+ * enough to read their operands as stored need no copies and are not limited).
+ * All calls on one GPU share that GPU's array: calls that may overlap in time on one GPU (different streams or
+ * threads) race and must be serialised by the caller; calls on one stream are ordered and safe. Nothing in the
+ * array has to survive between calls, and every byte a call reads from it was written by that call.
+ */
+#define MOE_GG_STATIC_SCRATCH_BYTES (32 << 20)
+int moe_gg_grouped_gemm_backward_bf16_static(const void* grad_out, int64_t ld_go, int grad_layout, const void* x,
+                                             const void* w, const int32_t* m_sizes, int G, int64_t M, int N, int K,
+                                             void* grad_x, void* grad_w, void* stream);
+
+/*
  * First GEMM of a gated MoE layer with the activation fused into its epilogue. Replaces the pair
  * invoke_fused_moe_kernel(hidden_states, w1, ...) + ops.silu_and_mul
  * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:271-284):
