@@ -31,7 +31,22 @@ def _require_cuda(*tensors: torch.Tensor) -> torch.device:
     return dev
 
 
-def _grouped_gemm_bf16(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, out_layout: int) -> torch.Tensor:
+def check_m_sizes(m_sizes: torch.Tensor, M: int) -> None:
+    """The opt-in host check behind validate=True: one copy of m_sizes to the host, ValueError for a negative entry
+    or a sum beyond the M rows of x - the two cases the reference's tests expect an exception for
+    (dev/triton_groupGEMM/testing/unit_tests.py:191-212). Without it the kernels clamp such sizes on the device
+    (negative -> 0, running sum capped at M), so nothing out of bounds is ever touched; the check costs a device
+    synchronisation, which is why it is off by default."""
+    sizes = m_sizes.detach().to("cpu", torch.int64)
+    if sizes.numel() and int(sizes.min()) < 0:
+        raise ValueError(f"m_sizes has a negative entry: {sizes.tolist()}")
+    total = int(sizes.sum())
+    if total > M:
+        raise ValueError(f"sum(m_sizes) = {total} exceeds the {M} rows of x")
+
+
+def _grouped_gemm_bf16(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, out_layout: int,
+                       validate: bool = False) -> torch.Tensor:
     # Mirrors _grouped_gemm (dev/triton_groupGEMM/groupgemm.py:407-427): contiguity asserts,
     # G from m_sizes, N = w.shape[0] // G, K check, torch.empty output.
     assert x.is_contiguous()
@@ -49,6 +64,8 @@ def _grouped_gemm_bf16(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, 
         raise ValueError("grouped_gemm takes bf16 (or fp16) x and w of the same dtype")
     if m_sizes.dtype != torch.int32:
         raise ValueError("m_sizes must be int32")
+    if validate:
+        check_m_sizes(m_sizes, M)
     dev = _require_cuda(x, w, m_sizes)
     cols = N * G if out_layout == OUT_BLOCK else N
     y = torch.empty((M, cols), device=dev, dtype=x.dtype)
@@ -63,21 +80,22 @@ def _grouped_gemm_bf16(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, 
     return y
 
 
-def grouped_gemm(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor) -> torch.Tensor:
+def grouped_gemm(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, validate: bool = False) -> torch.Tensor:
     """y[off_g:off_g+m_g] = x[off_g:off_g+m_g] @ w[g*N:(g+1)*N].T for every expert g; y is [M, N] in the dtype of
     x and w (bf16 as in the reference, or fp16).
 
     Drop-in for grouped_gemm (dev/triton_groupGEMM/groupgemm.py:518-521). Rows at or beyond
     sum(m_sizes) are left uninitialised, as in the reference (torch.empty, groupgemm.py:427).
+    validate=True adds the host check of check_m_sizes (ValueError for negative sizes or sum(m_sizes) > M).
     """
-    return _grouped_gemm_bf16(x, w, m_sizes, OUT_MN)
+    return _grouped_gemm_bf16(x, w, m_sizes, OUT_MN, validate)
 
 
-def grouped_gemm_forward(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor) -> torch.Tensor:
+def grouped_gemm_forward(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, validate: bool = False) -> torch.Tensor:
     """Same product with the [M, N*G] output of the MoE-training copy: expert g writes columns
     [g*N, (g+1)*N) of its own rows (kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:626-629,
     280-289); everything else is left uninitialised."""
-    return _grouped_gemm_bf16(x, w, m_sizes, OUT_BLOCK)
+    return _grouped_gemm_bf16(x, w, m_sizes, OUT_BLOCK, validate)
 
 
 def grouped_gemm_swiglu(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor) -> torch.Tensor:
@@ -257,7 +275,8 @@ SCALE_ROWWISE = 0
 SCALE_BLOCK128 = 1
 
 
-def _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, scale_mode: int, out_layout: int = OUT_MN) -> torch.Tensor:
+def _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, scale_mode: int, out_layout: int = OUT_MN,
+                      validate: bool = False) -> torch.Tensor:
     # Mirrors _grouped_gemm with scales (dev/triton_groupGEMM/groupgemm.py:407-427, 478-494).
     assert x.is_contiguous()
     assert w.is_contiguous()
@@ -284,6 +303,8 @@ def _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, scale_mode: int, out_layo
         want_x, want_w = (M, K // 128), (G * N // 128, K // 128)
     if tuple(x_scale.shape) != want_x or tuple(w_scale.shape) != want_w:
         raise ValueError(f"scale shapes must be {want_x} and {want_w}")
+    if validate:
+        check_m_sizes(m_sizes, M)
     dev = _require_cuda(x, w, m_sizes, x_scale, w_scale)
     cols = N * G if out_layout == OUT_BLOCK else N
     y = torch.empty((M, cols), device=dev, dtype=torch.bfloat16)
@@ -297,25 +318,25 @@ def _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, scale_mode: int, out_layo
 
 
 def grouped_gemm_fp8_rowwise(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, x_scale: torch.Tensor,
-                             w_scale: torch.Tensor) -> torch.Tensor:
+                             w_scale: torch.Tensor, validate: bool = False) -> torch.Tensor:
     """fp8 grouped GEMM with one scale per activation row and per weight row:
     y = (x @ w_g.T) * x_scale[:, None] * w_scale[g*N:(g+1)*N][None, :], bf16 out.
     Drop-in for grouped_gemm_fp8_rowwise (dev/triton_groupGEMM/groupgemm.py:524-531)."""
-    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_ROWWISE)
+    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_ROWWISE, validate=validate)
 
 
 def grouped_gemm_fp8_rowwise_forward(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, x_scale: torch.Tensor,
-                                     w_scale: torch.Tensor) -> torch.Tensor:
+                                     w_scale: torch.Tensor, validate: bool = False) -> torch.Tensor:
     """The same with the [M, N*G] output of the MoE-training copy: expert g writes columns [g*N, (g+1)*N) of its
     own rows, the rest stays uninitialised. Drop-in for that copy's grouped_gemm_fp8_rowwise
     (kernels/MoE/group_GEMM/triton/tgroup_gemm_forward.py:632-639, store at :468-480)."""
-    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_ROWWISE, OUT_BLOCK)
+    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_ROWWISE, OUT_BLOCK, validate)
 
 
 def grouped_gemm_fp8_blockwise(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor, x_scale: torch.Tensor,
-                               w_scale: torch.Tensor) -> torch.Tensor:
+                               w_scale: torch.Tensor, validate: bool = False) -> torch.Tensor:
     """fp8 grouped GEMM with 1x128 activation scales x_scale[M, K/128] (the output layout of
     float8_groupwise_quantize, kernels/triton/inference/fp8/float8_groupwise_quant.py:53-91) and 128x128
     weight scales w_scale[G*N/128, K/128]; bf16 out. No counterpart in the reference (its fp8 grouped GEMM is
     row-wise only); it is the block-scaled extension of that entry point."""
-    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_BLOCK128)
+    return _grouped_gemm_fp8(x, w, m_sizes, x_scale, w_scale, SCALE_BLOCK128, validate=validate)

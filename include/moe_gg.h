@@ -4,7 +4,9 @@
  * Plain pointers and sizes only; no torch types. Every pointer marked "device" must be HIP device
  * memory on the current device. All entry points are asynchronous: they enqueue kernels on `stream`
  * (a hipStream_t passed as void*; NULL = the default stream) and return without synchronising.
- * The library keeps no per-call state, never allocates device memory and never synchronises.
+ * The library keeps no per-call state, never allocates device memory and never synchronises. Its only mutable
+ * state is process-wide and set explicitly: the kernel-variant pins of moe_gg_set_variant (a test / tuning hook,
+ * see there) and the per-device address of the static scratch array of moe_gg_grouped_gemm_backward_bf16_static.
  *
  * Return value: 0 on success, a negative MOE_GG_E* code for a rejected argument (nothing was
  * launched), or a positive hipError_t from the HIP runtime.
@@ -277,7 +279,12 @@ int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scale
 
 /*
  * Test / tuning hooks (no counterpart in the reference).
- * moe_gg_set_variant pins the kernel variant used by an op (-1 = automatic choice).
+ * moe_gg_set_variant pins the kernel variant used by an op (-1 = automatic choice). The pin is one process-global
+ * setting per op (an atomic int): it applies to every later call of that op from any thread, on any device and
+ * stream, until it is set back. It is NOT thread-safe in the sense that matters to a caller: two threads that pin
+ * different variants, or one thread that pins while another launches, see each other's setting, and a caller that
+ * pins must restore -1 itself (also on its error paths). Production code never calls it; the automatic choice is
+ * the supported mode.
  * moe_gg_host_enumerate_tiles runs the kernels' tile scheduler on the host: for a host copy of
  * m_sizes it writes, for every persistent workgroup in launch order, the tiles it would visit as
  * int32 quintuples (workgroup, group, tile_m, tile_n, first_row_of_group). Returns the number of
