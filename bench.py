@@ -21,46 +21,154 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM traffic per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what the
-# same counters read for a plain copy of known size (profiles/gg_bf16_pingpong_mixtral_prefill_traffic.md):
-# 1.94 GB fetched + 0.235 GB written.
-PREFILL_TRAFFIC_BYTES = 2.18e9
-# The same for the other workloads (profiles/bench_all_kernels_traffic.md): fetched + written bytes per launch.
-DECODE_TRAFFIC_BYTES = {"up": 0.946e9 + 1.8e6, "down": 0.957e9 + 0.5e6}
-W4A16_TRAFFIC_BYTES = {1: 32.3e6 + 0.03e6, 16: 32.3e6 + 0.46e6, 64: 44.9e6 + 1.8e6}
-W4A16_GROUPED_TRAFFIC_BYTES = 254.2e6 + 1.8e6
-W4A16_GROUPED_FP8OUT_TRAFFIC_BYTES = 254.4e6 + 1.15e6
-FP8_BLOCK_TRAFFIC_BYTES = 9.04e9 + 0.27e9
+# HBM traffic per launch of the timed kernels comes from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what
+# the same counters read for a plain copy of known size. The figures live in profiles/traffic.json together with the
+# commit they were measured at; the JSON line carries that commit ("traffic_measured_at") so that a figure older
+# than a kernel change can be told. A missing file gives traffic = null.
+def load_traffic():
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            d = json.load(f)
+        return d.get("bytes_per_launch", {}), d.get("measured_at_commit")
+    except (OSError, ValueError):
+        return {}, None
 
 
-def cpu_baseline_prefill(c, n_experts_sample=2):
-    """The reference's CPU path - a per-expert torch.matmul loop (dev/triton_groupGEMM/testing/unit_tests.py:49-55)
-    in fp32 on the host cores - timed on the first `n_experts_sample` experts of the same workload."""
+TRAFFIC, TRAFFIC_COMMIT = load_traffic()
+
+
+def cpu_info():
+    """(threads torch uses, os.cpu_count(), CPU model string)."""
     import torch
-    from oracle import oracle as O
+
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return torch.get_num_threads(), os.cpu_count(), model
+
+
+def cpu_median_seconds(fn, reps=3):
+    """1 warm-up + `reps` timed repetitions of fn(), median wall-clock seconds."""
+    fn()
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2]
+
+
+def cpu_threads():
+    import torch
 
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
     torch.set_num_threads(cores)
-    m_sizes = c["m_sizes"].tolist()[:n_experts_sample]
+    return torch.get_num_threads()
+
+
+def cpu_baseline_prefill(c):
+    """The reference's CPU path - a per-expert torch.matmul loop (dev/triton_groupGEMM/testing/unit_tests.py:49-55)
+    in fp32 on the host cores - timed on the whole workload (all experts, all rows): 1 warm-up + 3 repetitions,
+    median."""
+    from oracle import oracle as O
+
+    threads = cpu_threads()
+    m_sizes = c["m_sizes"].tolist()
     rows = sum(m_sizes)
-    N = c["w"].shape[0] // len(c["m_sizes"])
+    N = c["w"].shape[0] // len(m_sizes)
     K = c["w"].shape[1]
-    x = c["x_sorted"][:rows].float()
-    w = c["w"][: n_experts_sample * N].float()
-    O.grouped_gemm_torch_loop(x[:64], w, [64] + [0] * (n_experts_sample - 1))  # warm-up
-    times = []
-    for _ in range(2):
-        t0 = time.perf_counter()
-        O.grouped_gemm_torch_loop(x, w, m_sizes)
-        times.append(time.perf_counter() - t0)
-    t = min(times)
+    x = c["x_sorted"].float()
+    w = c["w"].float()
+    t = cpu_median_seconds(lambda: O.grouped_gemm_torch_loop(x, w, m_sizes))
+    _, ncpu, model = cpu_info()
     return {
         "value": round(2.0 * rows * N * K / t / 1e12, 3),
         "unit": "TFLOP/s",
-        "cores": torch.get_num_threads(),
+        "cores": threads,
+        "os_cpu_count": ncpu,
+        "cpu_model": model,
         "kind": "port",
-        "sample": f"first {n_experts_sample} of 8 experts ({rows} of {sum(c['m_sizes'].tolist())} rows), fp32 per-expert torch.matmul loop, best of 2",
+        "seconds": round(t, 3),
+        "extrapolated": False,
+        "sample": f"the whole workload ({rows} rows, {len(m_sizes)} experts), fp32 per-expert torch.matmul loop, 1 warm-up + 3 repetitions, median",
     }
+
+
+def cpu_baseline_decode(m_sizes, K, N):
+    """Per-expert fp32 torch.matmul loop at the decode shape (weights pre-converted to fp32, distinct per expert)."""
+    import torch
+    from oracle import oracle as O
+
+    threads = cpu_threads()
+    G = len(m_sizes)
+    gen = torch.Generator().manual_seed(3)
+    base = torch.randn(N, K, generator=gen) * 0.02
+    w = torch.empty(G * N, K)
+    for g in range(G):
+        w[g * N:(g + 1) * N] = base * (1.0 + 0.01 * g)
+    x = torch.randn(sum(m_sizes), K, generator=gen)
+    t = cpu_median_seconds(lambda: O.grouped_gemm_torch_loop(x, w, m_sizes))
+    active = sum(1 for m in m_sizes if m > 0)
+    byt = active * N * K * 4 + sum(m_sizes) * (K + N) * 4
+    return {"value": round(byt / t / 1e9, 2), "unit": "GB/s", "bytes": "fp32 operands as the CPU reads them", "cores": threads,
+            "kind": "port", "seconds": round(t, 4), "extrapolated": False,
+            "sample": "the whole workload, fp32 per-expert torch.matmul loop, 1 warm-up + 3 repetitions, median"}
+
+
+def cpu_baseline_w4a16(M, K, N):
+    """Dequantise (closed form of splitk_dequant_gemm.py:56-77) inside the timed region, then torch.matmul, fp32."""
+    import torch
+    from oracle import oracle as O
+
+    threads = cpu_threads()
+    gen = torch.Generator().manual_seed(4)
+    qw = torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, generator=gen)
+    sc = torch.rand(K // 128, N, generator=gen) * 0.015 + 0.005
+    qz = torch.randint(-2**31, 2**31 - 1, (K // 128, N // 8), dtype=torch.int32, generator=gen)
+    a = torch.randn(M, K, generator=gen)
+    t = cpu_median_seconds(lambda: O.w4a16_torch(a, qw, sc, qz, 128, 0))
+    byt = K * N // 2 + (K // 128) * N * 2 + (K // 128) * N // 2 + M * K * 2 + M * N * 2
+    return {"value": round(byt / t / 1e9, 3), "unit": "GB/s", "bytes": "the GPU path's algorithmic bytes", "cores": threads,
+            "kind": "port", "seconds": round(t, 4), "extrapolated": False,
+            "sample": "the whole workload, dequantisation inside the timed region + torch.matmul, 1 warm-up + 3 repetitions, median"}
+
+
+def cpu_baseline_fp8_block(xq, wq, xs, ws, m_sizes, N, K, n_experts=32):
+    """Config 5 on the host cores: the first `n_experts` non-empty experts (the most popular ones under the Zipf
+    routing come first), dequantisation with the block scales inside the timed per-expert loop, scaled to the whole
+    workload by FLOPs. xq / wq / xs / ws are the GPU tensors of the timed launch; only the sample is copied."""
+    import torch
+    from oracle import oracle as O
+
+    threads = cpu_threads()
+    sizes = [int(m) for m in m_sizes]
+    take, seen = 0, 0
+    for m in sizes:
+        if seen == n_experts:
+            break
+        take += 1
+        seen += m > 0
+    sample = sizes[:take]
+    rows = sum(sample)
+    xq_h = xq[:rows].view(torch.uint8).cpu()
+    xs_h = xs[:rows].cpu()
+    wq_h = wq[:take * N].view(torch.uint8).cpu()
+    ws_h = ws[:take * N // 128].cpu()
+    t = cpu_median_seconds(lambda: O.grouped_gemm_fp8_block_torch_loop(xq_h, wq_h, xs_h, ws_h, sample, N))
+    flop_sample = 2.0 * rows * N * K
+    flop_all = 2.0 * sum(sizes) * N * K
+    return {"value": round(flop_sample / t / 1e12, 3), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "seconds": round(t, 3), "extrapolated": True,
+            "seconds_whole_workload_by_flops": round(t * flop_all / flop_sample, 2),
+            "sample": f"first {seen} non-empty experts of {len(sizes)} ({rows} of {sum(sizes)} rows, {100.0 * flop_sample / flop_all:.0f} % of the FLOPs), "
+                      "per-expert dequantise + torch.matmul, 1 warm-up + 3 repetitions, median"}
 
 
 # After a change of load the GPU's power management overshoots and settles again: the first launch of the prefill
@@ -82,37 +190,61 @@ def settle(torch, fn, seconds=SETTLE_SECONDS):
 
 def event_time_ms(torch, fn, iters, warmup):
     """Average duration of fn() over `iters` back-to-back calls, HIP events on the current stream."""
+    return event_stats(torch, fn, iters, warmup, batches=1)["avg"]
+
+
+def event_stats(torch, fn, iters, warmup, batches=5):
+    """Durations of fn() in milliseconds from HIP events on the current stream: `batches` batches of
+    iters // batches back-to-back calls each, one event pair per batch (an event pair per launch would cost more than
+    the microsecond kernels it brackets). Returns the per-launch time of every batch as avg / p50 / p20 / p80."""
     settle(torch, fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    s = torch.cuda.Event(enable_timing=True)
-    e = torch.cuda.Event(enable_timing=True)
-    s.record()
-    for _ in range(iters):
-        fn()
-    e.record()
+    per = max(1, iters // batches)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(batches)]
+    for s_ev, e_ev in ev:
+        s_ev.record()
+        for _ in range(per):
+            fn()
+        e_ev.record()
     torch.cuda.synchronize()
-    return s.elapsed_time(e) / iters
+    t = sorted(s_ev.elapsed_time(e_ev) / per for s_ev, e_ev in ev)
+    n = len(t)
+    return {"avg": sum(t) / n, "p50": t[n // 2], "p20": t[n // 5], "p80": t[min(n - 1, (n * 4) // 5)],
+            "batches": n, "launches_per_batch": per}
 
 
-def secondary_workloads(torch, A, dev):
-    """Decode (config 3), W4A16 (config 4) and fp8 block-scaled (config 5) shapes: HBM-bound kernels, reported as
-    GB/s of algorithmic bytes against the 8 TB/s HBM peak. Weights rotate over enough distinct copies that the
-    footprint exceeds the 256 MB Infinity Cache. Calls go straight through the C ABI so that the ~10 us kernels
-    are not timed through Python allocation overhead."""
+def timing_fields(st, unit):
+    """JSON fields for an event_stats result; unit "us" or "ms" per launch."""
+    k = 1e3 if unit == "us" else 1.0
+    nd = 2 if unit == "us" else 3
+    return {f"{unit}_per_launch": round(st["p50"] * k, nd), f"{unit}_p20": round(st["p20"] * k, nd),
+            f"{unit}_p80": round(st["p80"] * k, nd), f"{unit}_avg": round(st["avg"] * k, nd),
+            "timing": f"median (p20, p80) over {st['batches']} batches of {st['launches_per_batch']} back-to-back launches, HIP events"}
+
+
+def hbm_roofline(kernel, byt, ms, traffic_key):
+    gbs = byt / ms / 1e6
+    return {"bound": "hbm", "kernel": kernel, "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC.get(traffic_key)}
+
+
+# The secondary workloads: decode (config 3), W4A16 (config 4) and fp8 block-scaled (config 5) shapes are HBM-bound
+# kernels, reported as GB/s of algorithmic bytes against the 8 TB/s HBM peak; the MoE layer and the backward pass as
+# TFLOP/s. Weights rotate over enough distinct copies that the footprint exceeds the 256 MB Infinity Cache. Calls go
+# straight through the C ABI so that the ~10 us kernels are not timed through Python allocation overhead. Every
+# workload is a function of its own returning a list of JSON entries; one that raises is reported as an "error" entry
+# and the others still run.
+def wl_decode(torch, A, dev, lib, stream, cpu):
     from applied_ai_amd import configs
 
-    lib = A._lib.lib()
-    stream = torch.cuda.current_stream().cuda_stream
     out = []
-
-    # ---- config 3: Mixtral decode, bf16, 64 rows over 8 experts ----
     c3 = configs.cfg3()
     m_sizes = c3["m_sizes"].tolist()
     ms_dev = c3["m_sizes"].to(dev)
     active = sum(1 for m in m_sizes if m > 0)
-    for name, K, N in (("up-proj K=4096 N=14336", 4096, 14336), ("down-proj K=14336 N=4096", 14336, 4096)):
+    for name, key, K, N in (("up-proj K=4096 N=14336", "decode_up", 4096, 14336), ("down-proj K=14336 N=4096", "decode_down", 14336, 4096)):
         x = torch.randn(64, K, device=dev).to(torch.bfloat16)
         ws = [(torch.randn(8 * N, K, device=dev) * 0.02).to(torch.bfloat16) for _ in range(2)]
         y = torch.empty(64, N, device=dev, dtype=torch.bfloat16)
@@ -123,16 +255,21 @@ def secondary_workloads(torch, A, dev):
             state["i"] += 1
             lib.moe_gg_grouped_gemm_bf16(x.data_ptr(), w.data_ptr(), y.data_ptr(), ms_dev.data_ptr(), 8, 64, N, K, N, 0, stream)
 
-        ms = event_time_ms(torch, call, 40, 6)
+        st = event_stats(torch, call, 40, 6)
+        ms = st["p50"]
         byt = active * N * K * 2 + 64 * K * 2 + 64 * N * 2
-        out.append({"workload": f"Mixtral decode bf16, T=32 top-2 (64 rows, m_sizes {m_sizes}), {name}",
-                    "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
-                    "roofline": {"bound": "hbm", "kernel": "gg_bf16_decode", "achieved": round(byt / ms / 1e6, 1),
-                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
-                                 "traffic": DECODE_TRAFFIC_BYTES[name.split("-")[0]]}})
+        e = {"workload": f"Mixtral decode bf16, T=32 top-2 (64 rows, m_sizes {m_sizes}), {name}"}
+        e.update(timing_fields(st, "us"))
+        e.update({"value": round(byt / ms / 1e6, 1), "unit": "GB/s", "roofline": hbm_roofline("gg_bf16_decode", byt, ms, key)})
         del ws
+        if cpu:
+            e["cpu_baseline"] = cpu_baseline_decode(m_sizes, K, N)
+        out.append(e)
+    return out
 
-    # ---- config 4: W4A16 split-K, K=4096, N=14336, group 128, (q - z) * s ----
+
+def wl_w4a16(torch, A, dev, lib, stream, cpu):
+    out = []
     K, N, copies = 4096, 14336, 12
     qws = [torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device=dev) for _ in range(copies)]
     sc = (torch.rand(K // 128, N, device=dev) * 0.015 + 0.005).to(torch.bfloat16)
@@ -147,23 +284,30 @@ def secondary_workloads(torch, A, dev):
             state["i"] += 1
             lib.moe_gg_w4a16_splitk(a.data_ptr(), qw.data_ptr(), sc.data_ptr(), qz.data_ptr(), c.data_ptr(), M, N, K, 128, 0, 0, stream)
 
-        ms = event_time_ms(torch, call, 120, 24)
+        st = event_stats(torch, call, 120, 24)
+        ms = st["p50"]
 
         def call_hot():  # always the same 29 MB of weights: they stay in the 256 MB last-level cache
             lib.moe_gg_w4a16_splitk(a.data_ptr(), qws[0].data_ptr(), sc.data_ptr(), qz.data_ptr(), c.data_ptr(), M, N, K, 128, 0, 0, stream)
 
-        ms_hot = event_time_ms(torch, call_hot, 120, 24)
+        ms_hot = event_stats(torch, call_hot, 120, 24)["p50"]
         byt = K * N // 2 + (K // 128) * N * 2 + (K // 128) * N // 2 + M * K * 2 + M * N * 2
-        out.append({"workload": f"W4A16 split-K M={M} K=4096 N=14336 group 128",
-                    "us_per_launch": round(ms * 1e3, 2), "cache_hot_us_per_launch": round(ms_hot * 1e3, 2),
-                    "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
-                    "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128", "achieved": round(byt / ms / 1e6, 1),
-                                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
-                                 "traffic": W4A16_TRAFFIC_BYTES.get(M)}})
-    del qws
+        e = {"workload": f"W4A16 split-K M={M} K=4096 N=14336 group 128"}
+        e.update(timing_fields(st, "us"))
+        e.update({"cache_hot_us_per_launch": round(ms_hot * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
+                  "roofline": hbm_roofline("w4a16_splitk_g128", byt, ms, f"w4a16_m{M}")})
+        if cpu:
+            e["cpu_baseline"] = cpu_baseline_w4a16(M, K, N)
+        out.append(e)
+    return out
 
-    # ---- W4A16 grouped (int4 experts), Mixtral decode: config 3's 64 rows over 8 experts, config 4's weight format ----
-    E = 8
+
+def wl_w4a16_grouped(torch, A, dev, lib, stream, cpu):
+    from applied_ai_amd import configs
+
+    out = []
+    K, N, E = 4096, 14336, 8
+    c3 = configs.cfg3()
     qwe = [torch.randint(-2**31, 2**31 - 1, (E, K // 8, N), dtype=torch.int32, device=dev) for _ in range(2)]
     sce = (torch.rand(E, K // 128, N, device=dev) * 0.015 + 0.005).to(torch.bfloat16)
     qze = torch.randint(-2**31, 2**31 - 1, (E, K // 128, N // 8), dtype=torch.int32, device=dev)
@@ -178,14 +322,15 @@ def secondary_workloads(torch, A, dev):
         lib.moe_gg_w4a16_grouped(a.data_ptr(), q.data_ptr(), sce.data_ptr(), qze.data_ptr(), c.data_ptr(), ms3.data_ptr(),
                                  E, 64, N, K, 128, 0, 0, stream)
 
-    ms = event_time_ms(torch, call, 40, 6)
+    st = event_stats(torch, call, 40, 6)
+    ms = st["p50"]
     act = sum(1 for m in c3["m_sizes"].tolist() if m > 0)
     byt = act * (K * N // 2 + K // 128 * N * 2 + K // 128 * N // 2) + 64 * K * 2 + 64 * N * 2
-    out.append({"workload": f"W4A16 grouped GEMM (int4 experts), Mixtral decode: 64 rows over 8 experts, K={K} N={N} group 128",
-                "us_per_launch": round(ms * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
-                "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128 (grid.y = experts)", "achieved": round(byt / ms / 1e6, 1),
-                             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
-                             "traffic": W4A16_GROUPED_TRAFFIC_BYTES}})
+    e = {"workload": f"W4A16 grouped GEMM (int4 experts), Mixtral decode: 64 rows over 8 experts, K={K} N={N} group 128"}
+    e.update(timing_fields(st, "us"))
+    e.update({"value": round(byt / ms / 1e6, 1), "unit": "GB/s",
+              "roofline": hbm_roofline("w4a16_splitk_g128 (grid.y = experts)", byt, ms, "w4a16_grouped")})
+    out.append(e)
 
     # the same call with the 1 x 128 fp8 quantiser as its epilogue, beside the two launches it replaces
     cq = torch.empty(64, N, device=dev, dtype=torch.uint8)
@@ -201,77 +346,85 @@ def secondary_workloads(torch, A, dev):
         call()
         lib.moe_gg_fp8_groupwise_quant(c.data_ptr(), 0, cq.data_ptr(), cs.data_ptr(), 64 * N, stream)
 
-    ms_q = event_time_ms(torch, call_q, 40, 6)
-    ms_two = event_time_ms(torch, call_two, 40, 6)
+    st_q = event_stats(torch, call_q, 40, 6)
+    ms_q = st_q["p50"]
+    ms_two = event_stats(torch, call_two, 40, 6)["p50"]
     byt_q = byt - 64 * N * 2 + 64 * N + 64 * (N // 128) * 4
-    out.append({"workload": f"W4A16 grouped GEMM with the fp8 1x128 quantiser as epilogue, same shape (fp8 codes + scales out)",
-                "us_per_launch": round(ms_q * 1e3, 2), "gemm_then_quantiser_us": round(ms_two * 1e3, 2),
-                "value": round(byt_q / ms_q / 1e6, 1), "unit": "GB/s",
-                "roofline": {"bound": "hbm", "kernel": "w4a16_splitk_g128 (fp8 output)", "achieved": round(byt_q / ms_q / 1e6, 1),
-                             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt_q / ms_q / 1e6 / PEAK_HBM_GBS, 4),
-                             "traffic": W4A16_GROUPED_FP8OUT_TRAFFIC_BYTES}})
-    del qwe
+    e = {"workload": "W4A16 grouped GEMM with the fp8 1x128 quantiser as epilogue, same shape (fp8 codes + scales out)"}
+    e.update(timing_fields(st_q, "us"))
+    e.update({"gemm_then_quantiser_us": round(ms_two * 1e3, 2), "value": round(byt_q / ms_q / 1e6, 1), "unit": "GB/s",
+              "roofline": hbm_roofline("w4a16_splitk_g128 (fp8 output)", byt_q, ms_q, "w4a16_grouped_fp8out")})
+    out.append(e)
+    return out
 
-    # ---- config 5: DeepSeek-V3-style fp8 block-scaled, 256 experts top-8, Zipf(1.1) routing ----
+
+def wl_fp8_cfg5(torch, A, dev, lib, stream, cpu):
+    """Config 5 with the inputs BASELINE states: x ~ N(0, 1) through the 1 x 128 quantiser, weights ~ N(0, 0.02)
+    through the 128 x 128 block quantiser (drawn and quantised expert by expert to bound memory)."""
+    from applied_ai_amd import configs
+
     _, _, _, m5 = configs.cfg5_routing()
     G, N, K = 256, 4096, 7168
     M = int(m5.sum())
     f8 = torch.float8_e4m3fn
-
-    def rand_fp8(rows):
-        t = torch.randint(0, 256, (rows, K), dtype=torch.uint8, device=dev)
-        return torch.where((t & 0x7F) == 0x7F, t & 0xF0, t)  # no NaN codes
-
-    xq = rand_fp8(M).view(f8)
-    wq = torch.empty(G * N, K, dtype=torch.uint8, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(1005)
+    xq, xs = A.float8_groupwise_quantize(torch.randn(M, K, generator=gen, device=dev))
+    wq = torch.empty(G * N, K, dtype=f8, device=dev)
+    ws = torch.empty(G * N // 128, K // 128, dtype=torch.float32, device=dev)
     for g in range(G):
-        wq[g * N:(g + 1) * N] = rand_fp8(N)
-    wq = wq.view(f8)
-    xs = torch.rand(M, K // 128, device=dev) * 0.01 + 0.001
-    ws = torch.rand(G * N // 128, K // 128, device=dev) * 0.01 + 0.001
+        q, sc = A.float8_blockwise_quantize_weight(torch.randn(N, K, generator=gen, device=dev) * 0.02)
+        wq[g * N:(g + 1) * N] = q
+        ws[g * N // 128:(g + 1) * N // 128] = sc
     y = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
-    ms_dev = m5.to(dev)
+    ms_dev = m5.to(torch.int32).to(dev)
 
     def call():
         lib.moe_gg_grouped_gemm_fp8(xq.data_ptr(), wq.data_ptr(), y.data_ptr(), xs.data_ptr(), ws.data_ptr(), 1,
                                     ms_dev.data_ptr(), G, M, N, K, N, 0, stream)
 
-    ms = event_time_ms(torch, call, 5, 2)
+    st = event_stats(torch, call, 10, 2, batches=5)
+    ms = st["p50"]
     active = int((m5 > 0).sum())
     byt = M * K + active * N * K + M * N * 2 + M * (K // 128) * 4 + active * (N // 128) * (K // 128) * 4
     flop = 2.0 * M * N * K
-    out.append({"workload": "DeepSeek-V3-style fp8 e4m3 block-scaled grouped GEMM: 256 experts top-8, T=4096 (32768 rows, Zipf 1.1), K=7168, N=4096",
-                "ms_per_launch": round(ms, 3), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
-                "tflops": round(flop / ms / 1e9, 1),
-                "roofline": {"bound": "hbm", "kernel": "gg_fp8_pingpong_block", "achieved": round(byt / ms / 1e6, 1),
-                             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(byt / ms / 1e6 / PEAK_HBM_GBS, 4),
-                             "traffic": FP8_BLOCK_TRAFFIC_BYTES}})
-    del xq, wq, xs, ws, y
+    e = {"workload": "DeepSeek-V3-style fp8 e4m3 block-scaled grouped GEMM: 256 experts top-8, T=4096 (32768 rows, Zipf 1.1), K=7168, N=4096; "
+                     "x ~ N(0,1) through the 1x128 quantiser, w ~ N(0,0.02) through the 128x128 block quantiser"}
+    e.update(timing_fields(st, "ms"))
+    e.update({"value": round(byt / ms / 1e6, 1), "unit": "GB/s", "tflops": round(flop / ms / 1e9, 1),
+              "roofline": hbm_roofline("gg_fp8_pingpong_block", byt, ms, "fp8_block_cfg5")})
+    if cpu:
+        e["cpu_baseline"] = cpu_baseline_fp8_block(xq, wq, xs, ws, m5.tolist(), N, K)
+    return [e]
 
-    # ---- whole MoE layer (fused_moe): Mixtral 8x7B, T=4096 top-2, bf16 ----
+
+def wl_moe_layer(torch, A, dev, lib, stream, cpu):
     T, K, n, E, topk = 4096, 4096, 14336, 8, 2
     gen = torch.Generator(device=dev).manual_seed(1002)
     h = (torch.randn(T, K, device=dev, generator=gen) / 10).to(torch.bfloat16)
     w1 = torch.empty(E, 2 * n, K, device=dev, dtype=torch.bfloat16)
     w2 = torch.empty(E, K, n, device=dev, dtype=torch.bfloat16)
-    for e in range(E):
-        w1[e] = (torch.randn(2 * n, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
-        w2[e] = (torch.randn(K, n, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    for ex in range(E):
+        w1[ex] = (torch.randn(2 * n, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        w2[ex] = (torch.randn(K, n, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
     score = torch.softmax(torch.randn(T, E, device=dev, generator=gen), dim=-1)
     tw, ids = torch.topk(score, topk)
     ids = ids.to(torch.int32)
-    ms = event_time_ms(torch, lambda: A.fused_moe(h, w1, w2, tw, ids), 10, 3)
+    st = event_stats(torch, lambda: A.fused_moe(h, w1, w2, tw, ids), 10, 3, batches=5)
+    ms = st["p50"]
     flop = 2.0 * T * topk * (2 * n * K + K * n)
-    out.append({"workload": "Mixtral 8x7B MoE layer (fused_moe: group, gather, w1 GEMM, SiLU-and-mul, w2 GEMM, top-2 combine), T=4096, bf16",
-                "m_sizes": torch.bincount(ids.flatten().long(), minlength=E).tolist(),
-                "ms_per_launch": round(ms, 3), "value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
-                "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong (two launches) + glue kernels", "achieved": round(flop / ms / 1e9, 1),
-                             "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
-                             "traffic": None}})
-    del h, w1, w2
+    e = {"workload": "Mixtral 8x7B MoE layer (fused_moe: group, gather, w1 GEMM, SiLU-and-mul, w2 GEMM, top-2 combine), T=4096, bf16",
+         "m_sizes": torch.bincount(ids.flatten().long(), minlength=E).tolist()}
+    e.update(timing_fields(st, "ms"))
+    e.update({"value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
+              "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong (two launches) + glue kernels", "achieved": round(flop / ms / 1e9, 1),
+                           "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                           "traffic": None}})
+    return [e]
 
-    # ---- backward of the grouped GEMM (training), Mixtral w1 shape, [M, N] gradient ----
+
+def wl_backward(torch, A, dev, lib, stream, cpu):
     G, M, N, K = 8, 8192, 14336, 4096
+    gen = torch.Generator(device=dev).manual_seed(1002)
     ms_dev = torch.tensor([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], dtype=torch.int32, device=dev)  # config 2's routing
     x = (torch.randn(M, K, device=dev, generator=gen) / 8).to(torch.bfloat16)
     w = torch.empty(G * N, K, device=dev, dtype=torch.bfloat16)
@@ -287,13 +440,31 @@ def secondary_workloads(torch, A, dev):
         lib.moe_gg_grouped_gemm_backward_bf16(go.data_ptr(), N, 0, x.data_ptr(), w.data_ptr(), ms_dev.data_ptr(), G, M, N, K,
                                               gx.data_ptr(), gw.data_ptr(), wsp.data_ptr(), nbytes, stream)
 
-    ms = event_time_ms(torch, call, 5, 2)
+    st = event_stats(torch, call, 10, 2, batches=5)
+    ms = st["p50"]
     flop = 4.0 * M * N * K
-    out.append({"workload": "grouped GEMM backward (grad_x and grad_w), Mixtral 8x7B w1 shape: 8192 rows, K=4096, N=14336, 8 experts, bf16",
-                "ms_per_launch": round(ms, 3), "value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
-                "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong_nt + gg_bf16_pingpong_wgrad_direct",
-                             "achieved": round(flop / ms / 1e9, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                             "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None}})
+    e = {"workload": "grouped GEMM backward (grad_x and grad_w), Mixtral 8x7B w1 shape: 8192 rows, K=4096, N=14336, 8 experts, bf16"}
+    e.update(timing_fields(st, "ms"))
+    e.update({"value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
+              "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong_nt + gg_bf16_pingpong_wgrad_direct",
+                           "achieved": round(flop / ms / 1e9, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                           "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None}})
+    return [e]
+
+
+SECONDARY = (wl_decode, wl_w4a16, wl_w4a16_grouped, wl_fp8_cfg5, wl_moe_layer, wl_backward)
+
+
+def secondary_workloads(torch, A, dev, cpu=True):
+    lib = A._lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    out = []
+    for wl in SECONDARY:
+        try:
+            out.extend(wl(torch, A, dev, lib, stream, cpu))
+        except Exception as exc:  # one workload failing must not lose the line
+            out.append({"workload": wl.__name__, "error": f"{type(exc).__name__}: {exc}"})
+        torch.cuda.empty_cache()
     return out
 
 
@@ -374,7 +545,7 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-            "traffic": PREFILL_TRAFFIC_BYTES,
+            "traffic": TRAFFIC.get("prefill_cfg2"),
             "kernel_ms": {"avg": round(avg_kernel_ms, 4), "p20": round(kern_ms[len(kern_ms) // 5], 4),
                           "p50": round(kern_ms[len(kern_ms) // 2], 4), "p80": round(kern_ms[(len(kern_ms) * 4) // 5], 4)},
         },
@@ -383,9 +554,12 @@ def main():
     # (one [8192, 4096] x [4096, 14336] product through torch.matmul -> hipBLASLt), timed the same way. With
     # random operands the MFMA clock is power-limited well below the 2.5 PFLOP/s figure, for the library too.
     wd = w[:N]
-    lib_ms = event_time_ms(torch, lambda: torch.matmul(x, wd.t()), 20, 5)
-    out["dense_gemm_library"] = {"value": round(2.0 * x.shape[0] * N * K / lib_ms / 1e9, 1), "unit": "TFLOP/s",
-                                 "what": "torch.matmul (hipBLASLt) bf16 [8192,4096]x[4096,14336], same FLOPs, no grouping"}
+    try:
+        lib_ms = event_time_ms(torch, lambda: torch.matmul(x, wd.t()), 20, 5)
+        out["dense_gemm_library"] = {"value": round(2.0 * x.shape[0] * N * K / lib_ms / 1e9, 1), "unit": "TFLOP/s",
+                                     "what": "torch.matmul (hipBLASLt) bf16 [8192,4096]x[4096,14336], same FLOPs, no grouping"}
+    except Exception as exc:
+        out["dense_gemm_library"] = {"error": f"{type(exc).__name__}: {exc}"}
     del x, w, y, wd
     if args.copy_calibration:
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
@@ -394,10 +568,14 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    out["traffic_measured_at"] = TRAFFIC_COMMIT
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_prefill(c)
+        try:
+            out["cpu_baseline"] = cpu_baseline_prefill(c)
+        except Exception as exc:
+            out["cpu_baseline"] = {"error": f"{type(exc).__name__}: {exc}"}
     if not args.no_secondary:
-        out["secondary"] = secondary_workloads(torch, A, dev)
+        out["secondary"] = secondary_workloads(torch, A, dev, cpu=not args.no_cpu_baseline)
     print(json.dumps(out))
 
 

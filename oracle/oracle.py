@@ -231,6 +231,50 @@ def grouped_gemm_torch_loop(x, w, m_sizes):
     return y
 
 
+def w4a16_torch(a, qweight, scales, qzeros, group_size=128, zero_offset=1):
+    """W4A16 on the host cores the way the reference's path states it: dequantise the GPTQ-packed weights with the
+    closed form of kernels/triton/inference/gptq/splitk_dequant_gemm.py:56-77 (vectorised torch ops, fp32), then
+    torch.matmul. Tensors in (a [M, K] float, qweight [K/8, N] int32, scales [K/g, N] float, qzeros [K/g, N/8] int32),
+    fp32 tensor out. bench.py times it (dequantisation included) as the CPU baseline of the W4A16 workloads; tests
+    check it against the scalar C form."""
+    import torch
+
+    K8, N = qweight.shape
+    shifts = torch.arange(8, dtype=torch.int32) * 4
+    q = ((qweight[:, None, :] >> shifts[None, :, None]) & 15).reshape(K8 * 8, N)
+    z = ((qzeros[:, :, None] >> shifts[None, None, :]) & 15).reshape(qzeros.shape[0], N) + zero_offset
+    w = (q - z.repeat_interleave(group_size, dim=0)).float() * scales.float().repeat_interleave(group_size, dim=0)
+    return a.float() @ w
+
+
+def grouped_gemm_fp8_block_torch_loop(xq, wq, x_scale, w_scale, m_sizes, N, block=128):
+    """Block-scaled fp8 grouped GEMM on the host cores: per expert, dequantise codes with their 1 x 128 / 128 x 128
+    scales (torch's e4m3fn cast and broadcasting) and torch.matmul, streamed one expert at a time (the per-expert
+    loop of dev/triton_groupGEMM/testing/unit_tests.py:49-55 with the dequantisation of base_testing.py:83-88 inside
+    it). xq [R, K] / wq [G*N, K] torch.float8_e4m3fn (or uint8 codes), x_scale [R, K/128], w_scale [G*N/128, K/128];
+    only the experts listed in m_sizes are computed (len(m_sizes) may be a prefix of all experts). fp32 out [R', N]."""
+    import torch
+
+    f8 = torch.float8_e4m3fn
+    if xq.dtype == torch.uint8:
+        xq = xq.view(f8)
+    if wq.dtype == torch.uint8:
+        wq = wq.view(f8)
+    K = xq.shape[1]
+    rows = int(sum(int(m) for m in m_sizes))
+    y = torch.zeros((rows, N), dtype=torch.float32)
+    start = 0
+    for g, m in enumerate(m_sizes):
+        m = int(m)
+        if m > 0:
+            xd = xq[start:start + m].float() * x_scale[start:start + m].repeat_interleave(block, dim=1)
+            sw = w_scale[g * N // block:(g + 1) * N // block]
+            wd = (wq[g * N:(g + 1) * N].float().view(N // block, block, K // block, block) * sw[:, None, :, None]).view(N, K)
+            y[start:start + m] = xd @ wd.T
+        start += m
+    return y
+
+
 def silu_and_mul(x):
     """out = silu(x[:, :n]) * x[:, n:] (ops.silu_and_mul, v0_moe_fused.py:284)."""
     x = _f32(x)

@@ -502,3 +502,37 @@ def test_grouped_gemm_backward_vs_autograd_and_closed_forms():
     gx, gw = O.grouped_gemm_backward(go, x, w, [6])
     np.testing.assert_allclose(gx, go.astype(np.float64) @ w, rtol=1e-6, atol=1e-6)
     np.testing.assert_allclose(gw, go.astype(np.float64).T @ x, rtol=1e-6, atol=1e-6)
+
+
+# ---- torch forms used as bench.py's CPU baselines ---------------------------------------------------
+def test_w4a16_torch_form_equals_the_c_form():
+    rng = np.random.default_rng(31)
+    M, K, N, g = 5, 256, 64, 128
+    q = rng.integers(0, 16, size=(K, N)).astype(np.uint8)
+    z = rng.integers(0, 16, size=(K // g, N)).astype(np.uint8)
+    sc = rng.uniform(0.005, 0.02, size=(K // g, N)).astype(np.float32)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    qw, qz = O.pack_int4_along_k(q), O.pack_int4_along_n(z)
+    for zo in (0, 1):
+        ref = O.w4a16_gemm(a, qw, sc, qz, g, zo)
+        got = O.w4a16_torch(torch.from_numpy(a), torch.from_numpy(qw), torch.from_numpy(sc), torch.from_numpy(qz), g, zo)
+        np.testing.assert_allclose(got.numpy(), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_fp8_block_torch_loop_equals_the_c_form():
+    rng = np.random.default_rng(32)
+    G, N, K = 3, 128, 256
+    m_sizes = [4, 0, 9]
+    R = sum(m_sizes)
+    x = rng.standard_normal((R, K)).astype(np.float32)
+    w = (rng.standard_normal((G * N, K)) * 0.02).astype(np.float32)
+    xq, xs = O.fp8_groupwise_quant(x)
+    wq, ws = O.fp8_block_quant_weight(w)
+    ref = O.grouped_gemm_fp8(xq, wq, xs, ws, m_sizes, 1)
+    got = O.grouped_gemm_fp8_block_torch_loop(torch.from_numpy(xq), torch.from_numpy(wq), torch.from_numpy(xs),
+                                              torch.from_numpy(ws), m_sizes, N)
+    np.testing.assert_allclose(got.numpy(), ref, rtol=1e-4, atol=1e-5)
+    # a prefix of the experts only (what the bounded baseline sample does)
+    got2 = O.grouped_gemm_fp8_block_torch_loop(torch.from_numpy(xq), torch.from_numpy(wq), torch.from_numpy(xs),
+                                               torch.from_numpy(ws), m_sizes[:1], N)
+    np.testing.assert_allclose(got2.numpy(), ref[:4], rtol=1e-4, atol=1e-5)
