@@ -1,8 +1,10 @@
-"""Random shapes and expert-size distributions: every fast path against the generic kernel (one thread per output
-element, fp32 accumulation in k order), which the other GPU tests pin against the oracle. Covers what fixed cases
-miss: tile tables with many experts, empty experts, sizes around the tile edges, N and K that are not multiples
-of the tiles. Bar: the grouped-GEMM bar of the parity tests, 1e-2 + 1e-2 |ref| on bf16 results (the two sides
-round the same fp32 sums, accumulated in different orders)."""
+"""NOT an oracle comparison: every fast kernel against the generic HIP kernel of the same library, a self-comparison
+that earns parity credit only through the chain generic kernel -> oracle (tests/test_gpu_grouped_gemm_bf16.py pins
+the generic kernel, variant 4, against the CPU oracle). Random shapes and expert-size distributions; the generic
+kernel is one thread per output element with fp32 accumulation in k order. Covers what the fixed oracle cases miss:
+tile tables with many experts, empty experts, sizes around the tile edges, N and K that are not multiples of the
+tiles. Bar: the grouped-GEMM bar of the parity tests, 1e-2 + 1e-2 |ref| on bf16 results (the two sides round the
+same fp32 sums, accumulated in different orders)."""
 import random
 
 import pytest
