@@ -166,7 +166,7 @@ def cpu_baseline_fp8_block(xq, wq, xs, ws, m_sizes, N, K, n_experts=32):
     flop_all = 2.0 * sum(sizes) * N * K
     return {"value": round(flop_sample / t / 1e12, 3), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "seconds": round(t, 3), "extrapolated": True,
-            "seconds_whole_workload_by_flops": round(t * flop_all / flop_sample, 2),
+            "seconds_whole_workload_by_flops": round(t * flop_all / flop_sample, 3),
             "sample": f"first {seen} non-empty experts of {len(sizes)} ({rows} of {sum(sizes)} rows, {100.0 * flop_sample / flop_all:.0f} % of the FLOPs), "
                       "per-expert dequantise + torch.matmul, 1 warm-up + 3 repetitions, median"}
 
