@@ -1,5 +1,5 @@
 """GPU side of the opt-in m_sizes validation of the Python mirror (the host logic itself is covered without a GPU in
-tests/test_host_checks.py). Collected late on purpose: it was added after the last GPU session of its round."""
+tests/test_host_checks.py). Collected late on purpose, so that a failure here cannot hide the parity tests before it."""
 import numpy as np
 import pytest
 import torch
