@@ -1,6 +1,6 @@
 """Benchmark of the MoE grouped-GEMM hot path on one MI355X.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu-baseline]
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu-baseline] [--moe-sweep]
 
 A step is one pass of the hot path over one batch of synthetic, HBM-resident input. The headline workload is the
 configuration the metric is quoted on: Mixtral 8x7B w1 grouped GEMM, bf16, T=4096 tokens top-2 (8192 expert-sorted
@@ -452,14 +452,39 @@ def wl_backward(torch, A, dev, lib, stream, cpu):
     return [e]
 
 
+def wl_moe_sweep(torch, A, dev, lib, stream, cpu):
+    """Context only, not a target: the sweep behind the one table of numbers the reference publishes for a
+    neighbouring kernel (kernels/triton/inference/col_major_moe_gemm/test.csv:1-11): the fused MoE layer at
+    m = 1 ... 512 tokens, n = 7168, k = 4096, 8 experts, top-2, fp16, reported with the reference's own formula
+    2 m n k / t (perf_test_moe.py:123), which counts one m x n x k GEMM for the whole two-GEMM layer."""
+    n, k, E, topk = 7168, 4096, 8, 2
+    gen = torch.Generator(device=dev).manual_seed(3227)
+    w1 = (torch.randn(E, 2 * n, k, device=dev, generator=gen) / 10).to(torch.float16)
+    w2 = (torch.randn(E, k, n, device=dev, generator=gen) / 10).to(torch.float16)
+    rows = []
+    for m in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512):
+        a = (torch.randn(m, k, device=dev, generator=gen) / 10).to(torch.float16)
+        score = torch.softmax(torch.randn(m, E, device=dev, generator=gen), dim=-1)
+        tw, ids = torch.topk(score, topk)
+        ids = ids.to(torch.int32)
+        st = event_stats(torch, lambda: A.fused_moe(a, w1, w2, tw, ids), 40, 8)
+        rows.append({"m": m, "us": round(st["p50"] * 1e3, 1), "tflops_reference_formula": round(2.0 * m * n * k / st["p50"] / 1e9, 3)})
+    return [{"workload": "fused_moe sweep as the reference's perf_test_moe.py runs it: n=7168, k=4096, 8 experts, top-2, fp16; "
+                         "TFLOPS = 2 m n k / t (one GEMM counted for the whole layer); context for test.csv:1-11, not a target",
+             "timing": "median over 5 batches of 8 back-to-back calls through the Python entry function, HIP events",
+             "rows": rows}]
+
+
 SECONDARY = (wl_decode, wl_w4a16, wl_w4a16_grouped, wl_fp8_cfg5, wl_moe_layer, wl_backward)
+# Run only on request (--moe-sweep).
+OPTIONAL = (wl_moe_sweep,)
 
 
-def secondary_workloads(torch, A, dev, cpu=True):
+def secondary_workloads(torch, A, dev, cpu=True, optional=False):
     lib = A._lib.lib()
     stream = torch.cuda.current_stream().cuda_stream
     out = []
-    for wl in SECONDARY:
+    for wl in SECONDARY + (OPTIONAL if optional else ()):
         try:
             out.extend(wl(torch, A, dev, lib, stream, cpu))
         except Exception as exc:  # one workload failing must not lose the line
@@ -475,6 +500,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
+    ap.add_argument("--moe-sweep", action="store_true",
+                    help="also time fused_moe over m = 1 ... 512 (the shape of the reference's published sweep; context only)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, so that a rocprofv3 --pmc run of this command sees a kernel of known traffic")
     args = ap.parse_args()
@@ -575,7 +602,7 @@ def main():
         except Exception as exc:
             out["cpu_baseline"] = {"error": f"{type(exc).__name__}: {exc}"}
     if not args.no_secondary:
-        out["secondary"] = secondary_workloads(torch, A, dev, cpu=not args.no_cpu_baseline)
+        out["secondary"] = secondary_workloads(torch, A, dev, cpu=not args.no_cpu_baseline, optional=args.moe_sweep)
     print(json.dumps(out))
 
 
