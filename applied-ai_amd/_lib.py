@@ -86,6 +86,7 @@ SIGNATURES = {
         [_i32_p, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _i32_p, _c_int],
     ),
     "moe_gg_host_tails_apart": (_c_int, [_i32_p, _c_int, _c_i64, _c_int, _c_int, _c_int]),
+    "moe_gg_host_tail_pieces": (_c_int, [_c_int, _c_int, _c_int]),
 }
 
 _lib = None

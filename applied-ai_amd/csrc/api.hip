@@ -663,6 +663,11 @@ int moe_gg_host_tails_apart(const int32_t* m_sizes_host, int G, int64_t M, int N
              : 0;
 }
 
+int moe_gg_host_tail_pieces(int n_long, int n_low, int num_workgroups) {
+  if (n_long < 0 || n_low < 0 || num_workgroups <= 0) return MOE_GG_EINVAL;
+  return moe_gg_tail_pieces_low(n_long, n_low, num_workgroups);
+}
+
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                           int block_n, int num_workgroups, int xcds, int32_t* out,
                                           int max_tiles) {
@@ -671,6 +676,8 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     return MOE_GG_EINVAL;
   static thread_local int32_t row_off[MOE_GG_MAX_GROUPS_ABI + 1], long_off[MOE_GG_MAX_GROUPS_ABI + 1],
       low_off[MOE_GG_MAX_GROUPS_ABI + 1];
+  // The lists of a launch that computes its low tiles itself (split tails on); the decode below is the kernels' own.
+  const bool split = true;
   const int ntn = moe_gg_cdiv(N, block_n);
   int64_t r = 0;
   int nl = 0, ns = 0;
@@ -678,13 +685,13 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     row_off[g] = (int32_t)r; long_off[g] = nl; low_off[g] = ns;
     const int m = moe_gg_clamp_rows(m_sizes_host[g], r, M);
     r += m;
-    nl += moe_gg_long_row_tiles(m, block_m) * ntn;
-    ns += moe_gg_low_row_tiles(m, block_m) * ntn;
+    nl += moe_gg_long_row_tiles2(m, block_m, split) * ntn;
+    ns += moe_gg_low_row_tiles2(m, block_m, split) * ntn;
   }
   row_off[G] = (int32_t)r; long_off[G] = nl; low_off[G] = ns;
-  const int tail_s = moe_gg_tail_pieces(nl, num_workgroups);
-  const int tail_first = moe_gg_tail_first(nl, num_workgroups);
-  const int long_ids = moe_gg_long_ids(nl, num_workgroups);
+  const int tail_s = moe_gg_tail_pieces_low(nl, ns, num_workgroups);
+  const int tail_first = moe_gg_tail_first_s(nl, num_workgroups, tail_s);
+  const int long_ids = moe_gg_long_ids_s(nl, num_workgroups, tail_s);
   const int total = long_ids + ns;
   int written = 0;
   for (int wg = 0; wg < num_workgroups; ++wg) {
@@ -693,39 +700,13 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     while ((n_long + n_low) * num_workgroups < total && moe_gg_tile_of(wg, num_workgroups, xcds, n_long + n_low) < total) ++n_low;
     const int n_my = n_long + n_low, phase = moe_gg_low_phase(wg, xcds);
     for (int seq = 0; seq < n_my; ++seq) {
-      int L = moe_gg_tile_of(wg, num_workgroups, xcds, moe_gg_seq_round(seq, n_my, n_low, phase));
+      const int L = moe_gg_tile_of(wg, num_workgroups, xcds, moe_gg_seq_round(seq, n_my, n_low, phase));
       if (written >= max_tiles) return written;
-      int g, m0, h, n0, nc = block_n;
-      if (L < long_ids) {
-        int piece = 0;
-        if (L >= tail_first) {
-          piece = (L - tail_first) % tail_s;
-          L = tail_first + (L - tail_first) / tail_s;
-        }
-        g = moe_gg_find_group(long_off, G, L);
-        const int idx = L - long_off[g];
-        const int rows = row_off[g + 1] - row_off[g];
-        const int nf = moe_gg_long_row_tiles(rows, block_m);
-        const int tn = idx / nf;
-        n0 = tn * block_n;
-        m0 = (idx - tn * nf) * block_m;
-        h = rows - m0 < block_m ? rows - m0 : block_m;
-        if (tail_s > 1 && L >= tail_first) {
-          int off;
-          moe_gg_piece_rows(h, tail_s, piece, &off, &h);
-          if (h > 0) m0 += off;
-        }
-      } else {
-        const int Lp = L - long_ids;
-        if (Lp >= ns) return MOE_GG_EINVAL;  // cannot happen
-        g = moe_gg_find_group(low_off, G, Lp);
-        n0 = (Lp - low_off[g]) * block_n;
-        const int rows = row_off[g + 1] - row_off[g];
-        m0 = rows / block_m * block_m;
-        h = rows - m0;
-      }
+      if (L >= total) return MOE_GG_EINVAL;  // cannot happen
+      const MoeGgListTile t = moe_gg_two_list_decode(row_off, long_off, low_off, G, L, long_ids, tail_first, tail_s,
+                                                     block_m, block_n, split);
       int32_t* o = out + (size_t)written * 6;
-      o[0] = wg; o[1] = g; o[2] = m0; o[3] = h; o[4] = n0; o[5] = nc;
+      o[0] = wg; o[1] = t.g; o[2] = t.m0; o[3] = t.h; o[4] = t.n0; o[5] = block_n;
       ++written;
     }
   }

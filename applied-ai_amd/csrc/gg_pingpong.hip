@@ -666,6 +666,9 @@ DEVINL void pingpong_body(const GgParams& p) {
   static_assert(2 * MOE_GG_SEQ_CAP >= MOE_GG_MAX_GROUPS + 1, "seq_tab doubles as a prefix table below");
 
   int total, total_low = 0;
+  // Forward lists: tall groups with a few rows beyond their last full tile get two half tiles for their last rows
+  // (moe_gg_split_tail), unless the small-M kernel of the same call takes the low tiles.
+  bool split = true;
   if (OP == OP_BF16_WGRAD_DIRECT) {
     build_row_offsets(p.m_sizes, p.G, p.M, row_off);
     total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
@@ -677,24 +680,28 @@ DEVINL void pingpong_body(const GgParams& p) {
     const int ntn = (OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU) ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
     const int skip = p.skip_rows;
     build_row_offsets(p.m_sizes, p.G, p.M, row_off);
-    build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
-    build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
-    total_low = uni(part_off[p.G]);
-    total = uni(tile_off[p.G]);
     if ((OP == OP_BF16 || OP == OP_F16) && p.tails_apart) {
-      // Few low tiles that would open a round of their own are computed by the small-M kernel of the same call.
+      // Few low tiles that would open a round of their own are computed by the small-M kernel of the same call,
+      // which takes the same decision from the same counts (the lists without split tails).
+      build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
+      build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
       build_tile_prefix(row_off, p.G, seq_tab, [&](int rows) { return moe_gg_low_passes(rows, BM) * ntn; });
-      if (moe_gg_tails_apart(total, total_low, uni(seq_tab[p.G]), p.tails_apart)) total_low = 0;
-      __syncthreads();  // seq_tab is rewritten below
+      if (moe_gg_tails_apart(uni(tile_off[p.G]), uni(part_off[p.G]), uni(seq_tab[p.G]), p.tails_apart)) split = false;
+      __syncthreads();  // the tables are rewritten below
     }
+    build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles2(rows, BM, split) * ntn : 0; });
+    build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles2(rows, BM, split) * ntn : 0; });
+    total_low = split ? uni(part_off[p.G]) : 0;   // split off: the low tiles are the small-M kernel's
+    total = uni(tile_off[p.G]);
   }
   const int nwg = gridDim.x;
   // Tiles of this workgroup in each list: rounds 0 .. n - 1 (tile ids grow with the round).
-  // (Forward kernels: the long tiles of a sparsely filled last round are cut into row pieces, moe_gg_tail_pieces.)
+  // (Forward kernels: the long tiles of a sparsely filled last round are cut into row pieces, as many as make the
+  // busiest workgroup's load smallest with the second list dealt behind them, moe_gg_tail_pieces_low.)
   const bool fwd = OP != OP_BF16_WGRAD && OP != OP_BF16_WGRAD_DIRECT;
-  const int tail_s = fwd ? moe_gg_tail_pieces(total, nwg) : 1;
-  const int tail_first = fwd ? moe_gg_tail_first(total, nwg) : total;
-  const int long_ids = fwd ? moe_gg_long_ids(total, nwg) : total;
+  const int tail_s = fwd ? moe_gg_tail_pieces_low(total, total_low, nwg) : 1;
+  const int tail_first = moe_gg_tail_first_s(total, nwg, tail_s);
+  const int long_ids = moe_gg_long_ids_s(total, nwg, tail_s);
   const int low_ids = total_low;
   int n_long = 0, n_low = 0;
   while (n_long * nwg < long_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < long_ids) ++n_long;
@@ -703,9 +710,10 @@ DEVINL void pingpong_body(const GgParams& p) {
   if (n_long + n_low == 0) return;
   // The sequence of this workgroup (moe_gg_seq_round), decoded once into a table: the arithmetic runs per thread
   // here; in the K loop it would occupy scalar registers that the loop needs.
-  // Tile ids: the long tiles of all groups (group, then column tile, then row tile), then the low tiles (group,
-  // column tile; see moe_gg_long_row_tiles), dealt to the workgroups round-robin: every workgroup gets the same
-  // number (+- 1) of long tiles, and the low tiles go on where the long ones stopped.
+  // Tile ids: the long tiles of all groups (group, then column tile, then row tile), then the second list (group,
+  // column tile, then the group's low tile or its two half tiles; see moe_gg_long_row_tiles, moe_gg_split_tail),
+  // dealt to the workgroups round-robin: every workgroup gets the same number (+- 1) of long tiles, and the second
+  // list goes on where the long ones stopped.
   const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
   for (int i = threadIdx.x; i < n_my; i += NT) {
     int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
@@ -724,35 +732,12 @@ DEVINL void pingpong_body(const GgParams& p) {
       n0 = (band * 4 + idx - tm * wb) * BN;
       m0 = tm * BM;
       h = min(p.N - m0, BM);
-    } else if (L < long_ids) {
-      int piece = 0;
-      if (L >= tail_first) {  // a piece of a tile of the last round
-        piece = (L - tail_first) % tail_s;
-        L = tail_first + (L - tail_first) / tail_s;
-      }
-      g = moe_gg_find_group(tile_off, p.G, L);
-      const int idx = L - tile_off[g];
-      const int rows = row_off[g + 1] - row_off[g];
-      const int nf = moe_gg_long_row_tiles(rows, BM);
-      const int tn = idx / nf;
-      n0 = tn * TC;
-      m0 = (idx - tn * nf) * BM;
-      h = min(rows - m0, BM);
-      if (tail_s > 1 && L >= tail_first) {
-        int off;
-        moe_gg_piece_rows(h, tail_s, piece, &off, &h);
-        if (h > 0) m0 += off;  // a piece without rows keeps the tile's first row: its loads must stay in bounds
-      }
     } else {
-      // Low tiles. (Cutting few low tiles into column pieces for more workgroups was measured: no gain, a low
-      // tile is bound by the per-step cost of the K loop, not by the bytes it streams.)
-      const int Lp = L - long_ids;
-      g = moe_gg_find_group(part_off, p.G, Lp);
-      const int tn = Lp - part_off[g];
-      n0 = tn * TC;
-      const int rows = row_off[g + 1] - row_off[g];
-      m0 = rows / BM * BM;
-      h = rows - m0;
+      // Long tiles (the last round cut into row pieces when it is sparsely filled), then the second list.
+      // (Cutting few low tiles into column pieces for more workgroups was measured: no gain, a low tile is bound
+      // by the per-step cost of the K loop, not by the bytes it streams.)
+      const MoeGgListTile lt = moe_gg_two_list_decode(row_off, tile_off, part_off, p.G, L, long_ids, tail_first, tail_s, BM, TC, split);
+      g = lt.g; m0 = lt.m0; h = lt.h; n0 = lt.n0;
     }
     seq_tab[2 * i] = g | (h << 16) | ((nc / 32) << 26);
     seq_tab[2 * i + 1] = (m0 / 64) | ((n0 / 32) << 16);

@@ -171,3 +171,118 @@ MOE_GG_HD void moe_gg_piece_rows(int rv, int s, int p, int* off, int* h) {
   *h = left < 0 ? 0 : (left > per ? per : left);
 }
 
+// ---- Split tails -----------------------------------------------------------------------------------
+// A tall group (at least two full row tiles) whose last rows are few (at most BM / 4) does not get a full tile plus a
+// low tile of those few rows (1 + about 0.6 tile times, the low tile bound by its K steps' load latency, not by its
+// rows), but two tiles of about half height: the last BM + rem rows are cut into BM / 2 and BM / 2 + rem rows
+// (about 0.55 tile times each). Both go into the second list, next to each other, so that they run at the same time
+// on one XCD and share their weight slabs in its L2. `split` switches the rule on; with it off the functions below
+// are moe_gg_long_row_tiles / moe_gg_low_row_tiles (the lists of a launch whose low tiles go to the small-M kernel).
+MOE_GG_HD bool moe_gg_split_tail(int rows, int BM) {
+  const int full = rows / BM, rem = rows - full * BM;
+  return full >= 2 && rem > 0 && rem * 4 <= BM;
+}
+MOE_GG_HD int moe_gg_long_row_tiles2(int rows, int BM, bool split) {
+  return split && moe_gg_split_tail(rows, BM) ? rows / BM - 1 : moe_gg_long_row_tiles(rows, BM);
+}
+MOE_GG_HD int moe_gg_low_row_tiles2(int rows, int BM, bool split) {
+  return split && moe_gg_split_tail(rows, BM) ? 2 : moe_gg_low_row_tiles(rows, BM);
+}
+
+// Row pieces of the last round of long tiles when a second list follows it: the ids after the last full round are
+// P pieces of cost a (tail * s pieces of a tile, or the tail tiles themselves), then n_low tiles of the second list
+// of cost b, dealt round-robin; s in {1, 2, 4} (s > 1 only if tail * s <= num_wg) is chosen for the smallest load of
+// the busiest workgroup. Costs in hundredths of a full tile, from timings of row pieces and low tiles.
+#define MOE_GG_COST_FULL 100
+#define MOE_GG_COST_HALF 55
+#define MOE_GG_COST_QUARTER 43
+#define MOE_GG_COST_LOW 58
+MOE_GG_HD int moe_gg_rr_max_load(int P, int a, int Q, int b, int n) {
+  // load(w) = a * (P / n + (w < P % n)) + b * #{i < Q : (P + i) % n == w}; the maximum is at one of a few w.
+  const int s0 = P % n;
+  int best = 0;
+  const int cand[5] = {0, s0, (s0 + n - 1) % n, (int)(((long long)P + Q - 1 + n) % n), (int)(((long long)P + Q) % n)};
+  for (int c = 0; c < 5; ++c) {
+    const int w = cand[c];
+    const int d = (w - s0 + n) % n;
+    const int low = Q > d ? (Q - d - 1) / n + 1 : 0;
+    const int load = a * (P / n + (w < s0 ? 1 : 0)) + b * low;
+    if (load > best) best = load;
+  }
+  return best;
+}
+MOE_GG_HD int moe_gg_tail_pieces_low(int n_long, int n_low, int num_wg) {
+  const int tail = n_long % num_wg;
+  if (tail == 0) return 1;
+  int best_s = 1, best = moe_gg_rr_max_load(tail, MOE_GG_COST_FULL, n_low, MOE_GG_COST_LOW, num_wg);
+  if (tail * 2 <= num_wg) {
+    const int l2 = moe_gg_rr_max_load(tail * 2, MOE_GG_COST_HALF, n_low, MOE_GG_COST_LOW, num_wg);
+    if (l2 < best) { best = l2; best_s = 2; }
+  }
+  if (tail * 4 <= num_wg) {
+    const int l4 = moe_gg_rr_max_load(tail * 4, MOE_GG_COST_QUARTER, n_low, MOE_GG_COST_LOW, num_wg);
+    if (l4 < best) { best = l4; best_s = 4; }
+  }
+  return best_s;
+}
+MOE_GG_HD int moe_gg_tail_first_s(int n_long, int num_wg, int s) { return s == 1 ? n_long : n_long - n_long % num_wg; }
+MOE_GG_HD int moe_gg_long_ids_s(int n_long, int num_wg, int s) {
+  const int first = moe_gg_tail_first_s(n_long, num_wg, s);
+  return first + (n_long - first) * s;
+}
+
+// Tile or row piece with id L of the two-list order: ids 0 .. long_ids - 1 are the long tiles (group, then column
+// tile, then row tile; the last round cut into tail_s pieces each from id tail_first on), the ids after them the
+// second list (group, then column tile, then the group's one or two tiles). long_off / low_off: prefix tables of
+// the tile counts of the two lists per group. The same code decodes on the device and in the host mirror. A tile
+// never reaches beyond its group's rows, whatever the tables hold (h is cut, and m0 falls back to the group's
+// first row): the kernels load from row m0 also when h is 0.
+struct MoeGgListTile { int g, m0, h, n0; };
+MOE_GG_HD MoeGgListTile moe_gg_two_list_decode(const int32_t* row_off, const int32_t* long_off, const int32_t* low_off,
+                                               int G, int L, int long_ids, int tail_first, int tail_s, int BM, int TC,
+                                               bool split) {
+  MoeGgListTile t;
+  int rows;
+  if (L < long_ids) {
+    int piece = 0;
+    if (L >= tail_first) {  // a piece of a tile of the last round
+      piece = (L - tail_first) % tail_s;
+      L = tail_first + (L - tail_first) / tail_s;
+    }
+    t.g = moe_gg_find_group(long_off, G, L);
+    const int idx = L - long_off[t.g];
+    rows = row_off[t.g + 1] - row_off[t.g];
+    int nf = moe_gg_long_row_tiles2(rows, BM, split);
+    if (nf < 1) nf = 1;
+    const int tn = idx / nf;
+    t.n0 = tn * TC;
+    t.m0 = (idx - tn * nf) * BM;
+    t.h = rows - t.m0 < BM ? rows - t.m0 : BM;
+    if (tail_s > 1 && L >= tail_first) {
+      int off;
+      moe_gg_piece_rows(t.h, tail_s, piece, &off, &t.h);
+      if (t.h > 0) t.m0 += off;  // a piece without rows keeps the tile's first row: its loads must stay in bounds
+    }
+  } else {
+    const int Lp = L - long_ids;
+    t.g = moe_gg_find_group(low_off, G, Lp);
+    rows = row_off[t.g + 1] - row_off[t.g];
+    const int idx = Lp - low_off[t.g];
+    if (split && moe_gg_split_tail(rows, BM)) {
+      const int tn = idx >> 1, half = idx & 1;
+      t.n0 = tn * TC;
+      t.m0 = (rows / BM - 1) * BM + half * (BM / 2);
+      t.h = half ? rows - t.m0 : BM / 2;
+    } else {
+      t.n0 = idx * TC;
+      t.m0 = rows / BM * BM;
+      t.h = rows - t.m0;
+    }
+  }
+  if (t.h < 0) t.h = 0;
+  if (t.m0 < 0 || t.m0 >= rows) { t.m0 = 0; t.h = 0; }
+  if (t.m0 + t.h > rows) t.h = rows - t.m0;
+  if (t.h > BM) t.h = BM;
+  return t;
+}
+

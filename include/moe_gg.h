@@ -308,14 +308,19 @@ int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,
                                 int max_tiles);
-/* The same for the 256 x 256 ping-pong kernels (block_m must be 256), which keep two tile lists (long tiles, low
- * tiles), give every workgroup its low tiles spread between its long ones, and cut the long tiles of a sparsely
- * filled last round into row pieces. Six int32 per tile here: (workgroup,
+/* The same for the 256 x 256 ping-pong kernels (block_m must be 256), which keep two tile lists (long tiles; low
+ * tiles and the two half tiles that replace the last full tile + few rows of a tall group), give every workgroup
+ * its tiles of the second list spread between its long ones, and cut the long tiles of a sparsely filled last
+ * round into row pieces. Six int32 per tile here: (workgroup,
  * group, first row inside the group, rows, first column, columns), for each workgroup in the order in which it
- * computes them; a piece may have 0 rows, and the columns may reach beyond N. */
+ * computes them; a piece may have 0 rows, and the columns may reach beyond N. The tile decode is the kernels' own
+ * code (compiled for the host). */
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                           int block_n, int num_workgroups, int xcds, int32_t* out,
                                           int max_tiles);
+/* Into how many row pieces (1, 2 or 4) the ping-pong kernels cut the long tiles of their last round when the long
+ * list has n_long tiles, the second list n_low and the launch num_workgroups workgroups. */
+int moe_gg_host_tail_pieces(int n_long, int n_low, int num_workgroups);
 
 /* bf16 forward, automatic kernel choice with 256 x 256 tiles: 1 if for these (host) m_sizes the low tiles (an
  * expert's rows beyond its last full 256-row tile, when fewer than 128 and the expert has at least two full tiles

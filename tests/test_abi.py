@@ -174,10 +174,12 @@ def test_scheduler_rejects_bad_arguments(lib):
     ("cfg5", 4096, 256),                                             # 256 experts, 32768 Zipf-routed rows (fp8 config)
 ])
 def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
-    """The ping-pong kernels' order: every output element of every group exactly once; a low tile has fewer than
-    128 rows and is the only row tile of its group or the last one of a group with at least two full tiles; the
-    long tiles of a last round that is at most half full are cut into 2 or 4 row pieces; every workgroup gets the
-    same number of tiles (+- 1)."""
+    """The ping-pong kernels' order, decoded by the kernels' own code compiled for the host: every output element of
+    every group exactly once. Second list: a low tile (fewer than 128 rows, the only row tile of its group or the last
+    one of a group with at least two full tiles and more than 64 rows left over), or the two half tiles (128 and
+    128 + rem rows) that replace the last full tile and the rem <= 64 rows behind it in a group with at least two full
+    tiles. The long tiles of a sparsely filled last round are cut into 2 or 4 row pieces; every workgroup gets the same
+    number of tiles (+- 1), and the same number (+- 1) from the second list."""
     if isinstance(m_sizes, str):
         from applied_ai_amd import configs
 
@@ -204,35 +206,122 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
                 seen[m0:m0 + h, n0:min(n0 + nc, N)] += 1
         assert (seen == 1).all(), g
 
-    def is_low(g, m0, h):
+    def kind(g, m0, h):
         m = m_sizes[g]
-        return m0 == m // 256 * 256 and h == m % 256 and 0 < h < 128 and (m // 256 >= 2 or m // 256 == 0)
+        full, rem = divmod(m, 256)
+        if full >= 2 and 0 < rem <= 64:
+            if m0 == (full - 1) * 256 and h == 128:
+                return "half0"
+            if m0 == (full - 1) * 256 + 128 and h == 128 + rem:
+                return "half1"
+            assert m0 + h <= (full - 1) * 256, (g, m0, h)      # nothing else reaches into the split rows
+            return "long"
+        if m0 == full * 256 and h == rem and 0 < h < 128 and (full >= 2 or full == 0):
+            return "low"
+        return "long"
 
-    per_wg = {}
+    per_wg, halves = {}, {}
     for wg, g, m0, h, n0, nc in tiles:
-        per_wg.setdefault(wg, []).append(is_low(g, m0, h))
+        k = kind(g, m0, h)
+        per_wg.setdefault(wg, []).append(k)
+        if k.startswith("half"):
+            halves.setdefault((g, n0), {})[k] = wg
     counts = [len(v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
     assert max(counts) - min(counts) <= 1
-    lows = [sum(v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
-    assert max(lows) - min(lows) <= 1
-    col_pieces = sum(1 for t in tiles if t[5] < 256)
-    row_pieces = sum(1 for wg, g, m0, h, n0, nc in tiles if not is_low(g, m0, h) and (m0 % 256 or h < min(256, m_sizes[g] - m0)))
+    second = [sum(k != "long" for k in v) for v in per_wg.values()] + [0] * (nwg - len(per_wg))
+    assert max(second) - min(second) <= 1
+    # the two halves of a pair are neighbours in the second list: almost always on workgroups of one XCD (wg % 8),
+    # which run them at the same time and share their weight slabs in its L2
+    assert all(len(v) == 2 for v in halves.values())
+    if halves:
+        same = sum(v["half0"] % 8 == v["half1"] % 8 for v in halves.values())
+        assert same >= 0.9 * len(halves) - 1
+    row_pieces = sum(1 for wg, g, m0, h, n0, nc in tiles
+                     if kind(g, m0, h) == "long" and (m0 % 256 or h < min(256, m_sizes[g] - m0)))
     if m_sizes[0] == 1012 and N == 14336:
-        # 7 long tiles and at most one low tile per workgroup: the XCDs (wg % 8) take their low tile at 8 different
-        # positions of the sequence, the workgroups of one XCD at the same one
-        assert col_pieces == 0 and row_pieces == 0
-        pos = {}
-        for wg, v in per_wg.items():
-            if any(v):
-                pos.setdefault(wg % 8, set()).add(v.index(True))
-        assert all(len(p) == 1 for p in pos.values())
-        assert len(pos) == 7 and len({next(iter(p)) for p in pos.values()}) == 7   # 224 low tiles: 7 XCDs of 32
+        # 1568 full tiles = 6 rounds + 32 tiles that are cut in two, then 448 half tiles: 8 rounds, every workgroup
+        # 6 full tiles and 2 tiles or pieces of about half height (before: 7 full + 1 low tile for 224 workgroups)
+        assert len(tiles) == 2048 and row_pieces == 64 and len(halves) == 4 * 56
+        for v in per_wg.values():
+            assert len(v) == 8
+        full_per_wg = {}
+        for wg, g, m0, h, n0, nc in tiles:
+            full_per_wg[wg] = full_per_wg.get(wg, 0) + (h == 256 or (kind(g, m0, h) == "long" and h >= 228))
+        assert set(full_per_wg.values()) == {6}
     if m_sizes[0] == 1012 and N == 4096:
-        # 512 long tiles = 2 full rounds, then the 64 low tiles: nothing is cut
-        assert row_pieces == 0 and col_pieces == 0 and len(tiles) == 576
+        # 448 long tiles (1.75 rounds: too many to cut), then 128 half tiles
+        assert row_pieces == 0 and len(tiles) == 576 and len(halves) == 4 * 16
     if m_sizes == [530]:
-        # 2 long tiles on 8 workgroups: 4 row pieces each; then the low tile (18 rows)
-        assert row_pieces == 8
+        # 530 = 2 x 256 + 18: one full tile, cut in two for the 8 workgroups, and the two half tiles of 128 and 146 rows
+        assert sorted((m0, h) for wg, g, m0, h, n0, nc in tiles) == [(0, 128), (128, 128), (256, 128), (384, 146)]
+
+
+def test_two_list_order_random_sizes_exact_cover(lib):
+    """Random expert counts and sizes (with sizes around the tile edges and the split rule's limits 2 x 256 + 1 .. 64,
+    and corrupt entries that the scheduler clamps): every output element once, every tile inside its group."""
+    rng = np.random.default_rng(77)
+    edge = [0, 1, 63, 64, 65, 127, 128, 129, 255, 256, 257, 319, 320, 321, 511, 512, 513, 576, 577, 640, 767, 768, 769, 832, 833]
+    for case in range(60):
+        G = int(rng.integers(1, 40))
+        sizes = [int(rng.choice(edge)) if rng.random() < 0.6 else int(rng.integers(0, 1500)) for _ in range(G)]
+        N = int(rng.choice([64, 256, 300, 512, 1000, 2048]))
+        nwg = int(rng.choice([8, 16, 64, 256, 304]))
+        ms = np.ascontiguousarray(sizes, dtype=np.int32)
+        M = int(ms.sum())
+        if case % 7 == 0 and G > 2:       # a negative entry and a sum beyond M: clamped to 0 and cut at M
+            ms = ms.copy(); ms[1] = -5
+            M = max(0, M - sizes[1] - sizes[-1] // 2)
+        eff, run = [], 0
+        for v in ms.tolist():
+            v = max(v, 0); v = min(v, M - run); run += v; eff.append(v)
+        cap = 1 << 15
+        out = np.zeros((cap, 6), dtype=np.int32)
+        n = lib.moe_gg_host_enumerate_tiles_two_lists(ms.ctypes.data_as(I32P), G, M, N, 256, 256, nwg, 8, out.ctypes.data_as(I32P), cap)
+        assert 0 <= n < cap, (case, n)
+        ntn = -(-N // 256)
+        seen = [np.zeros((m, ntn), dtype=np.int32) for m in eff]
+        for wg, g, m0, h, n0, nc in out[:n].tolist():
+            assert 0 <= wg < nwg and 0 <= g < G and eff[g] > 0, (case, wg, g)
+            assert 0 <= m0 < eff[g] and 0 <= h <= 256 and m0 + h <= eff[g] and m0 % 64 == 0 and 0 <= n0 < N and n0 % 256 == 0, (case, g, m0, h, n0)
+            if h:
+                seen[g][m0:m0 + h, n0 // 256] += 1
+        for g in range(G):
+            assert (seen[g] == 1).all(), (case, g, eff[g], N, nwg)
+
+
+def test_tail_piece_choice_minimises_the_busiest_workgroup():
+    """moe_gg_host_tail_pieces against a brute-force simulation of the round-robin dealing with the same costs
+    (hundredths of a full tile: whole 100, half piece 55, quarter piece 43, tile of the second list 58)."""
+    import ctypes
+
+    import applied_ai_amd
+
+    L = applied_ai_amd._lib.lib()
+    rng = np.random.default_rng(5)
+
+    def busiest(P, a, Q, b, n):
+        load = np.zeros(n, dtype=np.int64)
+        np.add.at(load, np.arange(P) % n, a)
+        np.add.at(load, (P + np.arange(Q)) % n, b)
+        return int(load.max())
+
+    for _ in range(400):
+        n = int(rng.choice([8, 16, 64, 256, 304]))
+        n_long = int(rng.integers(0, 6 * n))
+        n_low = int(rng.integers(0, 3 * n)) if rng.random() < 0.8 else 0
+        tail = n_long % n
+        cands = {1: busiest(tail, 100, n_low, 58, n)}
+        if tail and tail * 2 <= n:
+            cands[2] = busiest(tail * 2, 55, n_low, 58, n)
+        if tail and tail * 4 <= n:
+            cands[4] = busiest(tail * 4, 43, n_low, 58, n)
+        s = L.moe_gg_host_tail_pieces(n_long, n_low, n)
+        assert s in cands, (n_long, n_low, n, s)
+        assert cands[s] == min(cands.values()), (n_long, n_low, n, s, cands)
+    assert L.moe_gg_host_tail_pieces(512, 0, 256) == 1          # full last round
+    assert L.moe_gg_host_tail_pieces(520, 0, 256) == 4          # 8 tiles left over, no second list: quarters
+    assert L.moe_gg_host_tail_pieces(1568, 448, 256) == 2       # Mixtral prefill: 32 tiles in halves + 448 half tiles = 2 rounds
+    assert L.moe_gg_host_tail_pieces(-1, 0, 256) < 0
 
 
 def test_tails_apart_decision():
