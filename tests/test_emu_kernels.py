@@ -1,0 +1,255 @@
+"""The library's device code on the CPU: every .hip source compiled as host C++ behind a stand-in HIP header
+(tests/emu) and run under a lockstep-wave emulation, called through the same C ABI as on the GPU and checked against
+the oracle. This covers what the host-side tests cannot reach without a GPU: the indexing of the kernels, their tile
+tables, LDS layouts, MFMA fragment layouts, wave-level exchanges, the counted waits behind the global->LDS loads, and
+the dispatch in api.hip. It says nothing about speed, and rounding inside a matrix instruction may differ from the
+hardware's, so products are checked bit-exactly only on data whose sums are exact (small integers, power-of-two
+scales) and to the GPU tests' tolerance otherwise."""
+import ctypes
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EMU = os.path.join(ROOT, "tests", "emu")
+sys.path.insert(0, EMU)
+
+import build_emu  # noqa: E402
+
+if not os.path.exists(build_emu.CXX):
+    pytest.skip("host clang++ of the ROCm toolchain not found: the emulated build needs it", allow_module_level=True)
+
+import harness as H  # noqa: E402
+from oracle import oracle as O  # noqa: E402
+
+
+@pytest.fixture(scope="module", autouse=True)
+def built():
+    H.lib()
+
+
+def ints(rng, shape, lo=-4, hi=5):
+    return rng.integers(lo, hi, shape).astype(np.float32)
+
+
+def exact16(got16, want, fp16=False):
+    mask = ~np.isnan(want)
+    got = H.from16(got16, fp16)
+    return bool((got[mask] == H.from16(H.to16(np.nan_to_num(want), fp16), fp16)[mask]).all())
+
+
+SIZES = [300, 0, 70, 530]   # a full tile + a low tile, an empty expert, a short one, a tall one whose tail is split
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, -1])
+def test_bf16_every_kernel_variant(variant):
+    rng = np.random.default_rng(variant + 1)
+    x, w = ints(rng, (sum(SIZES), 128)), ints(rng, (4 * 512, 128))
+    y = H.grouped_gemm(H.to_bf16(x), H.to_bf16(w), SIZES, 512, variant=variant)
+    assert exact16(y, O.grouped_gemm(x, w, SIZES))
+
+
+@pytest.mark.parametrize("fp16,block", [(True, False), (False, True), (True, True)])
+def test_fp16_and_block_layout(fp16, block):
+    rng = np.random.default_rng(7)
+    x, w = ints(rng, (sum(SIZES), 128)), ints(rng, (4 * 256, 128))
+    y = H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), SIZES, 256, fp16=fp16, block_layout=block)
+    ref = O.grouped_gemm(x, w, SIZES, block_layout=block)
+    assert exact16(y, ref, fp16)
+    assert (y[np.isnan(ref)] == H.NAN16).all()   # the other experts' column blocks stay untouched
+
+
+@pytest.mark.parametrize("sizes,N,K", [([3, 0, 7, 5], 256, 256), ([1], 64, 128), ([20, 10, 20], 33, 40), ([0, 0, 70, 0, 0], 100, 72),
+                                       ([4] * 32, 16, 16)])
+def test_small_and_odd_shapes_take_the_decode_and_generic_kernels(sizes, N, K):
+    rng = np.random.default_rng(len(sizes))
+    x, w = ints(rng, (sum(sizes), K)), ints(rng, (len(sizes) * N, K))
+    for fp16 in (False, True):
+        assert exact16(H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), sizes, N, fp16=fp16), O.grouped_gemm(x, w, sizes), fp16)
+
+
+@pytest.mark.parametrize("sizes", [[530], [520, 30]])
+def test_low_tiles_computed_by_the_small_m_kernel(sizes):
+    """K >= 8192 with few experts: the ping-pong launch leaves the rows behind the last full tile to a launch of the
+    small-M kernel (both decide it from m_sizes on the device)."""
+    G, M, N, K = len(sizes), sum(sizes), 256, 8192
+    ms = np.array(sizes, dtype=np.int32)
+    assert H.lib().moe_gg_host_tails_apart(ms.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), G, M, N, K, 8) == 1
+    rng = np.random.default_rng(1)
+    x, w = ints(rng, (M, K), -2, 3), ints(rng, (G * N, K), -2, 3)
+    assert exact16(H.grouped_gemm(H.to_bf16(x), H.to_bf16(w), sizes, N), O.grouped_gemm(x, w, sizes))
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, -1])
+def test_fp8_every_kernel_variant(mode, variant):
+    rng = np.random.default_rng(10 * mode + variant + 3)
+    sizes, N, K = [300, 0, 70, 30, 530], 256, 256
+    G, M = len(sizes), sum(sizes)
+    xq = (rng.integers(0, 0x40, (M, K)) | (rng.integers(0, 2, (M, K)) << 7)).astype(np.uint8)
+    wq = (rng.integers(0, 0x40, (G * N, K)) | (rng.integers(0, 2, (G * N, K)) << 7)).astype(np.uint8)
+    xs = (2.0 ** rng.integers(-2, 3, M if mode == 0 else (M, K // 128))).astype(np.float32)
+    ws = (2.0 ** rng.integers(-2, 3, G * N if mode == 0 else (G * N // 128, K // 128))).astype(np.float32)
+    y = H.grouped_gemm_fp8(xq, wq, xs, ws, mode, sizes, N, variant)
+    assert exact16(y, O.grouped_gemm_fp8(xq, wq, xs, ws, sizes, mode))
+
+
+@pytest.mark.parametrize("fp16", [False, True])
+def test_fused_silu_and_mul_gemm(fp16):
+    rng = np.random.default_rng(5)
+    n, K = 192, 128
+    x = (rng.standard_normal((sum(SIZES), K)) * 0.5).astype(np.float32)
+    w = (rng.standard_normal((4 * 2 * n, K)) * 0.1).astype(np.float32)
+    x16, w16 = H.to16(x, fp16), H.to16(w, fp16)
+    got = H.from16(H.grouped_gemm_swiglu(x16, w16, SIZES, n, fp16), fp16)
+    want = O.silu_and_mul(O.grouped_gemm(H.from16(x16, fp16), H.from16(w16, fp16), SIZES))
+    np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("sizes,N,K,block,static", [
+    (SIZES, 256, 128, False, False), (SIZES, 256, 128, True, False), (SIZES, 256, 128, False, True),
+    ([30, 0, 7, 53], 64, 64, False, False), ([0, 5, 0], 64, 64, False, False), ([300, 200], 68, 36, False, False)])
+def test_backward(sizes, N, K, block, static):
+    rng = np.random.default_rng(N + K)
+    G, M = len(sizes), sum(sizes)
+    x, w = ints(rng, (M, K), -2, 3), ints(rng, (G * N, K), -2, 3)
+    go = ints(rng, (M, N * G if block else N), -2, 3)
+    gx, gw = H.backward(H.to_bf16(go), H.to_bf16(x), H.to_bf16(w), sizes, N, block, static)
+    ox, ow = O.grouped_gemm_backward(go, x, w, sizes)
+    assert exact16(gx, ox) and exact16(gw, ow)   # experts without rows: zero grad_w, written
+
+
+def w4_inputs(rng, E, K, N, gs):
+    qv, zv = rng.integers(0, 16, (E, K, N)), rng.integers(0, 15, (E, K // gs, N))
+    qw = np.stack([O.pack_int4_along_k(qv[e]) for e in range(E)])
+    qz = np.stack([O.pack_int4_along_n(zv[e]) for e in range(E)])
+    return qw, qz, (2.0 ** rng.integers(-3, 1, (E, K // gs, N))).astype(np.float32)
+
+
+@pytest.mark.parametrize("M,N,K,gs,fp16", [(1, 256, 512, 128, False), (5, 128, 256, 128, True), (16, 192, 256, 128, False),
+                                           (33, 128, 256, 64, False), (70, 64, 256, 128, False)])
+def test_w4a16_splitk(M, N, K, gs, fp16):
+    rng = np.random.default_rng(M)
+    qw, qz, sc = w4_inputs(rng, 1, K, N, gs)
+    a = ints(rng, (M, K), -2, 3)
+    c = H.w4a16(H.to16(a, fp16), qw[0], H.to16(sc[0], fp16), qz[0], gs, 1, fp16)
+    assert exact16(c, O.w4a16_gemm(a, qw[0], sc[0], qz[0], gs, 1), fp16)
+
+
+def test_w4a16_grouped_and_its_fp8_epilogue():
+    rng = np.random.default_rng(4)
+    sizes, N, K = [3, 0, 9, 12], 256, 256
+    qw, qz, sc = w4_inputs(rng, 4, K, N, 128)
+    a = ints(rng, (sum(sizes), K), -2, 3)
+    want = O.w4a16_grouped(a, qw, sc, qz, sizes, 128, 1)
+    assert exact16(H.w4a16(H.to_bf16(a), qw, H.to_bf16(sc), qz, 128, 1, False, sizes), want)
+    cq, cs = H.w4a16(H.to_bf16(a), qw, H.to_bf16(sc), qz, 128, 1, False, sizes, fp8out=True)
+    oq, os_ = O.fp8_groupwise_quant(O.round_bf16(want))
+    assert (cq == oq).all() and (cs == os_).all()
+
+
+def test_routing_kernels():
+    rng = np.random.default_rng(6)
+    T, E, k = 300, 8, 2
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[5] = 0.25                                   # ties go to the lower expert index
+    ids, perm, ms, off = H.route_topk(logits, k)
+    oi = O.topk(logits, k)
+    op, om = O.route(oi, E)
+    assert (ids == oi).all() and (perm == op).all() and (ms == om).all() and (off == O.offsets(om)).all()
+    flat = rng.integers(-1, E + 1, 1000)               # ids outside [0, E) are masked slots
+    perm, ms, off = H.route_group(flat, E)
+    op, om = O.route(flat, E)
+    assert (perm == op).all() and (ms == om).all()
+    keep = flat[(flat >= 0) & (flat < E)]
+    s, e, post = H.align_block_size(perm, ms, 16)
+    os_, oe, opost = O.moe_align_block_size(keep, 16, E)
+    assert post == opost and (e[:post // 16] == oe[:post // 16]).all()
+    # the sorted list holds positions of the unmasked list in the oracle and of the full list in the kernel: compare experts
+    pad = len(flat)
+    for blk in range(post // 16):
+        mine = s[16 * blk:16 * blk + 16]
+        assert all(flat[i] == e[blk] for i in mine if i < pad)
+    nv = int(ms.sum())
+    x = rng.integers(0, 60000, (500, 64)).astype(np.uint16)
+    g = H.gather_rows(x, perm, 2, n_valid=nv)
+    assert (g[:nv] == x[perm[:nv] // 2]).all() and (g[nv:] == 0).all()
+    inv = H.invert_perm(perm, n_valid=nv)             # masked positions keep what the buffer held
+    assert (inv[perm[:nv]] == np.arange(nv)).all() and (np.delete(inv, perm[:nv]) == -7).all()
+
+
+def test_quantisers_bit_exact():
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((64, 512)) * 3).astype(np.float32)
+    x[3, :128] = 0.0                                   # an all-zero group: scale from the 1e-12 floor
+    for bf16_in in (False, True):
+        q, s = H.fp8_groupwise_quant(x, bf16_in)
+        oq, os_ = O.fp8_groupwise_quant(O.round_bf16(x) if bf16_in else x)
+        assert (q == oq).all() and (s == os_).all()
+    w = (rng.standard_normal((256, 384)) * 0.02).astype(np.float32)
+    for bf16_in in (False, True):
+        q, s = H.fp8_block128_quant(w, bf16_in)
+        oq, os_ = O.fp8_block_quant_weight(O.round_bf16(w) if bf16_in else w)
+        assert (q == oq).all() and (s == os_).all()
+
+
+def test_moe_layer_as_the_sequence_of_abi_calls():
+    """fused_moe's launch sequence (route, gather, w1 GEMM with SiLU-and-mul, w2 GEMM, un-permute and weighted sum)
+    on numpy buffers, against the layer oracle."""
+    rng = np.random.default_rng(9)
+    T, E, k, K, n, d = 96, 4, 2, 128, 128, 64
+    a = (rng.standard_normal((T, K)) * 0.5).astype(np.float32)
+    w1 = (rng.standard_normal((E, 2 * n, K)) * 0.1).astype(np.float32)
+    w2 = (rng.standard_normal((E, d, n)) * 0.1).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    a16, w1_16, w2_16 = H.to_bf16(a), H.to_bf16(w1), H.to_bf16(w2)
+    ids, perm, ms, off = H.route_topk(logits, k)
+    tw = np.take_along_axis(np.exp(logits) / np.exp(logits).sum(1, keepdims=True), ids, axis=1).astype(np.float32)
+    xs = H.gather_rows(a16, perm, k)
+    h = H.grouped_gemm_swiglu(xs, w1_16.reshape(E * 2 * n, K), ms, n)
+    y = H.grouped_gemm(h, w2_16.reshape(E * d, n), ms, d)
+    out = H.from_bf16(H.combine_topk(y, H.invert_perm(perm), tw, T, k))
+    want = O.fused_moe(H.from_bf16(a16), H.from_bf16(w1_16), H.from_bf16(w2_16), tw, ids)
+    np.testing.assert_allclose(out, want, rtol=2e-2, atol=2e-2)
+
+
+def test_glue_kernels():
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((50, 256)).astype(np.float32)
+    for fp16 in (False, True):
+        x16 = H.to16(x, fp16)
+        np.testing.assert_allclose(H.from16(H.silu_and_mul(x16, fp16), fp16), O.silu_and_mul(H.from16(x16, fp16)), rtol=1e-2, atol=1e-2)
+    T, k, d = 32, 2, 64
+    inv = rng.permutation(T * k).astype(np.int32)
+    y = ints(rng, (T * k, d))
+    wts = (2.0 ** rng.integers(-2, 1, (T, k))).astype(np.float32)
+    want = (wts[:, :, None] * y[inv].reshape(T, k, d)).sum(1)
+    for w16 in (False, True):
+        assert exact16(H.combine_topk(H.to_bf16(y), inv, wts, T, k, weights_16bit=w16), want)
+
+
+def test_argument_checks_reach_the_caller():
+    L = H.lib()
+    buf = np.zeros(64, dtype=np.uint16)
+    ms = np.array([1], dtype=np.int32)
+    assert L.moe_gg_grouped_gemm_bf16(None, H.P(buf), H.P(buf), H.P(ms), 1, 1, 8, 8, 8, 0, None) == -1
+    assert L.moe_gg_grouped_gemm_bf16(H.P(buf), H.P(buf), H.P(buf), H.P(ms), 2000, 1, 8, 8, 8, 0, None) == -4
+    assert L.moe_gg_grouped_gemm_fp8(H.P(buf), H.P(buf), H.P(buf), H.P(buf), H.P(buf), 1, H.P(ms), 1, 1, 128, 100, 128, 0, None) != 0
+
+
+FUZZ = [  # (compute units, load-landing model, wave order seed): few units = long tile sequences per workgroup
+    ("1", "late", "0"), ("2", "early", "0"), ("3", "late", "5"), ("8", "early", "9"), ("16", "late", "0"), ("5", "late", "77")]
+
+
+def test_pingpong_random_shapes_over_unit_counts_and_schedules():
+    procs = []
+    for i, (cus, dma, seed) in enumerate(FUZZ):
+        env = dict(os.environ, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed)
+        procs.append(subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_pingpong.py"), str(100 + i), "20"], env=env,
+                                      stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT))
+    for cfg, p in zip(FUZZ, procs):
+        log = p.communicate()[0].decode()
+        assert p.returncode == 0, (cfg, log[-2000:])
