@@ -14,8 +14,9 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
-CSRC = os.path.join(ROOT, "applied-ai_amd", "csrc")
-OUT = os.path.join(HERE, "_build")
+# EMU_CSRC / EMU_OUT: build another copy of the sources (a kernel under development) into another folder.
+CSRC = os.environ.get("EMU_CSRC") or os.path.join(ROOT, "applied-ai_amd", "csrc")
+OUT = os.environ.get("EMU_OUT") or os.path.join(HERE, "_build")
 CXX = "/opt/rocm/llvm/bin/clang++"
 FLAGS = ["-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-attributes", "-Wno-unused-value",
          "-Wno-ignored-attributes", "-I", os.path.join(HERE, "include"), "-I", CSRC]
@@ -64,7 +65,8 @@ def _asm_rule(template, outs, ins, where):
     if "global_load_lds_dwordx4" in t or "global_load_lds_dword " in t:
         assert "s_mov_b32 m0, %0" in t and len(ins) == 3 and not outs, where
         lds, voff, sbase = ins
-        return "emu::dma(%d, %s, %s, %s)" % (16 if "dwordx4" in t else 4, sbase, voff, lds)
+        # (the base may be a pointer with a device address space)
+        return "emu::dma(%d, (const void*)(uintptr_t)(%s), %s, %s)" % (16 if "dwordx4" in t else 4, sbase, voff, lds)
     m = re.fullmatch(r"\s*s_waitcnt vmcnt\((%0|\d+)\)\s*", t)
     if m:
         return "emu::wait_vm(%s)" % (ins[0] if m.group(1) == "%0" else m.group(1))

@@ -69,7 +69,7 @@ struct Wave {
   int alive, waiting;
   bool wait[64];
   const void* site[64];          // where the lane waits (the call that started the exchange, or its end)
-  uint64_t stamp[64];            // when it arrived
+  uint64_t epoch[64];            // how often the lane has moved backwards in the code (loop iterations, roughly)
   unsigned long long mask[64];   // lanes of the exchange the lane was released from last
   alignas(16) unsigned char slot[64][64];
 };
@@ -89,22 +89,30 @@ uint64_t g_nonuniform = 0;
 
 void yield() { emu_switch(&g_cur->ctx, &g_sched); }
 
-uint64_t g_clock = 0, g_divergent = 0;
+uint64_t g_divergent = 0;
 // Lanes of a wave that wait at the same place are released together once no lane of the wave can still join them:
 // all live lanes wait at exchanges (force = false), or nothing in the workgroup can run (force = true). When they wait
-// at different places (lanes took different branches, or left a loop at different times), the lanes that arrived last
-// go first: they are the ones behind, and the others meet them again further down.
+// at different places (lanes took different branches, or left a loop at different times), the lanes that are behind
+// in the program go first and meet the others further down, as the hardware runs a branch to its join point.
+// "Behind" is judged by (epoch, code address): a lane's epoch goes up whenever its next exchange lies at a lower
+// address than its last one (a loop's back edge); lanes released together continue with the same epoch.
 void try_release(Wave& w, bool force) {
   if (w.waiting == 0 || (!force && w.waiting < w.alive)) return;
   int pick = -1;
   for (int l = 0; l < 64; ++l)
-    if (w.wait[l] && (pick < 0 || w.stamp[l] > w.stamp[pick])) pick = l;
+    if (w.wait[l] && (pick < 0 || w.epoch[l] < w.epoch[pick] || (w.epoch[l] == w.epoch[pick] && w.site[l] < w.site[pick]))) pick = l;
   unsigned long long m = 0;
+  uint64_t top = 0;
   for (int l = 0; l < 64; ++l)
-    if (w.wait[l] && w.site[l] == w.site[pick]) m |= 1ull << l;
+    if (w.wait[l] && w.site[l] == w.site[pick]) { m |= 1ull << l; top = std::max(top, w.epoch[l]); }
   for (int l = 0; l < 64; ++l)
-    if ((m >> l) & 1) { w.wait[l] = false; w.mask[l] = m; --w.waiting; }
-  if (__builtin_popcountll(m) != w.alive) ++g_divergent;
+    if ((m >> l) & 1) { w.wait[l] = false; w.mask[l] = m; w.epoch[l] = top; --w.waiting; }
+  if (__builtin_popcountll(m) != w.alive && g_divergent++ < 8 && getenv("EMU_TRACE")) {
+    Dl_info info;
+    dladdr(w.site[pick], &info);
+    fprintf(stderr, "emu: exchange among part of a wave: lanes %016llx of %d live ones, caller +0x%zx (block %u wave %d)\n", m, w.alive,
+            (size_t)((const char*)w.site[pick] - (const char*)info.dli_fbase), blockIdx.x, (int)(&w - g_w));
+  }
 }
 void release_barrier() {
   g_bar_arrived = 0;
@@ -137,8 +145,8 @@ void wave_sync(const void* site) {
   Wave& w = g_w[f->tid >> 6];
   const int l = f->tid & 63;
   w.wait[l] = true;
+  if (site < w.site[l]) ++w.epoch[l];
   w.site[l] = site;
-  w.stamp[l] = ++g_clock;
   ++w.waiting;
   try_release(w, false);
   if (!w.wait[l]) return;
@@ -183,6 +191,8 @@ void run_workgroup(unsigned order_seed) {
     g_w[w].alive = std::min(64, nt - 64 * w);
     g_w[w].waiting = 0;
     memset(g_w[w].wait, 0, sizeof(g_w[w].wait));
+    memset(g_w[w].site, 0, sizeof(g_w[w].site));
+    memset(g_w[w].epoch, 0, sizeof(g_w[w].epoch));
   }
   g_alive = nt;
   g_bar_arrived = 0;

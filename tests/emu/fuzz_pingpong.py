@@ -43,8 +43,9 @@ def one_case(rng):
         mode = 0 if op == "fp8row" else 1
         K = 128 * int(rng.integers(1, 3))
         N = max(128, N // 128 * 128)
-        xq = rng.integers(0, 0x40, (M, K)).astype(np.uint8)
-        wq = rng.integers(0, 0x40, (G * N, K)).astype(np.uint8)
+        # magnitudes 0.5 ... 3.75: every partial sum is exact in fp32
+        xq = ((0x30 + rng.integers(0, 0x18, (M, K))) | (rng.integers(0, 2, (M, K)) << 7)).astype(np.uint8)
+        wq = ((0x30 + rng.integers(0, 0x18, (G * N, K))) | (rng.integers(0, 2, (G * N, K)) << 7)).astype(np.uint8)
         xs = np.ones(M if mode == 0 else (M, K // 128), np.float32)
         ws = np.ones(G * N if mode == 0 else (G * N // 128, K // 128), np.float32)
         y = H.grouped_gemm_fp8(xq, wq, xs, ws, mode, sizes, N, variant=3)

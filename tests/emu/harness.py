@@ -16,6 +16,13 @@ import build_emu  # noqa: E402
 from applied_ai_amd import _lib  # noqa: E402
 
 _L = None
+# GUARD = "end" / "start": every array handed to the library is copied into memory that ends (begins) at an
+# inaccessible page, so that a kernel reading or writing past the end (before the start) of a tensor faults at once
+# instead of touching a neighbour. None: plain numpy arrays.
+GUARD = os.environ.get("EMU_GUARD") or None
+_keep = []
+_libc = ctypes.CDLL(None, use_errno=True)
+_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
 BF16, FP16, FP32 = 0, 1, 2
 OP_BF16, OP_FP8 = 0, 1
 
@@ -32,11 +39,52 @@ def lib():
     return _L
 
 
+def guarded(a):
+    """A copy of `a` whose last (first) byte, up to 16-byte alignment, is followed (preceded) by a page without access."""
+    import mmap
+
+    a = np.ascontiguousarray(a)
+    n = (a.nbytes + 15) // 16 * 16
+    pages = (n + 4095) // 4096 + 2
+    m = mmap.mmap(-1, pages * 4096)
+    base = ctypes.addressof(ctypes.c_char.from_buffer(m))
+    for page in (0, pages - 1):
+        if _libc.mprotect(base + page * 4096, 4096, 0) != 0:
+            raise OSError(ctypes.get_errno(), "mprotect")
+    off = 4096 if GUARD == "start" else (pages - 1) * 4096 - n
+    out = np.frombuffer(m, dtype=a.dtype, count=a.size, offset=off).reshape(a.shape)
+    out[...] = a
+    _keep.append(m)
+    return out
+
+
+_guarded_ptrs = set()
+
+
+def G(a):
+    """Input or output array as the library sees it (guarded when GUARD is set)."""
+    if a is None or GUARD is None or a.size == 0 or a.ctypes.data in _guarded_ptrs:
+        return a
+    g = guarded(a)
+    _guarded_ptrs.add(g.ctypes.data)
+    return g
+
+
+def _full(shape, fill, dtype):
+    return G(np.full(shape, fill, dtype=dtype))
+
+
+def release():
+    """Drops the guarded mappings made so far (their arrays must not be used afterwards)."""
+    del _keep[:]
+    _guarded_ptrs.clear()
+
+
 def P(a):
     if a is None:
         return None
     assert a.flags["C_CONTIGUOUS"]
-    return a.ctypes.data
+    return G(a).ctypes.data   # inputs get their guarded copy here; outputs were made by _full
 
 
 def ok(rc):
@@ -75,7 +123,7 @@ def grouped_gemm(x16, w16, m_sizes, N, fp16=False, block_layout=False, variant=-
     ms = i32(m_sizes)
     G, (M, K) = len(ms), x16.shape
     ld = N * G if block_layout else N
-    y = np.full((M, ld), NAN16, dtype=np.uint16)
+    y = _full((M, ld), NAN16, dtype=np.uint16)
     L.moe_gg_set_variant(OP_BF16, variant)
     try:
         fn = L.moe_gg_grouped_gemm_f16 if fp16 else L.moe_gg_grouped_gemm_bf16
@@ -89,7 +137,7 @@ def grouped_gemm_fp8(xq, wq, x_scale, w_scale, mode, m_sizes, N, variant=-1):
     L = lib()
     ms = i32(m_sizes)
     G, (M, K) = len(ms), xq.shape
-    y = np.full((M, N), NAN16, dtype=np.uint16)
+    y = _full((M, N), NAN16, dtype=np.uint16)
     L.moe_gg_set_variant(OP_FP8, variant)
     try:
         ok(L.moe_gg_grouped_gemm_fp8(P(xq), P(wq), P(y), P(x_scale), P(w_scale), mode, P(ms), G, M, N, K, N, 0, None))
@@ -102,7 +150,7 @@ def grouped_gemm_swiglu(x16, w16, m_sizes, n, fp16=False):
     L = lib()
     ms = i32(m_sizes)
     G, (M, K) = len(ms), x16.shape
-    y = np.full((M, n), NAN16, dtype=np.uint16)
+    y = _full((M, n), NAN16, dtype=np.uint16)
     fn = L.moe_gg_grouped_gemm_swiglu_f16 if fp16 else L.moe_gg_grouped_gemm_swiglu_bf16
     ok(fn(P(x16), P(w16), P(y), P(ms), G, M, n, K, n, None))
     return y
@@ -112,14 +160,14 @@ def backward(go16, x16, w16, m_sizes, N, block_layout=False, static=False):
     L = lib()
     ms = i32(m_sizes)
     G, (M, K) = len(ms), x16.shape
-    gx = np.full((M, K), NAN16, dtype=np.uint16)
-    gw = np.full((G * N, K), NAN16, dtype=np.uint16)
+    gx = _full((M, K), NAN16, dtype=np.uint16)
+    gw = _full((G * N, K), NAN16, dtype=np.uint16)
     layout = 1 if block_layout else 0
     if static:
         ok(L.moe_gg_grouped_gemm_backward_bf16_static(P(go16), go16.shape[1], layout, P(x16), P(w16), P(ms), G, M, N, K, P(gx), P(gw), None))
     else:
         nbytes = L.moe_gg_grouped_gemm_backward_workspace(G, M, N, K, layout)
-        raw = np.zeros(nbytes + 256, dtype=np.uint8)
+        raw = _full(nbytes // 256 * 256 + 512, 0, np.uint8)   # ends at the guard page when guarded
         off = (-raw.ctypes.data) % 256
         ws = raw[off:off + nbytes]
         ok(L.moe_gg_grouped_gemm_backward_bf16(P(go16), go16.shape[1], layout, P(x16), P(w16), P(ms), G, M, N, K, P(gx), P(gw),
@@ -133,18 +181,18 @@ def w4a16(a16, qweight, scales16, qzeros, group_size=128, zero_offset=1, fp16=Fa
     dt = FP16 if fp16 else BF16
     if m_sizes is None:
         N = qweight.shape[1]
-        c = np.full((M, N), NAN16, dtype=np.uint16)
+        c = _full((M, N), NAN16, dtype=np.uint16)
         ok(L.moe_gg_w4a16_splitk(P(a16), P(qweight), P(scales16), P(qzeros), P(c), M, N, K, group_size, zero_offset, dt, None))
         return c
     ms = i32(m_sizes)
     G, N = len(ms), qweight.shape[2]
     if fp8out:
-        cq = np.full((M, N), 0x7F, dtype=np.uint8)
-        cs = np.full((M, N // 128), np.nan, dtype=np.float32)
+        cq = _full((M, N), 0x7F, dtype=np.uint8)
+        cs = _full((M, N // 128), np.nan, dtype=np.float32)
         ok(L.moe_gg_w4a16_grouped_fp8out(P(a16), P(qweight), P(scales16), P(qzeros), P(cq), P(cs), P(ms), G, M, N, K, group_size,
                                          zero_offset, dt, None))
         return cq, cs
-    c = np.full((M, N), NAN16, dtype=np.uint16)
+    c = _full((M, N), NAN16, dtype=np.uint16)
     ok(L.moe_gg_w4a16_grouped(P(a16), P(qweight), P(scales16), P(qzeros), P(c), P(ms), G, M, N, K, group_size, zero_offset, dt, None))
     return c
 
@@ -152,10 +200,10 @@ def w4a16(a16, qweight, scales16, qzeros, group_size=128, zero_offset=1, fp16=Fa
 def route_topk(logits, k):
     L = lib()
     T, E = logits.shape
-    ids = np.full((T, k), -7, dtype=np.int32)
-    perm = np.full(T * k, -7, dtype=np.int32)
-    ms = np.full(E, -7, dtype=np.int32)
-    off = np.full(E + 1, -7, dtype=np.int32)
+    ids = _full((T, k), -7, dtype=np.int32)
+    perm = _full(T * k, -7, dtype=np.int32)
+    ms = _full(E, -7, dtype=np.int32)
+    off = _full(E + 1, -7, dtype=np.int32)
     ok(L.moe_gg_route_topk(P(np.ascontiguousarray(logits, dtype=np.float32)), T, E, k, P(ids), P(perm), P(ms), P(off), None))
     return ids, perm, ms, off
 
@@ -164,9 +212,9 @@ def route_group(flat_ids, E):
     L = lib()
     flat = i32(flat_ids).ravel()
     n = flat.size
-    perm = np.full(n, -7, dtype=np.int32)
-    ms = np.full(E, -7, dtype=np.int32)
-    off = np.full(E + 1, -7, dtype=np.int32)
+    perm = _full(n, -7, dtype=np.int32)
+    ms = _full(E, -7, dtype=np.int32)
+    off = _full(E + 1, -7, dtype=np.int32)
     ok(L.moe_gg_route_group(P(flat), n, E, P(perm), P(ms), P(off), None))
     return perm, ms, off
 
@@ -174,9 +222,9 @@ def route_group(flat_ids, E):
 def align_block_size(perm, m_sizes, block_size):
     L = lib()
     E, n = len(m_sizes), len(perm)
-    sorted_ids = np.full(n + E * (block_size - 1), -7, dtype=np.int32)
-    expert_ids = np.full(n + E, -7, dtype=np.int32)
-    post = np.full(1, -7, dtype=np.int32)
+    sorted_ids = _full(n + E * (block_size - 1), -7, dtype=np.int32)
+    expert_ids = _full(n + E, -7, dtype=np.int32)
+    post = _full(1, -7, dtype=np.int32)
     ok(L.moe_gg_align_block_size(P(i32(perm)), P(i32(m_sizes)), E, n, block_size, P(sorted_ids), P(expert_ids), P(post), None))
     return sorted_ids, expert_ids, int(post[0])
 
@@ -185,7 +233,7 @@ def gather_rows(x, perm, k, n_valid=None):
     L = lib()
     x = np.ascontiguousarray(x)
     n = len(perm)
-    out = np.full((n,) + x.shape[1:], 0xAB, dtype=x.dtype) if x.dtype.kind in "ui" else np.full((n,) + x.shape[1:], np.nan, dtype=x.dtype)
+    out = _full((n,) + x.shape[1:], 0xAB, dtype=x.dtype) if x.dtype.kind in "ui" else _full((n,) + x.shape[1:], np.nan, dtype=x.dtype)
     nv = None if n_valid is None else np.array([n_valid], dtype=np.int32)
     ok(L.moe_gg_gather_rows(P(x), P(i32(perm)), k, P(out), n, x[0].nbytes, x.shape[0], P(nv), None))
     return out
@@ -194,8 +242,8 @@ def gather_rows(x, perm, k, n_valid=None):
 def fp8_groupwise_quant(x, bf16_in=False):
     L = lib()
     src = to_bf16(x) if bf16_in else np.ascontiguousarray(x, dtype=np.float32)
-    q = np.full(x.shape, 0x7F, dtype=np.uint8)
-    s = np.full(x.size // 128, np.nan, dtype=np.float32)
+    q = _full(x.shape, 0x7F, dtype=np.uint8)
+    s = _full(x.size // 128, np.nan, dtype=np.float32)
     ok(L.moe_gg_fp8_groupwise_quant(P(src), BF16 if bf16_in else FP32, P(q), P(s), x.size, None))
     return q, s.reshape(x.shape[:-1] + (x.shape[-1] // 128,))
 
@@ -204,8 +252,8 @@ def fp8_block128_quant(w, bf16_in=False):
     L = lib()
     rows, K = w.shape
     src = to_bf16(w) if bf16_in else np.ascontiguousarray(w, dtype=np.float32)
-    q = np.full(w.shape, 0x7F, dtype=np.uint8)
-    s = np.full((rows // 128, K // 128), np.nan, dtype=np.float32)
+    q = _full(w.shape, 0x7F, dtype=np.uint8)
+    s = _full((rows // 128, K // 128), np.nan, dtype=np.float32)
     ok(L.moe_gg_fp8_block128_quant(P(src), BF16 if bf16_in else FP32, P(q), P(s), rows, K, None))
     return q, s
 
@@ -213,7 +261,7 @@ def fp8_block128_quant(w, bf16_in=False):
 def silu_and_mul(x16, fp16=False):
     L = lib()
     rows, n2 = x16.shape
-    out = np.full((rows, n2 // 2), NAN16, dtype=np.uint16)
+    out = _full((rows, n2 // 2), NAN16, dtype=np.uint16)
     ok((L.moe_gg_silu_and_mul_f16 if fp16 else L.moe_gg_silu_and_mul)(P(x16), P(out), rows, n2 // 2, None))
     return out
 
@@ -221,7 +269,7 @@ def silu_and_mul(x16, fp16=False):
 def invert_perm(perm, n_valid=None):
     L = lib()
     n = len(perm)
-    inv = np.full(n, -7, dtype=np.int32)
+    inv = _full(n, -7, dtype=np.int32)
     nv = None if n_valid is None else np.array([n_valid], dtype=np.int32)
     ok(L.moe_gg_invert_perm(P(i32(perm)), P(inv), n, P(nv), None))
     return inv
@@ -230,7 +278,7 @@ def invert_perm(perm, n_valid=None):
 def combine_topk(y16, inv, weights, T, k, fp16=False, weights_16bit=False):
     L = lib()
     d = y16.shape[1]
-    out = np.full((T, d), NAN16, dtype=np.uint16)
+    out = _full((T, d), NAN16, dtype=np.uint16)
     wt = to16(weights, fp16) if weights_16bit else np.ascontiguousarray(weights, dtype=np.float32)
     wd = (FP16 if fp16 else BF16) if weights_16bit else FP32
     fn = L.moe_gg_combine_topk_f16 if fp16 else L.moe_gg_combine_topk

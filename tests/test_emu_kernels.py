@@ -89,10 +89,11 @@ def test_fp8_every_kernel_variant(mode, variant):
     rng = np.random.default_rng(10 * mode + variant + 3)
     sizes, N, K = [300, 0, 70, 30, 530], 256, 256
     G, M = len(sizes), sum(sizes)
-    xq = (rng.integers(0, 0x40, (M, K)) | (rng.integers(0, 2, (M, K)) << 7)).astype(np.uint8)
-    wq = (rng.integers(0, 0x40, (G * N, K)) | (rng.integers(0, 2, (G * N, K)) << 7)).astype(np.uint8)
-    xs = (2.0 ** rng.integers(-2, 3, M if mode == 0 else (M, K // 128))).astype(np.float32)
-    ws = (2.0 ** rng.integers(-2, 3, G * N if mode == 0 else (G * N // 128, K // 128))).astype(np.float32)
+    # codes of magnitude 0.5 ... 3.75 and scales of 1 or 2: every partial sum is exact in fp32, whatever the order
+    xq = ((0x30 + rng.integers(0, 0x18, (M, K))) | (rng.integers(0, 2, (M, K)) << 7)).astype(np.uint8)
+    wq = ((0x30 + rng.integers(0, 0x18, (G * N, K))) | (rng.integers(0, 2, (G * N, K)) << 7)).astype(np.uint8)
+    xs = (2.0 ** rng.integers(0, 2, M if mode == 0 else (M, K // 128))).astype(np.float32)
+    ws = (2.0 ** rng.integers(0, 2, G * N if mode == 0 else (G * N // 128, K // 128))).astype(np.float32)
     y = H.grouped_gemm_fp8(xq, wq, xs, ws, mode, sizes, N, variant)
     assert exact16(y, O.grouped_gemm_fp8(xq, wq, xs, ws, sizes, mode))
 
@@ -251,5 +252,21 @@ def test_pingpong_random_shapes_over_unit_counts_and_schedules():
         procs.append(subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_pingpong.py"), str(100 + i), "20"], env=env,
                                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT))
     for cfg, p in zip(FUZZ, procs):
+        log = p.communicate()[0].decode()
+        assert p.returncode == 0, (cfg, log[-2000:])
+
+
+GUARDED = [("end", "8", "late", "0"), ("start", "8", "early", "3"), ("end", "2", "late", "11"), ("start", "13", "late", "0")]
+
+
+def test_every_entry_point_on_random_shapes_with_tensors_against_guard_pages():
+    """Inputs, outputs and the workspace end (or begin) at an inaccessible page: a kernel that touches memory outside a
+    tensor, by one element or by one 16-byte load, ends the child process with a memory fault."""
+    procs = []
+    for i, (guard, cus, dma, seed) in enumerate(GUARDED):
+        env = dict(os.environ, EMU_GUARD=guard, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed, EMU_TRACE="1")
+        procs.append(subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_all.py"), str(200 + i), "40"], env=env,
+                                      stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT))
+    for cfg, p in zip(GUARDED, procs):
         log = p.communicate()[0].decode()
         assert p.returncode == 0, (cfg, log[-2000:])
