@@ -192,6 +192,12 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
+  // The two constants of the nibble unpack live in registers (the mask in a scalar, the exponent pattern in a vector
+  // one), hidden from constant folding: mask-and-or is then one v_and_or_b32, which takes no literal and one scalar
+  // operand; with literals it is an and and an or.
+  uint32_t nib_mask = 0x000F000Fu, magic = E::MAGIC;
+  asm volatile("" : "+s"(nib_mask));
+  asm volatile("" : "+v"(magic));
   const W4View v = w4_view(p);
   const int N = p.N, K = p.K, M = v.M;
   constexpr int CB = QOUT ? 2 : 1;                 // 64-column blocks per workgroup
@@ -260,7 +266,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
           for (int j = 0; j < 4; ++j) {
             u32x4_t af;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) af[e] = ((w4[j] >> (4 * e)) & 0x000F000Fu) | E::MAGIC;
+            for (int e = 0; e < 4; ++e) af[e] = ((w4[j] >> (4 * e)) & nib_mask) | magic;
 #pragma unroll
             for (int i = 0; i < MF; ++i) accg[i][j] = E::mfma(af, xb[i], accg[i][j]);
           }
@@ -323,6 +329,12 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
+  // The two constants of the nibble unpack live in registers (the mask in a scalar, the exponent pattern in a vector
+  // one), hidden from constant folding: mask-and-or is then one v_and_or_b32, which takes no literal and one scalar
+  // operand; with literals it is an and and an or.
+  uint32_t nib_mask = 0x000F000Fu, magic = E::MAGIC;
+  asm volatile("" : "+s"(nib_mask));
+  asm volatile("" : "+v"(magic));
   const W4View v = w4_view(p);
   const int N = p.N, K = p.K, M = v.M;
   constexpr int CB = QOUT ? 2 : 1;                      // 64-column blocks per workgroup
@@ -417,7 +429,7 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
             for (int j = 0; j < 4; ++j) {
               u32x4_t bf;
 #pragma unroll
-              for (int e2 = 0; e2 < 4; ++e2) bf[e2] = ((w4[j] >> (4 * e2)) & 0x000F000Fu) | E::MAGIC;
+              for (int e2 = 0; e2 < 4; ++e2) bf[e2] = ((w4[j] >> (4 * e2)) & nib_mask) | magic;
 #pragma unroll
               for (int i = 0; i < MF; ++i) accg[i][j] = E::mfma(xb[i], bf, accg[i][j]);
             }
