@@ -241,6 +241,47 @@ def test_argument_checks_reach_the_caller():
     assert L.moe_gg_grouped_gemm_fp8(H.P(buf), H.P(buf), H.P(buf), H.P(buf), H.P(buf), 1, H.P(ms), 1, 1, 128, 100, 128, 0, None) != 0
 
 
+GOLD = os.path.join(ROOT, "tests", "golden")
+
+
+def rel_fro(a, b):
+    a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def test_committed_golden_vectors():
+    """The fixtures of tests/golden with the bars of the GPU tests: config 1 (routing bit-exact, GEMM to 1e-2), the
+    tiny fp8 case in both scale modes and the tiny W4A16 case with both zero-point conventions (relative Frobenius
+    error <= 2e-2), the moe_align_block_size known answer."""
+    import json
+
+    z = np.load(os.path.join(GOLD, "cfg1.npz"))
+    ids, perm, ms, off = H.route_topk(z["logits"], 2)
+    assert (ids == z["ids"]).all() and (perm == z["perm"]).all() and (ms == z["m_sizes"]).all() and (off == z["offsets"]).all()
+    y = H.from_bf16(H.grouped_gemm(z["x_sorted_bf16_bits"], z["w_bf16_bits"], z["m_sizes"], 512))
+    np.testing.assert_allclose(y, z["y_bf16_inputs"], rtol=1e-2, atol=1e-2)
+
+    z = np.load(os.path.join(GOLD, "fp8_tiny.npz"))
+    m = z["m_sizes"].tolist()
+    tot = sum(m)
+    y = H.from_bf16(H.grouped_gemm_fp8(z["xq"], z["wq"], z["xs"], z["ws"], 1, m, 256))
+    assert rel_fro(y[:tot], z["y_block"][:tot]) <= 2e-2
+    y = H.from_bf16(H.grouped_gemm_fp8(z["xq_row"], z["wq_row"], z["xs_row"], z["ws_row"], 0, m, 256))
+    assert rel_fro(y[:tot], z["y_row"][:tot]) <= 2e-2
+
+    z = np.load(os.path.join(GOLD, "w4a16_tiny.npz"))
+    for zo in (0, 1):
+        for M in (1, 16):
+            c = H.from_bf16(H.w4a16(H.to_bf16(z["a"][:M]), z["qweight"], H.to_bf16(z["scales"]), z["qzeros"], 128, zo))
+            assert rel_fro(c, z[f"c_zo{zo}_m{M}"]) <= 2e-2
+
+    kat = json.load(open(os.path.join(GOLD, "moe_align_kat.json")))
+    flat = np.array(kat["topk_ids"], dtype=np.int32).ravel() - 1   # the docstring numbers experts from 1
+    perm, ms, off = H.route_group(flat, kat["num_experts"])
+    s, e, post = H.align_block_size(perm, ms, kat["block_size"])
+    assert post == 16 and s[:post].tolist() == kat["sorted_token_ids"] and e[:4].tolist() == [0, 1, 2, 3]
+
+
 FUZZ = [  # (compute units, load-landing model, wave order seed): few units = long tile sequences per workgroup
     ("1", "late", "0"), ("2", "early", "0"), ("3", "late", "5"), ("8", "early", "9"), ("16", "late", "0"), ("5", "late", "77")]
 
