@@ -311,3 +311,12 @@ def test_every_entry_point_on_random_shapes_with_tensors_against_guard_pages():
     for cfg, p in zip(GUARDED, procs):
         log = p.communicate()[0].decode()
         assert p.returncode == 0, (cfg, log[-2000:])
+
+
+def test_corrupt_m_sizes_are_clamped_by_every_kernel():
+    """Negative sizes, sums beyond M, a size of 2^30: every kernel that reads m_sizes (all GEMM variants, fp8, SwiGLU,
+    backward, W4A16 grouped) computes the rows of the clamped sizes, leaves the other rows alone and, with every tensor
+    against a guard page, touches nothing outside them."""
+    env = dict(os.environ, EMU_GUARD="end", EMU_TRACE="1")
+    p = subprocess.run([sys.executable, os.path.join(EMU, "corrupt_sizes.py")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT)
+    assert p.returncode == 0, p.stdout.decode()[-2000:]
