@@ -1,6 +1,6 @@
 """Benchmark of the MoE grouped-GEMM hot path on one MI355X.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu-baseline] [--moe-sweep]
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu-baseline] [--no-moe-sweep]
 
 A step is one pass of the hot path over one batch of synthetic, HBM-resident input. The headline workload is the
 configuration the metric is quoted on: Mixtral 8x7B w1 grouped GEMM, bf16, T=4096 tokens top-2 (8192 expert-sorted
@@ -476,7 +476,7 @@ def wl_moe_sweep(torch, A, dev, lib, stream, cpu):
 
 
 SECONDARY = (wl_decode, wl_w4a16, wl_w4a16_grouped, wl_fp8_cfg5, wl_moe_layer, wl_backward)
-# Run only on request (--moe-sweep).
+# Context entries (left out with --no-moe-sweep).
 OPTIONAL = (wl_moe_sweep,)
 
 
@@ -500,8 +500,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
-    ap.add_argument("--moe-sweep", action="store_true",
-                    help="also time fused_moe over m = 1 ... 512 (the shape of the reference's published sweep; context only)")
+    ap.add_argument("--no-moe-sweep", action="store_true",
+                    help="skip the fused_moe sweep over m = 1 ... 512 (the shape of the reference's published sweep; context only)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, so that a rocprofv3 --pmc run of this command sees a kernel of known traffic")
     args = ap.parse_args()
@@ -602,7 +602,7 @@ def main():
         except Exception as exc:
             out["cpu_baseline"] = {"error": f"{type(exc).__name__}: {exc}"}
     if not args.no_secondary:
-        out["secondary"] = secondary_workloads(torch, A, dev, cpu=not args.no_cpu_baseline, optional=args.moe_sweep)
+        out["secondary"] = secondary_workloads(torch, A, dev, cpu=not args.no_cpu_baseline, optional=not args.no_moe_sweep)
     print(json.dumps(out))
 
 
