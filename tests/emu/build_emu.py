@@ -71,7 +71,7 @@ def _asm_rule(template, outs, ins, where):
     if m:
         return "emu::wait_vm(%s)" % (ins[0] if m.group(1) == "%0" else m.group(1))
     if re.fullmatch(r"\s*s_waitcnt lgkmcnt\(0\)\s*", t):
-        return "((void)0)"  # LDS reads are synchronous here
+        return "emu::wait_lds()"
     if re.fullmatch(r"\s*v_mad_u32_u24 %0, %1, %2, %3\s*", t):
         assert len(outs) == 1 and len(ins) == 3, where
         return "%s = ((%s) & 0xFFFFFFu) * ((%s) & 0xFFFFFFu) + (%s)" % (outs[0], ins[0], ins[1], ins[2])

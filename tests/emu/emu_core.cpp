@@ -350,7 +350,19 @@ void dma(int bytes, const void* sbase, uint32_t voff, uint32_t lds_addr) {
   if (g_dma_early) memcpy(q.dst, q.src, bytes);
   else f->dmaq.push_back(q);
 }
-void wait_vm(int n) { drain(*g_cur, (size_t)n); }
+// s_waitcnt is a wave-wide instruction: when a lane passes it, every lane of the wave has issued the loads before it
+// and (all but the newest n of) them have landed, for all lanes.
+__attribute__((noinline)) void wait_vm(int n) {
+  const char* site = (const char*)__builtin_return_address(0);
+  wave_sync(site);
+  drain(*g_cur, (size_t)n);
+  wave_sync(site + 1);
+}
+// s_waitcnt lgkmcnt(0): the wave's LDS accesses so far are complete, for all lanes.
+__attribute__((noinline)) void wait_lds() {
+  const char* site = (const char*)__builtin_return_address(0);
+  wave_sync(site);
+}
 
 // ---- matrix instructions: lane l holds row / column l % 16 and the k chunk l / 16 of its operand; of the result,
 // rows 4 (l / 16) .. + 3 of column l % 16 (A = first operand: rows; B = second: columns).

@@ -57,6 +57,7 @@ void exchange_done(const void* site = nullptr);
 int lane();
 void dma(int bytes, const void* sbase, uint32_t voff, uint32_t lds_addr);
 void wait_vm(int n);
+void wait_lds();
 char* lds_ptr(uint32_t addr, int bytes);
 void fail(const char* what);
 
