@@ -168,5 +168,40 @@ def build(force=False, jobs=8):
     return lib
 
 
+def build_race_check(force=False, jobs=8):
+    """tests/emu/_build/tsan/race_check: race_check.cpp + the kernels under ThreadSanitizer + emu_core.cpp with EMU_TSAN
+    (itself not instrumented: its tables are shared by all fibers on purpose)."""
+    out = os.path.join(OUT, "tsan")
+    exe = os.path.join(out, "race_check")
+    if not force and not stale(exe) and all(os.path.getmtime(exe) > os.path.getmtime(os.path.join(HERE, f))
+                                            for f in ("race_check.cpp", "race_selftest.cpp")):
+        return exe
+    build(force=False, jobs=jobs)   # leaves the translated sources in OUT
+    os.makedirs(out, exist_ok=True)
+    tsan = ["-fsanitize=thread", "-mllvm", "-tsan-instrument-func-entry-exit=0"]
+    units = [(os.path.join(OUT, f.replace(".hip", ".emu.cpp")), tsan) for f in sources()]
+    units.append((os.path.join(HERE, "race_selftest.cpp"), tsan))
+    units.append((os.path.join(HERE, "emu_core.cpp"), ["-DEMU_TSAN"]))
+    units.append((os.path.join(HERE, "race_check.cpp"), []))
+    objs, running, pending = [], [], list(units)
+    while pending or running:
+        while pending and len(running) < jobs:
+            src, extra = pending.pop(0)
+            obj = os.path.join(out, os.path.basename(src).rsplit(".", 1)[0] + ".o")
+            objs.append(obj)
+            running.append((src, subprocess.Popen([CXX] + FLAGS + extra + ["-c", src, "-o", obj], stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+        src, p = running.pop(0)
+        log = p.communicate()[0].decode()
+        if p.returncode:
+            for _, q in running:
+                q.kill()
+            raise SystemExit("build_emu: %s failed:\n%s" % (src, log[-6000:]))
+    subprocess.run([CXX, "-fsanitize=thread", "-o", exe] + objs + ["-ldl", "-lpthread"], check=True)
+    return exe
+
+
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv))
+    if "--race-check" in sys.argv:
+        print(build_race_check(force="--force" in sys.argv))
+    else:
+        print(build(force="--force" in sys.argv))

@@ -22,6 +22,24 @@
 
 dim3 threadIdx, blockIdx, blockDim, gridDim;
 
+// EMU_TSAN: the kernels are compiled with ThreadSanitizer (this file is not) and every wave is one of its fibers, so
+// that it reports accesses of two waves of a workgroup to the same bytes (LDS or global memory) that no barrier
+// orders, whatever the order they happen to run in here. Lanes of one wave share a fiber: within a wave the
+// instruction order is the order. Workgroups and launches are ordered one after the other.
+#ifdef EMU_TSAN
+extern "C" {
+void* __tsan_get_current_fiber(void);
+void* __tsan_create_fiber(unsigned flags);
+void __tsan_destroy_fiber(void* fiber);
+void __tsan_switch_to_fiber(void* fiber, unsigned flags);
+void __tsan_acquire(void* addr);
+void __tsan_release(void* addr);
+}
+#define TSAN(x) x
+#else
+#define TSAN(x)
+#endif
+
 extern "C" char __start_emu_lds[];
 extern "C" char __stop_emu_lds[];
 
@@ -87,7 +105,21 @@ bool g_dma_early = false;
 unsigned g_seed = 0;
 uint64_t g_nonuniform = 0;
 
-void yield() { emu_switch(&g_cur->ctx, &g_sched); }
+#ifdef EMU_TSAN
+void* g_tsan_main = nullptr;
+void* g_tsan_wave[MAX_THREADS / 64];
+// Sync objects: one per barrier generation (mod 64), launch start, workgroup end. The sanitizer keys them by address
+// in 8-byte cells, so each gets a cache line of its own.
+struct alignas(64) SyncCell { char c[64]; };
+SyncCell g_tsan_bar_cells[64], g_tsan_launch_cell, g_tsan_done_cell;
+#define g_tsan_launch g_tsan_launch_cell.c[0]
+#define g_tsan_done g_tsan_done_cell.c[0]
+#endif
+
+void yield() {
+  TSAN(__tsan_switch_to_fiber(g_tsan_main, 1));  // 1 = no synchronisation implied by the switch
+  emu_switch(&g_cur->ctx, &g_sched);
+}
 
 uint64_t g_divergent = 0;
 // Lanes of a wave that wait at the same place are released together once no lane of the wave can still join them:
@@ -128,8 +160,10 @@ void drain(Fiber& f, size_t keep) {
 
 void fiber_main() {
   Fiber* f = g_cur;
+  TSAN(__tsan_acquire(&g_tsan_launch));
   (*g_body)();
   drain(*f, 0);
+  TSAN(__tsan_release(&g_tsan_done));
   f->state = DONE;
   Wave& w = g_w[f->tid >> 6];
   --w.alive;
@@ -196,6 +230,11 @@ void run_workgroup(unsigned order_seed) {
   }
   g_alive = nt;
   g_bar_arrived = 0;
+#ifdef EMU_TSAN
+  // A workgroup's fibers start knowing everything the main fiber knows, which includes the workgroups before it
+  // (LDS and the lanes' stacks are reused from one workgroup to the next): the check is for waves of one workgroup.
+  for (int w = 0; w < (nt + 63) / 64; ++w) g_tsan_wave[w] = __tsan_create_fiber(0);
+#endif
   while (g_alive > 0) {
     bool progress = false;
     for (int k = 0; k < nt; ++k) {
@@ -204,6 +243,7 @@ void run_workgroup(unsigned order_seed) {
       progress = true;
       g_cur = &f;
       threadIdx = dim3(f.tid % blockDim.x, (f.tid / blockDim.x) % blockDim.y, f.tid / (blockDim.x * blockDim.y));
+      TSAN(__tsan_switch_to_fiber(g_tsan_wave[f.tid >> 6], 1));
       emu_switch(&g_sched, &f.ctx);
     }
     if (progress) continue;
@@ -213,6 +253,10 @@ void run_workgroup(unsigned order_seed) {
       if (g_w[w].waiting > 0) { try_release(g_w[w], true); released = true; }
     if (!released) fail("deadlock: every thread of the workgroup waits at a barrier that cannot complete");
   }
+#ifdef EMU_TSAN
+  __tsan_acquire(&g_tsan_done);
+  for (int w = 0; w < (nt + 63) / 64; ++w) __tsan_destroy_fiber(g_tsan_wave[w]);
+#endif
 }
 
 }  // namespace
@@ -266,6 +310,8 @@ void launch(dim3 grid, dim3 block, size_t dyn, const std::function<void()>& body
   g_body = &body;
   blockDim = block;
   gridDim = grid;
+  TSAN(g_tsan_main = __tsan_get_current_fiber());
+  TSAN(__tsan_release(&g_tsan_launch));
   unsigned wg = 0;
   for (unsigned z = 0; z < grid.z; ++z)
     for (unsigned y = 0; y < grid.y; ++y)
@@ -280,11 +326,17 @@ void* dyn_lds() { return g_dyn_lds; }
 
 void syncthreads() {
   Fiber* f = g_cur;
-  if (++g_bar_arrived == g_alive) { release_barrier(); return; }
-  f->wait_gen = g_bar_gen;
-  f->state = BAR_WAIT;
-  while (g_bar_gen == f->wait_gen) yield();
-  f->state = READY;
+  TSAN(char* sync = &g_tsan_bar_cells[g_bar_gen & 63].c[0]);
+  TSAN(__tsan_release(sync));
+  if (++g_bar_arrived == g_alive) {
+    release_barrier();
+  } else {
+    f->wait_gen = g_bar_gen;
+    f->state = BAR_WAIT;
+    while (g_bar_gen == f->wait_gen) yield();
+    f->state = READY;
+  }
+  TSAN(__tsan_acquire(sync));
 }
 
 int lane() { return g_cur->tid & 63; }

@@ -96,7 +96,7 @@ template <class T> inline T __shfl(T v, int src, int = 64) { return emu::get_lan
 inline unsigned long long __ballot(int pred) { return emu::ballot(pred); }
 inline int __popcll(unsigned long long v) { return __builtin_popcountll(v); }
 inline int __ffsll(long long v) { return __builtin_ffsll(v); }
-template <class T> inline T atomicAdd(T* p, T v) { T o = *p; *p = o + v; return o; }
+template <class T> inline T atomicAdd(T* p, T v) { return __atomic_fetch_add(p, v, __ATOMIC_RELAXED); }
 
 // Fast-math exponential of the device library: the host's expf (results differ in the last bits).
 #define __expf(x) expf(x)

@@ -320,3 +320,21 @@ def test_corrupt_m_sizes_are_clamped_by_every_kernel():
     env = dict(os.environ, EMU_GUARD="end", EMU_TRACE="1")
     p = subprocess.run([sys.executable, os.path.join(EMU, "corrupt_sizes.py")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT)
     assert p.returncode == 0, p.stdout.decode()[-2000:]
+
+
+def test_no_data_race_between_the_waves_of_a_workgroup():
+    """The kernels compiled under ThreadSanitizer with every wave as one of its fibers (tests/emu/race_check.cpp): every
+    entry point runs without a report, i.e. each pair of accesses by two waves to the same LDS or global bytes is
+    ordered by a barrier - also where the emulation happens to run them in a harmless order. Two control kernels
+    show that the check sees a missing barrier, after ordinary stores and after a global->LDS load."""
+    exe = build_emu.build_race_check()
+    for kernel in ("0", "1"):
+        clean = subprocess.run([exe, "selftest", kernel, "1"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+        racy = subprocess.run([exe, "selftest", kernel, "0"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+        assert clean.returncode == 0 and b"data race" not in clean.stdout, clean.stdout.decode()[-1500:]
+        assert racy.returncode == 66 and b"data race" in racy.stdout, racy.stdout.decode()[-1500:]
+    procs = [subprocess.Popen([exe], env=dict(os.environ, EMU_CUS=cus, EMU_SEED=seed), stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+             for cus, seed in (("8", "0"), ("2", "7"))]
+    for p in procs:
+        log = p.communicate()[0].decode()
+        assert p.returncode == 0 and "data race" not in log and "calls that returned an error: 0" in log, log[-3000:]
