@@ -56,13 +56,47 @@ static void check(int rc, const char* what) {
 
 extern "C" int race_selftest(int kernel, int barrier);
 
-// race_check                     all entry points (exit status 0 unless the sanitizer reported something: then 66)
-// race_check selftest K B        control kernel K (0: stores, 1: global->LDS load), B = 1 with / 0 without the barrier
+// One grouped launch of the 256 x 256 ping-pong kernels (or the backward pass) on the given expert sizes.
+static int one_shape(const char* op, int N, int K, int G, char** sizes) {
+  Buf<int32_t> ms(G);
+  int M = 0;
+  for (int g = 0; g < G; ++g) M += (ms.v[g] = std::atoi(sizes[g]));
+  Buf<uint16_t> y((size_t)M * N + 64);
+  if (!std::strcmp(op, "fp8row") || !std::strcmp(op, "fp8block")) {
+    const int mode = !std::strcmp(op, "fp8block");
+    auto xq = fp8_codes((size_t)M * K), wq = fp8_codes((size_t)G * N * K);
+    auto xs = ones((size_t)M * (K / 128) + 1), wsc = ones((size_t)G * N);
+    moe_gg_set_variant(MOE_GG_OP_GG_FP8, MOE_GG_FP8_PINGPONG);
+    check(moe_gg_grouped_gemm_fp8(xq.p(), wq.p(), y.p(), xs.p(), wsc.p(), mode, ms.p(), G, M, N, K, N, MOE_GG_OUT_MN, nullptr), op);
+  } else if (!std::strcmp(op, "bwd")) {
+    auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * N * K), go = bf16_small((size_t)M * N);
+    Buf<uint16_t> gx((size_t)M * K), gw((size_t)G * N * K);
+    const size_t wsb = moe_gg_grouped_gemm_backward_workspace(G, M, N, K, 0);
+    Buf<uint8_t> ws(wsb + 512);
+    uint8_t* wsp = ws.p() + ((256 - ((uintptr_t)ws.p() & 255)) & 255);
+    check(moe_gg_grouped_gemm_backward_bf16(go.p(), N, 0, x.p(), w.p(), ms.p(), G, M, N, K, gx.p(), gw.p(), wsp, wsb, nullptr), op);
+  } else if (!std::strcmp(op, "swiglu")) {
+    auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * 2 * N * K);
+    check(moe_gg_grouped_gemm_swiglu_bf16(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, nullptr), op);
+  } else {
+    const bool f16 = !std::strcmp(op, "f16");
+    auto x = f16 ? f16_small((size_t)M * K) : bf16_small((size_t)M * K);
+    auto w = f16 ? f16_small((size_t)G * N * K) : bf16_small((size_t)G * N * K);
+    moe_gg_set_variant(MOE_GG_OP_GG_BF16, MOE_GG_GG_PINGPONG_256);
+    check((f16 ? moe_gg_grouped_gemm_f16 : moe_gg_grouped_gemm_bf16)(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, MOE_GG_OUT_MN, nullptr), op);
+  }
+  return failures ? 1 : 0;
+}
+
+// race_check                       all entry points (exit status 0 unless the sanitizer reported something: then 66)
+// race_check selftest K B          control kernel K (0: stores, 1: global->LDS load), B = 1 with / 0 without the barrier
+// race_check shape OP N K m1 m2 .. one launch; OP = bf16 | f16 | swiglu | fp8row | fp8block | bwd
 int main(int argc, char** argv) {
   if (argc == 4 && !std::strcmp(argv[1], "selftest")) {
     std::printf("sum %d\n", race_selftest(std::atoi(argv[2]), std::atoi(argv[3])));
     return 0;
   }
+  if (argc >= 6 && !std::strcmp(argv[1], "shape")) return one_shape(argv[2], std::atoi(argv[3]), std::atoi(argv[4]), argc - 5, argv + 5);
   {
     const int sizes[] = {300, 0, 70, 530};
     const int G = 4, M = 900, N = 512, K = 256;
