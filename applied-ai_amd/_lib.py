@@ -69,6 +69,9 @@ SIGNATURES = {
         _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_i64, _c_void_p]),
     "moe_gg_grouped_gemm_swiglu_f16": (
         _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_i64, _c_void_p]),
+    "moe_gg_grouped_gemm_swiglu_gather": (
+        _c_int, [_c_void_p, _c_i64, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_i64, _c_int, _c_int, _c_i64,
+                 _c_int, _c_void_p]),
     "moe_gg_silu_and_mul": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "moe_gg_silu_and_mul_f16": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "moe_gg_invert_perm": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_void_p, _c_void_p]),

@@ -336,12 +336,20 @@ int moe_gg_gather_rows(const void* x, const int32_t* perm, int k, void* out, int
   return (int)gather_rows_launch(x, perm, k, out, (int)n, row_bytes, src_rows, n_valid, (hipStream_t)stream);
 }
 
+// perm == nullptr: x is [M, K], the rows in expert-sorted order; else x is the token matrix [T, K] and sorted row i is
+// its row perm[i] / k.
 static int grouped_gemm_swiglu_16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M, int n,
-                                  int K, int64_t ldy, bool fp16, void* stream) {
+                                  int K, int64_t ldy, bool fp16, void* stream, const int32_t* perm = nullptr, int k = 1,
+                                  int64_t T = 0) {
   if (G < 0 || M < 0 || n < 0 || K < 0) return MOE_GG_EINVAL;
   if (ldy < n) return MOE_GG_ESHAPE;
   if (G == 0 || M == 0 || n == 0) return MOE_GG_OK;
   if (!x || !w || !y || !m_sizes) return MOE_GG_EINVAL;
+  if (perm) {
+    if (k <= 0 || T <= 0) return MOE_GG_EINVAL;
+    if (T * (int64_t)K * 2 >= INT32_MAX) return MOE_GG_EUNSUPPORTED;  // the loads add 32-bit byte offsets to the base
+    if (!aligned(perm, 4)) return MOE_GG_EALIGN;
+  }
   if (G > MOE_GG_MAX_GROUPS_ABI || M > INT32_MAX || ldy > INT32_MAX) return MOE_GG_EUNSUPPORTED;
   if (K == 0 || K % 64 != 0 || n % 4 != 0 || (int64_t)2 * n * K >= INT32_MAX || K >= PINGPONG_MAX_ROW_BYTES / 2 ||
       2 * (int64_t)n >= PINGPONG_MAX_ROW_BYTES)
@@ -360,6 +368,9 @@ static int grouped_gemm_swiglu_16(const void* x, const void* w, void* y, const i
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
   if (!moe_gg_two_list_fits(M, G, 256, (n + 127) / 128, num_wg)) return MOE_GG_EUNSUPPORTED;
   p.fp16 = fp16 ? 1 : 0;
+  p.gather_perm = perm;
+  p.gather_k = k;
+  p.gather_rows = (int)T;
   return (int)gg_bf16_pingpong_swiglu_launch(p, num_wg, (hipStream_t)stream);
 }
 
@@ -371,6 +382,15 @@ int moe_gg_grouped_gemm_swiglu_bf16(const void* x, const void* w, void* y, const
 int moe_gg_grouped_gemm_swiglu_f16(const void* x, const void* w, void* y, const int32_t* m_sizes, int G, int64_t M,
                                    int n, int K, int64_t ldy, void* stream) {
   return grouped_gemm_swiglu_16(x, w, y, m_sizes, G, M, n, K, ldy, true, stream);
+}
+
+int moe_gg_grouped_gemm_swiglu_gather(const void* tokens, int64_t T, const int32_t* perm, int k, const void* w, void* y,
+                                      const int32_t* m_sizes, int G, int64_t M, int n, int K, int64_t ldy, int dtype,
+                                      void* stream) {
+  if (dtype != MOE_GG_DTYPE_BF16 && dtype != MOE_GG_DTYPE_FP16) return MOE_GG_EINVAL;
+  if (T < 0 || k <= 0) return MOE_GG_EINVAL;
+  if (M > 0 && G > 0 && n > 0 && (!perm || T == 0)) return MOE_GG_EINVAL;
+  return grouped_gemm_swiglu_16(tokens, w, y, m_sizes, G, M, n, K, ldy, dtype == MOE_GG_DTYPE_FP16, stream, perm, k, T);
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }

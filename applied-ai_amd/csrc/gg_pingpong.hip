@@ -87,8 +87,16 @@ constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x
 // tensors), and group 0 overwrites them with zeros in the dY slab once it has landed, so they add nothing.
 // OP_F16, OP_F16_SWIGLU: OP_BF16 / OP_BF16_SWIGLU on IEEE half data (the same kernels with the f16 MFMA and half
 // conversions in the epilogue).
+// OP_BF16_SWIGLU_GATHER, OP_F16_SWIGLU_GATHER: the SWIGLU kernels reading their activation rows through the layer's
+// row permutation: row i of the expert-sorted order is row perm[i] / k of the token matrix p.x (the gather of
+// fused_moe folded into the slab loads; the reference's kernel reads A through sorted_token_ids in the same way,
+// kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:75-80). Per tile a loading lane keeps the byte
+// offsets of its eight rows; a K step's loads add only the chunk offset.
 constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4, OP_BF16_NT = 5,
-              OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7, OP_F16_SWIGLU = 8;
+              OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7, OP_F16_SWIGLU = 8, OP_BF16_SWIGLU_GATHER = 9, OP_F16_SWIGLU_GATHER = 10;
+constexpr bool op_gather(int op) { return op == OP_BF16_SWIGLU_GATHER || op == OP_F16_SWIGLU_GATHER; }
+constexpr bool op_swiglu(int op) { return op == OP_BF16_SWIGLU || op == OP_F16_SWIGLU || op_gather(op); }
+constexpr bool op_f16(int op) { return op == OP_F16 || op == OP_F16_SWIGLU || op == OP_F16_SWIGLU_GATHER; }
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
 // 64 lanes x 16 B (or 4 B) from global memory straight into LDS: lane l's bytes land at lds_addr + 16 l
@@ -158,10 +166,11 @@ struct Cursor {
 template <int GRP, int OP>
 DEVINL void run_group(const GgParams& p, const Shared& sh) {
   constexpr bool FP8 = OP == OP_FP8_ROW || OP == OP_FP8_BLOCK;
-  constexpr bool F16 = OP == OP_F16 || OP == OP_F16_SWIGLU;
+  constexpr bool F16 = op_f16(OP);
   constexpr bool BLOCK = OP == OP_FP8_BLOCK;
   constexpr bool WGRAD = OP == OP_BF16_WGRAD;
-  constexpr bool SWIGLU = OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU;
+  constexpr bool SWIGLU = op_swiglu(OP);
+  constexpr bool GATHER = op_gather(OP);
   constexpr bool WG2 = OP == OP_BF16_WGRAD_DIRECT;
   constexpr bool WNT = OP == OP_BF16_NT || WG2;  // weight slab: 64 reduction rows by 256 columns (transposing reads)
   constexpr int TILE_COLS = SWIGLU ? BN / 2 : BN;  // output columns of a tile
@@ -219,7 +228,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       r.t.row0 = uni(sh.row_off[g]);
       r.t.rows = uni(sh.row_off[g + 1]) - r.t.row0;
       r.KT = KT_fwd;
-      r.xoff = (int64_t)(r.t.row0 + r.m0) * XPITCH + (OP == OP_BF16_NT ? (int64_t)g * p.x_col_block * 2 : 0);
+      r.xoff = GATHER ? 0 : (int64_t)(r.t.row0 + r.m0) * XPITCH + (OP == OP_BF16_NT ? (int64_t)g * p.x_col_block * 2 : 0);
       if (WNT) r.woff = ((int64_t)g * p.K * N + r.n0) * 2;  // w[g][0][n0]
       else r.woff = ((int64_t)g * N + r.n0) * KROW;
     }
@@ -243,6 +252,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   bf16_t* __restrict__ yp = (bf16_t*)p.y;
 
   Cursor c;
+  uint32_t gather_off[8];  // GATHER, group 0: byte offset in p.x of the lane's row of its block idx * 4 + gw, idx = 0 .. 7
   auto cursor_tile = [&](int round) {
     c.round = round;
     if (round >= sh.n_my) return;  // past the last tile: keep re-loading the last tile (never read)
@@ -255,6 +265,17 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
     c.w_last = max(min(NCOLS - n0, tr.nc), 1) - 1;  // SWIGLU: last valid output column of the tile
     c.xg = uni_ptr(xp + tr.xoff);
     c.wg = uni_ptr(wp + tr.woff);
+    if (GATHER && GRP == 0) {
+      // The sorted rows t.row0 + m0 .. of this tile, looked up once per tile; rows beyond the tile's last one repeat
+      // it, as the plain kernel re-reads it. An entry that names no slot of the token matrix (a caller's corrupt
+      // perm) is folded into range, so that the loads stay inside p.x whatever perm holds.
+      const int32_t* pp = p.gather_perm + t.row0 + m0;
+#pragma unroll
+      for (int idx = 0; idx < 8; ++idx) {
+        const uint32_t slot = (uint32_t)pp[min((idx * 4 + gw) * 8 + d_r, c.x_last)];
+        gather_off[idx] = min(slot / (uint32_t)p.gather_k, (uint32_t)p.gather_rows - 1u) * XPITCH;
+      }
+    }
     if (BLOCK) {
       c.xsg = uni_ptr((const char*)(p.x_scale + (int64_t)(t.row0 + m0) * KT_fwd));
       c.wsg = uni_ptr((const char*)(p.w_scale + (((int64_t)t.g * N + n0) / 128) * KT_fwd));
@@ -284,7 +305,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
       return;
     }
     if (b * 8 > c.x_last) return;  // block entirely below the tile's last row: its fragments are never used
-    const uint32_t off = mad24((uint32_t)min(b * 8 + d_r, c.x_last), XPITCH, d_c16);
+    const uint32_t off = GATHER ? gather_off[b >> 2] + d_c16 : mad24((uint32_t)min(b * 8 + d_r, c.x_last), XPITCH, d_c16);
     dma16(c.xg + c.kt * 128, off, lds_base + (c.step & 1) * STAGE + b * 1024);
   };
   // Weight rows: of the cursor slab, or (prev) of the slab before it, whose state group 1 keeps in wp_*.
@@ -677,7 +698,7 @@ DEVINL void pingpong_body(const GgParams& p) {
     build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
     total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
   } else {
-    const int ntn = (OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU) ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
+    const int ntn = op_swiglu(OP) ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
     const int skip = p.skip_rows;
     build_row_offsets(p.m_sizes, p.G, p.M, row_off);
     if ((OP == OP_BF16 || OP == OP_F16) && p.tails_apart) {
@@ -717,7 +738,7 @@ DEVINL void pingpong_body(const GgParams& p) {
   const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
   for (int i = threadIdx.x; i < n_my; i += NT) {
     int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
-    constexpr int TC = (OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU) ? BN / 2 : BN;  // output columns of a tile
+    constexpr int TC = op_swiglu(OP) ? BN / 2 : BN;  // output columns of a tile
     int g, m0, h, n0, nc = TC;  // group, first row inside the group, rows, first column, columns
     if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
       // Tiles of an expert in bands of four column tiles, column tile fastest inside a band: the 32 tiles an XCD
@@ -755,6 +776,8 @@ __global__ __launch_bounds__(NT) void gg_f16_pingpong(GgParams p) { pingpong_bod
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
 __global__ __launch_bounds__(NT) void gg_f16_pingpong_swiglu(GgParams p) { pingpong_body<OP_F16_SWIGLU>(p); }
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu_gather(GgParams p) { pingpong_body<OP_BF16_SWIGLU_GATHER>(p); }
+__global__ __launch_bounds__(NT) void gg_f16_pingpong_swiglu_gather(GgParams p) { pingpong_body<OP_F16_SWIGLU_GATHER>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_nt(GgParams p) { pingpong_body<OP_BF16_NT>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad_direct(GgParams p) { pingpong_body<OP_BF16_WGRAD_DIRECT>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise(GgParams p) { pingpong_body<OP_FP8_ROW>(p); }
@@ -774,7 +797,10 @@ hipError_t gg_bf16_pingpong_wgrad_launch(const GgParams& p, int num_wg, hipStrea
 }
 
 hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
+  if (p.gather_perm) {
+    if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong_swiglu_gather, dim3(num_wg), dim3(NT), 0, stream, p);
+    else hipLaunchKernelGGL(gg_bf16_pingpong_swiglu_gather, dim3(num_wg), dim3(NT), 0, stream, p);
+  } else if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
   else hipLaunchKernelGGL(gg_bf16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }

@@ -25,6 +25,11 @@ struct GgParams {
   // then computed by the small-M kernel whenever moe_gg_tails_apart() says so (both kernels evaluate it).
   int tails_apart;
   int fp16;  // forward kernels: x, w and y are IEEE half instead of bf16 (same layouts)
+  // gg_bf16_pingpong_swiglu with a row gather: when gather_perm is set, x is the token matrix [gather_rows, K] and row
+  // i of the expert-sorted order (M of them) is its row gather_perm[i] / gather_k.
+  const int32_t* gather_perm;
+  int gather_k;
+  int gather_rows;
 };
 
 // block_m in {256, 128, 64}; the matching tile width is gg_bf16_tiled_block_n(block_m).

@@ -17,7 +17,8 @@ Everything runs in the HIP kernels behind include/moe_gg.h; torch only provides 
 import torch
 
 from . import _lib
-from .ops import _require_cuda, _stream_ptr, grouped_gemm, grouped_gemm_swiglu, matmul_split_k_grouped
+from .ops import (_require_cuda, _stream_ptr, grouped_gemm, grouped_gemm_swiglu, grouped_gemm_swiglu_gathered,
+                  matmul_split_k_grouped)
 from .routing import gather_sorted, route_group
 
 # fused_moe folds SiLU-and-mul into the first GEMM from this many expert-sorted rows on (the fused kernel is the
@@ -107,11 +108,13 @@ def invoke_fused_moe_kernel(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, t
 
 
 def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, topk_weights: torch.Tensor,
-              topk_ids: torch.Tensor, inplace: bool = False) -> torch.Tensor:
+              topk_ids: torch.Tensor, inplace: bool = False, fuse_gather: bool = False) -> torch.Tensor:
     """Mixture-of-experts layer with top-k gating; arguments as the reference's fused_moe
     (v0_moe_fused.py:222-227): hidden_states [M, K], w1 [E, 2n, K], w2 [E, d, n], topk_weights / topk_ids [M, k].
     bf16 or fp16 (:216). With inplace=True the result is written into hidden_states (d must equal K), as the
-    reference does (:291-294)."""
+    reference does (:291-294). fuse_gather=True lets the first GEMM read the token rows through the permutation
+    (as the reference's kernel does through sorted_token_ids, :75-80) instead of from a gathered copy, where the
+    fused first GEMM runs at all; the result has the same bits."""
     assert hidden_states.shape[1] == w1.shape[2], "Incompatible dimensions"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
     assert w1.is_contiguous(), "Expert weights1 must be contiguous"
@@ -126,13 +129,18 @@ def fused_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, t
     tw = topk_weights if topk_weights.dtype in (torch.float32, hidden_states.dtype) else topk_weights.float()
 
     perm, m_sizes, offsets = route_group(ids, E)
-    xs = gather_sorted(hidden_states, perm, k, offsets)
-    swiglu_tiles = (xs.shape[0] // 256 + E) * ((two_n // 2 + 127) // 128)   # bound of the fused kernel's tile table
-    if (xs.shape[0] >= FUSED_SWIGLU_MIN_ROWS and K % 64 == 0 and two_n % 8 == 0 and two_n * K < 2 ** 31
-            and swiglu_tiles <= 1023 * 256):
-        h2 = grouped_gemm_swiglu(xs, w1.view(E * two_n, K), m_sizes)
+    rows = perm.shape[0]
+    swiglu_tiles = (rows // 256 + E) * ((two_n // 2 + 127) // 128)   # bound of the fused kernel's tile table
+    fused_act = (rows >= FUSED_SWIGLU_MIN_ROWS and K % 64 == 0 and two_n % 8 == 0 and two_n * K < 2 ** 31
+                 and swiglu_tiles <= 1023 * 256)
+    if fused_act and fuse_gather and hidden_states.shape[0] * K * 2 < 2 ** 31:
+        h2 = grouped_gemm_swiglu_gathered(hidden_states, perm, k, w1.view(E * two_n, K), m_sizes)
     else:
-        h2 = silu_and_mul(grouped_gemm(xs, w1.view(E * two_n, K), m_sizes))
+        xs = gather_sorted(hidden_states, perm, k, offsets)
+        if fused_act:
+            h2 = grouped_gemm_swiglu(xs, w1.view(E * two_n, K), m_sizes)
+        else:
+            h2 = silu_and_mul(grouped_gemm(xs, w1.view(E * two_n, K), m_sizes))
     y2 = grouped_gemm(h2, w2.view(E * w2.shape[1], w2.shape[2]), m_sizes)
     return combine_topk(y2, perm, offsets, tw, out=hidden_states if inplace else None)
 

@@ -130,6 +130,41 @@ def grouped_gemm_swiglu(x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor)
     return y
 
 
+def grouped_gemm_swiglu_gathered(tokens: torch.Tensor, perm: torch.Tensor, k: int, w: torch.Tensor,
+                                 m_sizes: torch.Tensor) -> torch.Tensor:
+    """grouped_gemm_swiglu(tokens[perm // k], w, m_sizes) without the gathered copy: the kernel reads row perm[i] // k
+    of tokens [T, K] where the plain form reads sorted row i, as the reference's kernel reads A through
+    sorted_token_ids (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:75-80). perm [M] int32 and m_sizes
+    as route_group returns them; rows at or beyond sum(m_sizes) are left unwritten. Same bits as the two-step form.
+    Needs T * K * 2 < 2**31 bytes of tokens (ValueError beyond: gather first)."""
+    assert tokens.is_contiguous()
+    assert w.is_contiguous()
+    assert m_sizes.is_contiguous() and perm.is_contiguous()
+    if tokens.dim() != 2 or w.dim() != 2 or m_sizes.dim() != 1 or perm.dim() != 1:
+        raise ValueError("tokens must be [T, K], perm [M], w [G*2n, K], m_sizes [G]")
+    G = m_sizes.shape[0]
+    T, K = tokens.shape
+    M = perm.shape[0]
+    if G == 0 or w.shape[0] % (2 * G) != 0:
+        raise ValueError(f"w.shape[0]={w.shape[0]} is not a multiple of 2*G={2 * G}")
+    n = w.shape[0] // (2 * G)
+    assert K == w.shape[1], f"K mismatch: tokens have {K}, w has {w.shape[1]}"
+    if tokens.dtype not in (torch.bfloat16, torch.float16) or w.dtype != tokens.dtype:
+        raise ValueError("grouped_gemm_swiglu_gathered takes bf16 (or fp16) tokens and w of the same dtype")
+    if m_sizes.dtype != torch.int32 or perm.dtype != torch.int32:
+        raise ValueError("m_sizes and perm must be int32")
+    if k < 1:
+        raise ValueError("k must be at least 1")
+    dev = _require_cuda(tokens, w, m_sizes, perm)
+    y = torch.empty((M, n), device=dev, dtype=tokens.dtype)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().moe_gg_grouped_gemm_swiglu_gather(tokens.data_ptr(), T, perm.data_ptr(), k, w.data_ptr(), y.data_ptr(),
+                                                          m_sizes.data_ptr(), G, M, n, K, n, 1 if tokens.dtype == torch.float16 else 0,
+                                                          _stream_ptr(dev))
+    _lib.check(rc, "moe_gg_grouped_gemm_swiglu_gather")
+    return y
+
+
 def grouped_gemm_backward(grad_output: torch.Tensor, x: torch.Tensor, w: torch.Tensor, m_sizes: torch.Tensor):
     """Backward pass of the bf16 grouped GEMM: returns (grad_x [M, K], grad_w [G*N, K]).
 

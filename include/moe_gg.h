@@ -233,6 +233,22 @@ int moe_gg_grouped_gemm_swiglu_f16(const void* x, const void* w, void* y, const 
                                    int n, int K, int64_t ldy, void* stream);
 
 /*
+ * The same product with the layer's row gather folded into the activation loads: row i of the expert-sorted order
+ * is row perm[i] / k of the token matrix, as the reference's kernel reads A through sorted_token_ids
+ * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:75-80, 93-96) instead of from a gathered copy.
+ *   y[i, c] = silu(tokens[perm[i] / k] . w[g(i)*2n + c]) * (tokens[perm[i] / k] . w[g(i)*2n + n + c])
+ * tokens device [T, K] (bf16, or fp16 with dtype = MOE_GG_DTYPE_FP16); perm device [M] int32 as moe_gg_route_group
+ * writes it (entries of the first sum(m_sizes) positions are slots token * k + j < T * k; later ones are not read);
+ * everything else as moe_gg_grouped_gemm_swiglu_bf16, whose result on moe_gg_gather_rows(tokens, perm, k) it equals
+ * bit for bit. Requires in addition T * K * 2 < 2^31 (MOE_GG_EUNSUPPORTED otherwise: gather first). A perm entry
+ * outside [0, T * k) cannot make the loads leave the token matrix (it is folded into range); the row it produces is
+ * unspecified.
+ */
+int moe_gg_grouped_gemm_swiglu_gather(const void* tokens, int64_t T, const int32_t* perm, int k, const void* w, void* y,
+                                      const int32_t* m_sizes, int G, int64_t M, int n, int K, int64_t ldy, int dtype,
+                                      void* stream);
+
+/*
  * Glue between the two grouped GEMMs of a whole MoE layer, as in the reference's fused_moe
  * (kernels/triton/inference/col_major_moe_gemm/v0_moe_fused.py:222-296; oracle torch_moe,
  * kernels/triton/inference/col_major_moe_gemm/test_moe_gemm.py:16-30). All data bf16.

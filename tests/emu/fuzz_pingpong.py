@@ -25,13 +25,25 @@ def one_case(rng):
     M = sum(sizes)
     N = int(rng.choice([64, 256, 320, 512, 768]))
     K = int(rng.choice([64, 128, 192]))
-    op = str(rng.choice(["bf16", "f16", "swiglu", "fp8row", "fp8block"]))
+    op = str(rng.choice(["bf16", "f16", "swiglu", "gather", "fp8row", "fp8block"]))
     if op in ("bf16", "f16"):
         fp16 = op == "f16"
         x = rng.integers(-4, 5, (M, K)).astype(np.float32)
         w = rng.integers(-4, 5, (G * N, K)).astype(np.float32)
         y = H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), sizes, N, fp16=fp16, variant=0)
         good = (H.from16(y, fp16) == H.from16(H.to16(O.grouped_gemm(x, w, sizes), fp16), fp16)).all()
+    elif op == "gather":   # the fused activation kernel reading its rows through a permutation: same bits as gather + kernel
+        n, k = max(64, N // 2 // 4 * 4), int(rng.integers(1, 4))
+        T = max(1, -(-M // k))
+        tok = H.to_bf16(rng.integers(-2, 3, (T, K)).astype(np.float32))
+        w = H.to_bf16((rng.integers(-2, 3, (G * 2 * n, K)) * 0.125).astype(np.float32))
+        ids = np.repeat(np.arange(G), sizes)                      # expert of every sorted row
+        flat = np.full(T * k, -1, dtype=np.int64)
+        flat[rng.permutation(T * k)[:M]] = ids                    # scattered over the slots, the rest masked
+        perm, ms, _ = H.route_group(flat, G)
+        good = (ms == np.array(sizes)).all()
+        two_step = H.grouped_gemm_swiglu(H.gather_rows(tok, perm, k, n_valid=M), w, ms, n)
+        good = bool(good and (H.grouped_gemm_swiglu_gather(tok, perm, k, w, ms, n)[:M] == two_step[:M]).all())
     elif op == "swiglu":
         n = max(64, N // 2 // 4 * 4)
         x = rng.integers(-2, 3, (M, K)).astype(np.float32)

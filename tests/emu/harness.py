@@ -156,6 +156,15 @@ def grouped_gemm_swiglu(x16, w16, m_sizes, n, fp16=False):
     return y
 
 
+def grouped_gemm_swiglu_gather(tokens16, perm, k, w16, m_sizes, n, fp16=False):
+    L = lib()
+    ms, pm = i32(m_sizes), i32(perm)
+    G, (T, K), M = len(ms), tokens16.shape, len(pm)
+    y = _full((M, n), NAN16, dtype=np.uint16)
+    ok(L.moe_gg_grouped_gemm_swiglu_gather(P(tokens16), T, P(pm), k, P(w16), P(y), P(ms), G, M, n, K, n, FP16 if fp16 else BF16, None))
+    return y
+
+
 def backward(go16, x16, w16, m_sizes, N, block_layout=False, static=False):
     L = lib()
     ms = i32(m_sizes)

@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <utility>
 #include <vector>
 
 #include "../../include/moe_gg.h"
@@ -78,6 +79,13 @@ static int one_shape(const char* op, int N, int K, int G, char** sizes) {
   } else if (!std::strcmp(op, "swiglu")) {
     auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * 2 * N * K);
     check(moe_gg_grouped_gemm_swiglu_bf16(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, nullptr), op);
+  } else if (!std::strcmp(op, "gather")) {  // sorted row i = token row perm[i] / 2, perm a shuffle of the slots
+    const int T = (M + 1) / 2;
+    auto x = bf16_small((size_t)T * K), w = bf16_small((size_t)G * 2 * N * K);
+    Buf<int32_t> perm(M);
+    for (int i = 0; i < M; ++i) perm.v[i] = i;
+    for (int i = M - 1; i > 0; --i) std::swap(perm.v[i], perm.v[rnd() % (i + 1)]);
+    check(moe_gg_grouped_gemm_swiglu_gather(x.p(), T, perm.p(), 2, w.p(), y.p(), ms.p(), G, M, N, K, N, MOE_GG_DTYPE_BF16, nullptr), op);
   } else {
     const bool f16 = !std::strcmp(op, "f16");
     auto x = f16 ? f16_small((size_t)M * K) : bf16_small((size_t)M * K);
@@ -90,7 +98,7 @@ static int one_shape(const char* op, int N, int K, int G, char** sizes) {
 
 // race_check                       all entry points (exit status 0 unless the sanitizer reported something: then 66)
 // race_check selftest K B          control kernel K (0: stores, 1: global->LDS load), B = 1 with / 0 without the barrier
-// race_check shape OP N K m1 m2 .. one launch; OP = bf16 | f16 | swiglu | fp8row | fp8block | bwd
+// race_check shape OP N K m1 m2 .. one launch; OP = bf16 | f16 | swiglu | gather | fp8row | fp8block | bwd
 int main(int argc, char** argv) {
   if (argc == 4 && !std::strcmp(argv[1], "selftest")) {
     std::printf("sum %d\n", race_selftest(std::atoi(argv[2]), std::atoi(argv[3])));

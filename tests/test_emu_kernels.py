@@ -110,6 +110,48 @@ def test_fused_silu_and_mul_gemm(fp16):
     np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("fp16", [False, True])
+@pytest.mark.parametrize("T,E,k,n,K", [(200, 4, 2, 128, 128), (700, 8, 2, 192, 64), (300, 3, 3, 64, 256), (33, 2, 1, 256, 128)])
+def test_gather_folded_into_the_first_gemm_gives_the_same_bits(fp16, T, E, k, n, K):
+    """moe_gg_grouped_gemm_swiglu_gather on the token matrix and the permutation against moe_gg_gather_rows followed by
+    moe_gg_grouped_gemm_swiglu: bit for bit, with masked slots, and rows beyond sum(m_sizes) left alone."""
+    rng = np.random.default_rng(T + n)
+    tok = H.to16(ints(rng, (T, K), -3, 4), fp16)
+    w = H.to16(ints(rng, (E * 2 * n, K), -2, 3) * 0.125, fp16)
+    ids = rng.integers(0, E, (T, k))
+    ids.ravel()[rng.permutation(T * k)[:T * k // 10]] = -1
+    perm, ms, _ = H.route_group(ids, E)
+    nv = int(ms.sum())
+    two_step = H.grouped_gemm_swiglu(H.gather_rows(tok, perm, k, n_valid=nv), w, ms, n, fp16)
+    fused = H.grouped_gemm_swiglu_gather(tok, perm, k, w, ms, n, fp16)
+    assert (fused[:nv] == two_step[:nv]).all() and (fused[nv:] == H.NAN16).all()
+
+
+def test_gather_with_a_corrupt_permutation_stays_inside_the_token_matrix():
+    """Entries of perm outside [0, T k) (a caller's mistake: route_group never writes them in the rows that are read):
+    with the token matrix against guard pages on either side the call completes, and rows with valid entries are
+    still right."""
+    rng = np.random.default_rng(3)
+    T, E, k, n, K = 150, 2, 2, 64, 128
+    tok = H.to_bf16(ints(rng, (T, K), -3, 4))
+    w = H.to_bf16(ints(rng, (E * 2 * n, K), -2, 3) * 0.125)
+    ids = rng.integers(0, E, (T, k))
+    perm, ms, _ = H.route_group(ids, E)
+    want = H.grouped_gemm_swiglu(H.gather_rows(tok, perm, k), w, ms, n)
+    bad = perm.copy()
+    hit = rng.permutation(T * k)[:40]
+    bad[hit] = rng.choice([-1, -2 ** 31, 2 ** 31 - 1, T * k, T * k + 7, 10 ** 9], 40)
+    for guard in ("end", "start"):
+        H.GUARD = guard
+        try:
+            got = H.grouped_gemm_swiglu_gather(tok, bad, k, w, ms, n).copy()
+        finally:
+            H.GUARD = None
+            H.release()
+        keep = np.setdiff1d(np.arange(T * k), hit)
+        assert (got[keep] == want[keep]).all()
+
+
 @pytest.mark.parametrize("sizes,N,K,block,static", [
     (SIZES, 256, 128, False, False), (SIZES, 256, 128, True, False), (SIZES, 256, 128, False, True),
     ([30, 0, 7, 53], 64, 64, False, False), ([0, 5, 0], 64, 64, False, False), ([300, 200], 68, 36, False, False)])
@@ -337,6 +379,7 @@ def test_no_data_race_between_the_waves_of_a_workgroup():
              for cus, seed in (("8", "0"), ("2", "7"))]
     # long tile sequences in one workgroup: split tails, row pieces of the last round, short and empty experts
     shapes = [("bf16", "512", "128", "1", "0", ["530", "300", "0", "70"]), ("swiglu", "256", "128", "2", "5", ["833", "64", "257"]),
+              ("gather", "128", "128", "2", "3", ["530", "1", "300"]),
               ("fp8block", "384", "256", "1", "0", ["577", "33", "320"]), ("fp8row", "256", "128", "3", "9", ["129", "768", "1"]),
               ("f16", "384", "256", "2", "0", ["321", "511"]), ("bwd", "256", "128", "3", "4", ["300", "0", "41", "513"])]
     for op, N, K, cus, seed, sizes in shapes:

@@ -26,7 +26,9 @@ HARNESS_HEAD = r'''
 using std::min; using std::max;
 constexpr int BM = 256, BN = 256, NT = 512;
 constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4, OP_BF16_NT = 5,
-              OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7, OP_F16_SWIGLU = 8;
+              OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7, OP_F16_SWIGLU = 8, OP_BF16_SWIGLU_GATHER = 9, OP_F16_SWIGLU_GATHER = 10;
+constexpr bool op_gather(int op) { return op == OP_BF16_SWIGLU_GATHER || op == OP_F16_SWIGLU_GATHER; }
+constexpr bool op_swiglu(int op) { return op == OP_BF16_SWIGLU || op == OP_F16_SWIGLU || op_gather(op); }
 struct GgParams { const int32_t* m_sizes; int G, M, N, K, skip_rows, tails_apart, xcds; };
 struct Dim { int x; };
 static Dim blockIdx, threadIdx, gridDim;
@@ -69,6 +71,7 @@ extern "C" int emu_prologue(int op, const int32_t* m_sizes, int G, int M, int N,
     int n_my = 0;
     if (op == OP_BF16) prologue<OP_BF16>(p, seq, &n_my);
     else if (op == OP_BF16_SWIGLU) prologue<OP_BF16_SWIGLU>(p, seq, &n_my);
+    else if (op == OP_BF16_SWIGLU_GATHER) prologue<OP_BF16_SWIGLU_GATHER>(p, seq, &n_my);
     else if (op == OP_FP8_BLOCK) prologue<OP_FP8_BLOCK>(p, seq, &n_my);
     else return -1;
     for (int i = 0; i < n_my; ++i) {
@@ -146,8 +149,9 @@ def test_device_prologue_equals_the_host_mirror(emu, lib):
         assert h.shape == d.shape and (h == d).all(), ("bf16", sizes[:8], N, nwg)
         n_out = max(128, N // 2 // 128 * 128)       # fused gate/up kernel: p.N = 2 n, tiles of 128 output columns
         h = host_tiles(lib, sizes, n_out, 128, nwg)
-        d = device_tiles(emu, 4, sizes, 2 * n_out, 4096, nwg)
-        assert h.shape == d.shape and (h == d).all(), ("swiglu", sizes[:8], n_out, nwg)
+        for op in (4, 9):   # the fused gate/up kernel and its form with the row gather
+            d = device_tiles(emu, op, sizes, 2 * n_out, 4096, nwg)
+            assert h.shape == d.shape and (h == d).all(), ("swiglu", op, sizes[:8], n_out, nwg)
 
 
 def cover(tiles, sizes, N):
