@@ -1,7 +1,7 @@
 """GPU parity of the first MoE GEMM with the row gather folded into its loads (moe_gg_grouped_gemm_swiglu_gather,
 fused_moe(..., fuse_gather=True)): bit-identical to the gathered copy followed by the plain fused kernel, and the
-layer against the oracle. Collected late on purpose: the kernel has run under the CPU emulation only so far, and a
-failure here must not hide the parity tests before it."""
+layer against the oracle. Collected last on purpose: the kernel has run under the CPU emulation only so far, and a
+failure here must not hide any other test."""
 import numpy as np
 import pytest
 import torch
