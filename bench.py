@@ -359,7 +359,7 @@ def wl_w4a16_grouped(torch, A, dev, lib, stream, cpu):
 
 
 def wl_fp8_cfg5(torch, A, dev, lib, stream, cpu):
-    """Config 5 with the inputs BASELINE states: x ~ N(0, 1) through the 1 x 128 quantiser, weights ~ N(0, 0.02)
+    """Config 5 with the inputs its definition states: x ~ N(0, 1) through the 1 x 128 quantiser, weights ~ N(0, 0.02)
     through the 128 x 128 block quantiser (drawn and quantised expert by expert to bound memory)."""
     from applied_ai_amd import configs
 

@@ -45,7 +45,7 @@ def test_decode_small(G, N, K, m_sizes, variant):
 
 @pytest.mark.parametrize("down", [False, True])
 def test_mixtral_decode_shapes(down):
-    """BASELINE config 3: T=32 top-2 over 8 experts (64 rows); up-proj K=4096, N=14336 and down-proj K=14336,
+    """benchmark config 3: T=32 top-2 over 8 experts (64 rows); up-proj K=4096, N=14336 and down-proj K=14336,
     N=4096. Oracle on every row for a 512-column slice per expert; bitwise determinism; and the auto-dispatch picks
     the same result as the pinned decode variant."""
     from applied_ai_amd import configs

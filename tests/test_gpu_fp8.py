@@ -125,7 +125,7 @@ def test_block_quantiser_bit_exact(dtype):
 
 
 def test_config5_full_size():
-    """BASELINE config 5 as one launch: 256 experts, T = 4096 tokens top-8 -> 32768 rows with Zipf(1.1) routing,
+    """benchmark config 5 as one launch: 256 experts, T = 4096 tokens top-8 -> 32768 rows with Zipf(1.1) routing,
     x ~ N(0,1) [32768, 7168] through the 1 x 128 quantiser, fused gate+up weights ~ N(0, 0.02) [256, 4096, 7168]
     through the 128 x 128 block quantiser (drawn and quantised expert by expert to bound memory), bf16 out.
     Checked against the dequantise-then-matmul oracle (the recipe of dev/triton_groupGEMM/testing/
@@ -194,7 +194,7 @@ def test_config5_full_size():
 
 
 def test_config5_shape_sampled_experts():
-    """BASELINE config 5 at full K and N (7168, 4096) with its Zipf routing, on a sample of experts (largest,
+    """benchmark config 5 at full K and N (7168, 4096) with its Zipf routing, on a sample of experts (largest,
     smallest, two in between): activations quantised by the GPU quantiser, weights by the block quantiser,
     oracle on a 256-column slice."""
     import applied_ai_amd as A

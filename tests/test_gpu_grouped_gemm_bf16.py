@@ -138,7 +138,7 @@ def test_bitwise_deterministic():
 
 
 def test_config1_plumbing_from_golden_fixture():
-    # BASELINE config 1 (8 experts, K=256, N=512, 256 tokens top-2) run in bf16 against the committed vectors
+    # benchmark config 1 (8 experts, K=256, N=512, 256 tokens top-2) run in bf16 against the committed vectors
     import os
 
     z = np.load(os.path.join(os.path.dirname(__file__), "golden", "cfg1.npz"))
@@ -163,7 +163,7 @@ def test_invalid_inputs_raise():
 
 
 def test_mixtral_prefill_shape_sampled_rows():
-    """BASELINE config 2 at full size (T=4096 top-2, K=4096, N=14336, 8 experts); the oracle checks 8 sampled rows
+    """benchmark config 2 at full size (T=4096 top-2, K=4096, N=14336, 8 experts); the oracle checks 8 sampled rows
     per expert over all columns, and linearity checks the rest: y(2x) == 2 y(x) exactly in bf16."""
     from applied_ai_amd import configs
 
