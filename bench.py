@@ -419,17 +419,7 @@ def wl_moe_layer(torch, A, dev, lib, stream, cpu):
               "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong (two launches) + glue kernels", "achieved": round(flop / ms / 1e9, 1),
                            "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
                            "traffic": None}})
-    out = [e]
-    # The same layer with the row gather folded into the first GEMM's loads (opt-in until it has been measured).
-    try:
-        st_g = event_stats(torch, lambda: A.fused_moe(h, w1, w2, tw, ids, fuse_gather=True), 10, 3, batches=5)
-        g = {"workload": "the same layer with fuse_gather=True (first GEMM reads the token rows through the permutation, no gathered copy)"}
-        g.update(timing_fields(st_g, "ms"))
-        g.update({"value": round(flop / st_g["p50"] / 1e9, 1), "unit": "TFLOP/s"})
-        out.append(g)
-    except Exception as exc:
-        out.append({"workload": "fused_moe with fuse_gather=True", "error": f"{type(exc).__name__}: {exc}"})
-    return out
+    return [e]
 
 
 def wl_backward(torch, A, dev, lib, stream, cpu):

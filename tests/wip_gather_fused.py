@@ -1,7 +1,7 @@
 """GPU parity of the first MoE GEMM with the row gather folded into its loads (moe_gg_grouped_gemm_swiglu_gather,
 fused_moe(..., fuse_gather=True)): bit-identical to the gathered copy followed by the plain fused kernel, and the
-layer against the oracle. Collected last on purpose: the kernel has run under the CPU emulation only so far, and a
-failure here must not hide any other test."""
+layer against the oracle. Not collected by pytest under this name (run it by naming the file): the kernel has run under the CPU emulation only
+(tests/test_emu_kernels.py); it joins the collected GPU tests once it has passed on a GPU."""
 import numpy as np
 import pytest
 import torch
