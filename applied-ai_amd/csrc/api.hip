@@ -170,6 +170,7 @@ static int grouped_gemm_16(const void* x, const void* w, void* y, const int32_t*
       return (int)gg_bf16_decode_tails_launch(p, s);
     }
     case MOE_GG_GG_TILED_256: return (int)gg_bf16_tiled_launch(p, 256, num_wg, s);
+    case MOE_GG_GG_TILED_256_W4: return (int)gg_bf16_tiled_launch(p, GG_TILED_256_FOUR_WAVES, num_wg, s);
     case MOE_GG_GG_TILED_128: return (int)gg_bf16_tiled_launch(p, 128, num_wg, s);
     case MOE_GG_GG_TILED_64: return (int)gg_bf16_tiled_launch(p, 64, num_wg, s);
     default: return MOE_GG_EINVAL;

@@ -247,13 +247,15 @@ hipError_t launch(const GgParams& p, int num_wg, hipStream_t stream) {
 hipError_t gg_bf16_tiled_launch(const GgParams& p, int block_m, int num_wg, hipStream_t stream) {
   switch (block_m) {
     case 256: return launch<Cfg<256, 256, 2, 4>>(p, num_wg, stream);
+    // The same tile on four waves, 128 x 128 outputs each: accumulators in AGPRs, a third fewer LDS bytes per MFMA.
+    case GG_TILED_256_FOUR_WAVES: return launch<Cfg<256, 256, 2, 2>>(p, num_wg, stream);
     case 128: return launch<Cfg<128, 128, 2, 2>>(p, num_wg, stream);
     case 64: return launch<Cfg<64, 128, 2, 2>>(p, num_wg, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
-int gg_bf16_tiled_block_n(int block_m) { return block_m == 256 ? 256 : 128; }
+int gg_bf16_tiled_block_n(int block_m) { return (block_m == 256 || block_m == GG_TILED_256_FOUR_WAVES) ? 256 : 128; }
 
 hipError_t gg_bf16_wgrad_launch(const GgParams& p, int block, int num_wg, hipStream_t stream) {
   if (block == 256) return launch<Cfg<256, 256, 2, 4>, true>(p, num_wg, stream);

@@ -32,7 +32,9 @@ struct GgParams {
   int gather_rows;
 };
 
-// block_m in {256, 128, 64}; the matching tile width is gg_bf16_tiled_block_n(block_m).
+// block_m in {256, 128, 64}, or GG_TILED_256_FOUR_WAVES for the 256 x 256 tile on a four-wave workgroup; the matching
+// tile width is gg_bf16_tiled_block_n(block_m).
+constexpr int GG_TILED_256_FOUR_WAVES = 2564;
 hipError_t gg_bf16_tiled_launch(const GgParams& p, int block_m, int num_wg, hipStream_t stream);
 int gg_bf16_tiled_block_n(int block_m);
 // 256 x 256 tiles, ping-pong schedule (gg_pingpong.hip); the fp8 form takes the scale modes of gg_fp8_launch

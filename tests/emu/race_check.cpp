@@ -112,7 +112,7 @@ int main(int argc, char** argv) {
     std::memcpy(ms.p(), sizes, sizeof(sizes));
     auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * N * K);
     Buf<uint16_t> y((size_t)M * N * G);
-    for (int variant = -1; variant <= 5; ++variant) {
+    for (int variant = -1; variant <= 6; ++variant) {
       moe_gg_set_variant(MOE_GG_OP_GG_BF16, variant);
       check(moe_gg_grouped_gemm_bf16(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, MOE_GG_OUT_MN, nullptr), "grouped_gemm_bf16 (every variant)");
     }

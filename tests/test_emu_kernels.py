@@ -44,7 +44,7 @@ def exact16(got16, want, fp16=False):
 SIZES = [300, 0, 70, 530]   # a full tile + a low tile, an empty expert, a short one, a tall one whose tail is split
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, -1])
 def test_bf16_every_kernel_variant(variant):
     rng = np.random.default_rng(variant + 1)
     x, w = ints(rng, (sum(SIZES), 128)), ints(rng, (4 * 512, 128))
