@@ -36,6 +36,9 @@ int current_device_info(const DeviceInfo** out) {
   return MOE_GG_OK;
 }
 
+// Tile order of the forward ping-pong kernels (MOE_GG_OP_TILE_ORDER): the split-tail order only when it is pinned.
+int split_tails_on() { return g_variant[MOE_GG_OP_TILE_ORDER].load() == MOE_GG_ORDER_SPLIT_TAILS ? 1 : 0; }
+
 bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
 // How wide the kernels may store row segments of y: 2 = 16 bytes, 1 = 8 bytes, 0 = element by element. col_step
@@ -118,6 +121,7 @@ static int grouped_gemm_16(const void* x, const void* w, void* y, const int32_t*
   p.vec_store = vec_store_level(y, ldy, N);
   p.xcds = di->xcds;
   p.fp16 = fp16 ? 1 : 0;
+  p.split_tails = split_tails_on();
 
   hipStream_t s = (hipStream_t)stream;
   const bool tiled_ok = K % 64 == 0 && aligned(x, 16) && aligned(w, 16);
@@ -215,6 +219,7 @@ int moe_gg_grouped_gemm_fp8(const void* x, const void* w, void* y, const float* 
   p.col_block = out_layout == MOE_GG_OUT_BLOCK ? N : 0;
   p.vec_store = vec_store_level(y, ldy, N);
   p.xcds = di->xcds;
+  p.split_tails = split_tails_on();
   int num_wg = di->cus - di->cus % p.xcds;
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
   // A few rows per expert (see use_streaming_kernel): the experts with up to 64 rows go to the streaming
@@ -369,6 +374,7 @@ static int grouped_gemm_swiglu_16(const void* x, const void* w, void* y, const i
   if (num_wg <= 0) { num_wg = di->cus; p.xcds = 1; }
   if (!moe_gg_two_list_fits(M, G, 256, (n + 127) / 128, num_wg)) return MOE_GG_EUNSUPPORTED;
   p.fp16 = fp16 ? 1 : 0;
+  p.split_tails = split_tails_on();
   p.gather_perm = perm;
   p.gather_k = k;
   p.gather_rows = (int)T;
@@ -508,6 +514,7 @@ static int backward_bf16_impl(const void* grad_out, int64_t ld_go, int grad_layo
       q.ldx = (int)ld_go; q.x_col_block = x_col_block;
       q.vec_store = vec_store_level(grad_x, K, 0);
       q.xcds = xcds;
+      q.split_tails = split_tails_on();
       e = gg_bf16_pingpong_nt_launch(q, num_wg, s);
       if (e != hipSuccess) return (int)e;
     } else {
@@ -686,7 +693,7 @@ int moe_gg_host_tails_apart(const int32_t* m_sizes_host, int G, int64_t M, int N
 
 int moe_gg_host_tail_pieces(int n_long, int n_low, int num_workgroups) {
   if (n_long < 0 || n_low < 0 || num_workgroups <= 0) return MOE_GG_EINVAL;
-  return moe_gg_tail_pieces_low(n_long, n_low, num_workgroups);
+  return split_tails_on() ? moe_gg_tail_pieces_low(n_long, n_low, num_workgroups) : moe_gg_tail_pieces(n_long, num_workgroups);
 }
 
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
@@ -697,8 +704,9 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     return MOE_GG_EINVAL;
   static thread_local int32_t row_off[MOE_GG_MAX_GROUPS_ABI + 1], long_off[MOE_GG_MAX_GROUPS_ABI + 1],
       low_off[MOE_GG_MAX_GROUPS_ABI + 1];
-  // The lists of a launch that computes its low tiles itself (split tails on); the decode below is the kernels' own.
-  const bool split = true;
+  // The lists of a launch that computes its low tiles itself, in the tile order that is in force
+  // (MOE_GG_OP_TILE_ORDER); the decode below is the kernels' own.
+  const bool split = split_tails_on() != 0;
   const int ntn = moe_gg_cdiv(N, block_n);
   int64_t r = 0;
   int nl = 0, ns = 0;
@@ -710,7 +718,7 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     ns += moe_gg_low_row_tiles2(m, block_m, split) * ntn;
   }
   row_off[G] = (int32_t)r; long_off[G] = nl; low_off[G] = ns;
-  const int tail_s = moe_gg_tail_pieces_low(nl, ns, num_workgroups);
+  const int tail_s = split ? moe_gg_tail_pieces_low(nl, ns, num_workgroups) : moe_gg_tail_pieces(nl, num_workgroups);
   const int tail_first = moe_gg_tail_first_s(nl, num_workgroups, tail_s);
   const int long_ids = moe_gg_long_ids_s(nl, num_workgroups, tail_s);
   const int total = long_ids + ns;

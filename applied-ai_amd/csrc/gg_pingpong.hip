@@ -687,9 +687,10 @@ DEVINL void pingpong_body(const GgParams& p) {
   static_assert(2 * MOE_GG_SEQ_CAP >= MOE_GG_MAX_GROUPS + 1, "seq_tab doubles as a prefix table below");
 
   int total, total_low = 0;
-  // Forward lists: tall groups with a few rows beyond their last full tile get two half tiles for their last rows
-  // (moe_gg_split_tail), unless the small-M kernel of the same call takes the low tiles.
-  bool split = true;
+  // Forward lists with p.split_tails: tall groups with a few rows beyond their last full tile get two half tiles for
+  // their last rows (moe_gg_split_tail), unless the small-M kernel of the same call takes the low tiles.
+  bool split = p.split_tails != 0;
+  bool apart = false;  // the low tiles are the small-M kernel's
   if (OP == OP_BF16_WGRAD_DIRECT) {
     build_row_offsets(p.m_sizes, p.G, p.M, row_off);
     total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
@@ -707,20 +708,22 @@ DEVINL void pingpong_body(const GgParams& p) {
       build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
       build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
       build_tile_prefix(row_off, p.G, seq_tab, [&](int rows) { return moe_gg_low_passes(rows, BM) * ntn; });
-      if (moe_gg_tails_apart(uni(tile_off[p.G]), uni(part_off[p.G]), uni(seq_tab[p.G]), p.tails_apart)) split = false;
+      apart = moe_gg_tails_apart(uni(tile_off[p.G]), uni(part_off[p.G]), uni(seq_tab[p.G]), p.tails_apart);
+      if (apart) split = false;
       __syncthreads();  // the tables are rewritten below
     }
     build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles2(rows, BM, split) * ntn : 0; });
     build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles2(rows, BM, split) * ntn : 0; });
-    total_low = split ? uni(part_off[p.G]) : 0;   // split off: the low tiles are the small-M kernel's
+    total_low = apart ? 0 : uni(part_off[p.G]);
     total = uni(tile_off[p.G]);
   }
   const int nwg = gridDim.x;
   // Tiles of this workgroup in each list: rounds 0 .. n - 1 (tile ids grow with the round).
-  // (Forward kernels: the long tiles of a sparsely filled last round are cut into row pieces, as many as make the
-  // busiest workgroup's load smallest with the second list dealt behind them, moe_gg_tail_pieces_low.)
+  // (Forward kernels: the long tiles of a sparsely filled last round are cut into row pieces: by the fill of that
+  // round alone (moe_gg_tail_pieces), or, with p.split_tails, as many as make the busiest workgroup's load smallest
+  // with the second list dealt behind them, moe_gg_tail_pieces_low.)
   const bool fwd = OP != OP_BF16_WGRAD && OP != OP_BF16_WGRAD_DIRECT;
-  const int tail_s = fwd ? moe_gg_tail_pieces_low(total, total_low, nwg) : 1;
+  const int tail_s = !fwd ? 1 : p.split_tails ? moe_gg_tail_pieces_low(total, total_low, nwg) : moe_gg_tail_pieces(total, nwg);
   const int tail_first = moe_gg_tail_first_s(total, nwg, tail_s);
   const int long_ids = moe_gg_long_ids_s(total, nwg, tail_s);
   const int low_ids = total_low;

@@ -30,6 +30,9 @@ struct GgParams {
   const int32_t* gather_perm;
   int gather_k;
   int gather_rows;
+  // Forward ping-pong kernels: 1 = split-tail tile order (moe_gg_split_tail, row pieces chosen by
+  // moe_gg_tail_pieces_low), 0 = the plain two-list order (row pieces by moe_gg_tail_pieces).
+  int split_tails;
 };
 
 // block_m in {256, 128, 64}, or GG_TILED_256_FOUR_WAVES for the 256 x 256 tile on a four-wave workgroup; the matching

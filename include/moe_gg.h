@@ -321,12 +321,20 @@ int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scale
 #define MOE_GG_FP8_STREAM_PINGPONG 1 /* experts with <= 64 rows: streaming split-K kernel; others: 256x256 ping-pong */
 #define MOE_GG_FP8_STREAM_TILED 2    /* experts with <= 64 rows: streaming split-K kernel; others: 128x128 tiles */
 #define MOE_GG_FP8_PINGPONG 3        /* 256x256 ping-pong kernel for every expert */
+#define MOE_GG_OP_TILE_ORDER 2
+/* variants of MOE_GG_OP_TILE_ORDER: tile order of the forward 256x256 ping-pong kernels (bf16, f16, fp8, the fused
+ * SiLU-and-mul GEMM, grad_x of the backward pass) and of the host enumerators below. -1 means TWO_LISTS: the
+ * split-tail order is opt-in until a timed run on the hardware has shown what it is worth. */
+#define MOE_GG_ORDER_TWO_LISTS 0   /* long tiles, then low tiles; last round cut by its fill alone */
+#define MOE_GG_ORDER_SPLIT_TAILS 1 /* + a tall expert's last full tile and few rows become two half tiles; row
+                                      pieces of the last round chosen with the second list in view */
 int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,
                                 int max_tiles);
 /* The same for the 256 x 256 ping-pong kernels (block_m must be 256), which keep two tile lists (long tiles; low
- * tiles and the two half tiles that replace the last full tile + few rows of a tall group), give every workgroup
+ * tiles and, with MOE_GG_ORDER_SPLIT_TAILS pinned, the two half tiles that replace the last full tile + few rows of
+ * a tall group), give every workgroup
  * its tiles of the second list spread between its long ones, and cut the long tiles of a sparsely filled last
  * round into row pieces. Six int32 per tile here: (workgroup,
  * group, first row inside the group, rows, first column, columns), for each workgroup in the order in which it
@@ -336,7 +344,8 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
                                           int block_n, int num_workgroups, int xcds, int32_t* out,
                                           int max_tiles);
 /* Into how many row pieces (1, 2 or 4) the ping-pong kernels cut the long tiles of their last round when the long
- * list has n_long tiles, the second list n_low and the launch num_workgroups workgroups. */
+ * list has n_long tiles, the second list n_low and the launch num_workgroups workgroups, in the tile order that is
+ * in force (n_low only matters to MOE_GG_ORDER_SPLIT_TAILS). */
 int moe_gg_host_tail_pieces(int n_long, int n_low, int num_workgroups);
 
 /* bf16 forward, automatic kernel choice with 256 x 256 tiles: 1 if for these (host) m_sizes the low tiles (an

@@ -24,7 +24,7 @@ _keep = []
 _libc = ctypes.CDLL(None, use_errno=True)
 _libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
 BF16, FP16, FP32 = 0, 1, 2
-OP_BF16, OP_FP8 = 0, 1
+OP_BF16, OP_FP8, OP_TILE_ORDER = 0, 1, 2
 
 
 def lib():
@@ -36,6 +36,9 @@ def lib():
             f.restype, f.argtypes = res, args
         for name in ("emu_nonuniform_readfirstlane", "emu_divergent_exchanges"):
             getattr(_L, name).restype = ctypes.c_ulonglong
+        # EMU_TILE_ORDER = 0 / 1: the ping-pong kernels' tile order for this process (MOE_GG_OP_TILE_ORDER)
+        if os.environ.get("EMU_TILE_ORDER"):
+            assert _L.moe_gg_set_variant(OP_TILE_ORDER, int(os.environ["EMU_TILE_ORDER"])) == 0
     return _L
 
 

@@ -100,6 +100,8 @@ static int one_shape(const char* op, int N, int K, int G, char** sizes) {
 // race_check selftest K B          control kernel K (0: stores, 1: global->LDS load), B = 1 with / 0 without the barrier
 // race_check shape OP N K m1 m2 .. one launch; OP = bf16 | f16 | swiglu | gather | fp8row | fp8block | bwd
 int main(int argc, char** argv) {
+  // EMU_TILE_ORDER = 0 / 1: the ping-pong kernels' tile order for this run (MOE_GG_OP_TILE_ORDER)
+  if (const char* order = std::getenv("EMU_TILE_ORDER")) moe_gg_set_variant(MOE_GG_OP_TILE_ORDER, std::atoi(order));
   if (argc == 4 && !std::strcmp(argv[1], "selftest")) {
     std::printf("sum %d\n", race_selftest(std::atoi(argv[2]), std::atoi(argv[3])));
     return 0;

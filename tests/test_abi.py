@@ -162,6 +162,20 @@ def test_scheduler_rejects_bad_arguments(lib):
     assert lib.moe_gg_host_enumerate_tiles(*args, 0, 1, out.ctypes.data_as(I32P), 8) == -1
 
 
+OP_TILE_ORDER, ORDER_TWO_LISTS, ORDER_SPLIT_TAILS = 2, 0, 1
+
+
+@pytest.fixture(params=[-1, ORDER_TWO_LISTS, ORDER_SPLIT_TAILS], ids=["default", "two_lists", "split_tails"])
+def tile_order(lib, request):
+    """Pins the tile order of the ping-pong kernels and their host mirror for one test; yields whether split tails
+    are on (the default, -1, is the plain two-list order)."""
+    assert lib.moe_gg_set_variant(OP_TILE_ORDER, request.param) == 0
+    try:
+        yield request.param == ORDER_SPLIT_TAILS
+    finally:
+        lib.moe_gg_set_variant(OP_TILE_ORDER, -1)
+
+
 @pytest.mark.parametrize("m_sizes,N,nwg", [
     ([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], 14336, 256),   # Mixtral prefill: 4 experts end in a low tile
     ([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], 4096, 256),    # 2.x rounds: the last one is cut into pieces
@@ -173,13 +187,15 @@ def test_scheduler_rejects_bad_arguments(lib):
     ([130, 128], 200, 64),                                           # row pieces of tiles with 128-130 rows
     ("cfg5", 4096, 256),                                             # 256 experts, 32768 Zipf-routed rows (fp8 config)
 ])
-def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
+def test_two_list_order_is_an_exact_cover_and_balanced(lib, tile_order, m_sizes, N, nwg):
     """The ping-pong kernels' order, decoded by the kernels' own code compiled for the host: every output element of
     every group exactly once. Second list: a low tile (fewer than 128 rows, the only row tile of its group or the last
-    one of a group with at least two full tiles and more than 64 rows left over), or the two half tiles (128 and
+    one of a group with at least two full tiles), or, in the split-tail order, the two half tiles (128 and
     128 + rem rows) that replace the last full tile and the rem <= 64 rows behind it in a group with at least two full
-    tiles. The long tiles of a sparsely filled last round are cut into 2 or 4 row pieces; every workgroup gets the same
-    number of tiles (+- 1), and the same number (+- 1) from the second list."""
+    tiles (a low tile then has more than 64 rows left over). The long tiles of a sparsely filled last round are cut
+    into 2 or 4 row pieces; every workgroup gets the same number of tiles (+- 1), and the same number (+- 1) from the
+    second list."""
+    split = tile_order
     if isinstance(m_sizes, str):
         from applied_ai_amd import configs
 
@@ -209,7 +225,7 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
     def kind(g, m0, h):
         m = m_sizes[g]
         full, rem = divmod(m, 256)
-        if full >= 2 and 0 < rem <= 64:
+        if split and full >= 2 and 0 < rem <= 64:
             if m0 == (full - 1) * 256 and h == 128:
                 return "half0"
             if m0 == (full - 1) * 256 + 128 and h == 128 + rem:
@@ -238,6 +254,25 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
         assert same >= 0.9 * len(halves) - 1
     row_pieces = sum(1 for wg, g, m0, h, n0, nc in tiles
                      if kind(g, m0, h) == "long" and (m0 % 256 or h < min(256, m_sizes[g] - m0)))
+    if not split:
+        assert not halves
+        if m_sizes[0] == 1012 and N == 14336:
+            # 7 long tiles and at most one low tile per workgroup: the XCDs (wg % 8) take their low tile at 8 different
+            # positions of the sequence, the workgroups of one XCD at the same one
+            assert row_pieces == 0 and len(tiles) == 7 * 256 + 4 * 56
+            pos = {}
+            for wg, v in per_wg.items():
+                if "low" in v:
+                    pos.setdefault(wg % 8, set()).add(v.index("low"))
+            assert all(len(q) == 1 for q in pos.values())
+            assert len(pos) == 7 and len({next(iter(q)) for q in pos.values()}) == 7   # 224 low tiles: 7 XCDs of 32
+        if m_sizes[0] == 1012 and N == 4096:
+            # 512 long tiles = 2 full rounds, then the 64 low tiles: nothing is cut
+            assert row_pieces == 0 and len(tiles) == 576
+        if m_sizes == [530]:
+            # 2 long tiles on 8 workgroups: 4 row pieces each; then the low tile (18 rows)
+            assert row_pieces == 8
+        return
     if m_sizes[0] == 1012 and N == 14336:
         # 1568 full tiles = 6 rounds + 32 tiles that are cut in two, then 448 half tiles: 8 rounds, every workgroup
         # 6 full tiles and 2 tiles or pieces of about half height (before: 7 full + 1 low tile for 224 workgroups)
@@ -256,7 +291,7 @@ def test_two_list_order_is_an_exact_cover_and_balanced(lib, m_sizes, N, nwg):
         assert sorted((m0, h) for wg, g, m0, h, n0, nc in tiles) == [(0, 128), (128, 128), (256, 128), (384, 146)]
 
 
-def test_two_list_order_random_sizes_exact_cover(lib):
+def test_two_list_order_random_sizes_exact_cover(lib, tile_order):
     """Random expert counts and sizes (with sizes around the tile edges and the split rule's limits 2 x 256 + 1 .. 64,
     and corrupt entries that the scheduler clamps): every output element once, every tile inside its group."""
     rng = np.random.default_rng(77)
@@ -289,15 +324,33 @@ def test_two_list_order_random_sizes_exact_cover(lib):
             assert (seen[g] == 1).all(), (case, g, eff[g], N, nwg)
 
 
+def test_tail_piece_choice_of_the_plain_order(lib):
+    """Without split tails the last round of long tiles is cut by its fill alone: quarters up to a quarter full, halves
+    up to half full."""
+    assert lib.moe_gg_set_variant(OP_TILE_ORDER, -1) == 0
+    for n_long, n_low, n, want in [(512, 0, 256, 1), (520, 0, 256, 4), (520, 300, 256, 4), (512 + 64, 9, 256, 4),
+                                   (512 + 65, 0, 256, 2), (512 + 128, 77, 256, 2), (512 + 129, 0, 256, 1), (7, 0, 8, 1)]:
+        assert lib.moe_gg_host_tail_pieces(n_long, n_low, n) == want, (n_long, n_low, n)
+    assert lib.moe_gg_host_tail_pieces(-1, 0, 256) < 0
+
+
 def test_tail_piece_choice_minimises_the_busiest_workgroup():
-    """moe_gg_host_tail_pieces against a brute-force simulation of the round-robin dealing with the same costs
-    (hundredths of a full tile: whole 100, half piece 55, quarter piece 43, tile of the second list 58)."""
+    """Split-tail order: moe_gg_host_tail_pieces against a brute-force simulation of the round-robin dealing with the
+    same costs (hundredths of a full tile: whole 100, half piece 55, quarter piece 43, tile of the second list 58)."""
     import ctypes
 
     import applied_ai_amd
 
     L = applied_ai_amd._lib.lib()
     rng = np.random.default_rng(5)
+    assert L.moe_gg_set_variant(OP_TILE_ORDER, ORDER_SPLIT_TAILS) == 0
+    try:
+        _tail_piece_cases(L, rng)
+    finally:
+        L.moe_gg_set_variant(OP_TILE_ORDER, -1)
+
+
+def _tail_piece_cases(L, rng):
 
     def busiest(P, a, Q, b, n):
         load = np.zeros(n, dtype=np.int64)

@@ -41,11 +41,22 @@ def exact16(got16, want, fp16=False):
     return bool((got[mask] == H.from16(H.to16(np.nan_to_num(want), fp16), fp16)[mask]).all())
 
 
+@pytest.fixture(params=[0, 1], ids=["two_lists", "split_tails"])
+def tile_order(request):
+    """Both tile orders of the ping-pong kernels (MOE_GG_OP_TILE_ORDER) for one test."""
+    L = H.lib()
+    assert L.moe_gg_set_variant(H.OP_TILE_ORDER, request.param) == 0
+    try:
+        yield request.param
+    finally:
+        L.moe_gg_set_variant(H.OP_TILE_ORDER, -1)
+
+
 SIZES = [300, 0, 70, 530]   # a full tile + a low tile, an empty expert, a short one, a tall one whose tail is split
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, -1])
-def test_bf16_every_kernel_variant(variant):
+def test_bf16_every_kernel_variant(variant, tile_order):
     rng = np.random.default_rng(variant + 1)
     x, w = ints(rng, (sum(SIZES), 128)), ints(rng, (4 * 512, 128))
     y = H.grouped_gemm(H.to_bf16(x), H.to_bf16(w), SIZES, 512, variant=variant)
@@ -53,7 +64,7 @@ def test_bf16_every_kernel_variant(variant):
 
 
 @pytest.mark.parametrize("fp16,block", [(True, False), (False, True), (True, True)])
-def test_fp16_and_block_layout(fp16, block):
+def test_fp16_and_block_layout(fp16, block, tile_order):
     rng = np.random.default_rng(7)
     x, w = ints(rng, (sum(SIZES), 128)), ints(rng, (4 * 256, 128))
     y = H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), SIZES, 256, fp16=fp16, block_layout=block)
@@ -72,7 +83,7 @@ def test_small_and_odd_shapes_take_the_decode_and_generic_kernels(sizes, N, K):
 
 
 @pytest.mark.parametrize("sizes", [[530], [520, 30]])
-def test_low_tiles_computed_by_the_small_m_kernel(sizes):
+def test_low_tiles_computed_by_the_small_m_kernel(sizes, tile_order):
     """K >= 8192 with few experts: the ping-pong launch leaves the rows behind the last full tile to a launch of the
     small-M kernel (both decide it from m_sizes on the device)."""
     G, M, N, K = len(sizes), sum(sizes), 256, 8192
@@ -85,7 +96,7 @@ def test_low_tiles_computed_by_the_small_m_kernel(sizes):
 
 @pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, -1])
-def test_fp8_every_kernel_variant(mode, variant):
+def test_fp8_every_kernel_variant(mode, variant, tile_order):
     rng = np.random.default_rng(10 * mode + variant + 3)
     sizes, N, K = [300, 0, 70, 30, 530], 256, 256
     G, M = len(sizes), sum(sizes)
@@ -99,7 +110,7 @@ def test_fp8_every_kernel_variant(mode, variant):
 
 
 @pytest.mark.parametrize("fp16", [False, True])
-def test_fused_silu_and_mul_gemm(fp16):
+def test_fused_silu_and_mul_gemm(fp16, tile_order):
     rng = np.random.default_rng(5)
     n, K = 192, 128
     x = (rng.standard_normal((sum(SIZES), K)) * 0.5).astype(np.float32)
@@ -112,7 +123,7 @@ def test_fused_silu_and_mul_gemm(fp16):
 
 @pytest.mark.parametrize("fp16", [False, True])
 @pytest.mark.parametrize("T,E,k,n,K", [(200, 4, 2, 128, 128), (700, 8, 2, 192, 64), (300, 3, 3, 64, 256), (33, 2, 1, 256, 128)])
-def test_gather_folded_into_the_first_gemm_gives_the_same_bits(fp16, T, E, k, n, K):
+def test_gather_folded_into_the_first_gemm_gives_the_same_bits(fp16, T, E, k, n, K, tile_order):
     """moe_gg_grouped_gemm_swiglu_gather on the token matrix and the permutation against moe_gg_gather_rows followed by
     moe_gg_grouped_gemm_swiglu: bit for bit, with masked slots, and rows beyond sum(m_sizes) left alone."""
     rng = np.random.default_rng(T + n)
@@ -155,7 +166,7 @@ def test_gather_with_a_corrupt_permutation_stays_inside_the_token_matrix():
 @pytest.mark.parametrize("sizes,N,K,block,static", [
     (SIZES, 256, 128, False, False), (SIZES, 256, 128, True, False), (SIZES, 256, 128, False, True),
     ([30, 0, 7, 53], 64, 64, False, False), ([0, 5, 0], 64, 64, False, False), ([300, 200], 68, 36, False, False)])
-def test_backward(sizes, N, K, block, static):
+def test_backward(sizes, N, K, block, static, tile_order):
     rng = np.random.default_rng(N + K)
     G, M = len(sizes), sum(sizes)
     x, w = ints(rng, (M, K), -2, 3), ints(rng, (G * N, K), -2, 3)
@@ -331,7 +342,7 @@ FUZZ = [  # (compute units, load-landing model, wave order seed): few units = lo
 def test_pingpong_random_shapes_over_unit_counts_and_schedules():
     procs = []
     for i, (cus, dma, seed) in enumerate(FUZZ):
-        env = dict(os.environ, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed)
+        env = dict(os.environ, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed, EMU_TILE_ORDER=str(i % 2))
         procs.append(subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_pingpong.py"), str(100 + i), "20"], env=env,
                                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT))
     for cfg, p in zip(FUZZ, procs):
@@ -347,7 +358,7 @@ def test_every_entry_point_on_random_shapes_with_tensors_against_guard_pages():
     tensor, by one element or by one 16-byte load, ends the child process with a memory fault."""
     procs = []
     for i, (guard, cus, dma, seed) in enumerate(GUARDED):
-        env = dict(os.environ, EMU_GUARD=guard, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed, EMU_TRACE="1")
+        env = dict(os.environ, EMU_GUARD=guard, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed, EMU_TRACE="1", EMU_TILE_ORDER=str(i % 2))
         procs.append(subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_all.py"), str(200 + i), "40"], env=env,
                                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT))
     for cfg, p in zip(GUARDED, procs):
@@ -359,9 +370,10 @@ def test_corrupt_m_sizes_are_clamped_by_every_kernel():
     """Negative sizes, sums beyond M, a size of 2^30: every kernel that reads m_sizes (all GEMM variants, fp8, SwiGLU,
     backward, W4A16 grouped) computes the rows of the clamped sizes, leaves the other rows alone and, with every tensor
     against a guard page, touches nothing outside them."""
-    env = dict(os.environ, EMU_GUARD="end", EMU_TRACE="1")
-    p = subprocess.run([sys.executable, os.path.join(EMU, "corrupt_sizes.py")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT)
-    assert p.returncode == 0, p.stdout.decode()[-2000:]
+    for order in ("0", "1"):
+        env = dict(os.environ, EMU_GUARD="end", EMU_TRACE="1", EMU_TILE_ORDER=order)
+        p = subprocess.run([sys.executable, os.path.join(EMU, "corrupt_sizes.py")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT)
+        assert p.returncode == 0, (order, p.stdout.decode()[-2000:])
 
 
 def test_no_data_race_between_the_waves_of_a_workgroup():
@@ -375,16 +387,19 @@ def test_no_data_race_between_the_waves_of_a_workgroup():
         racy = subprocess.run([exe, "selftest", kernel, "0"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
         assert clean.returncode == 0 and b"data race" not in clean.stdout, clean.stdout.decode()[-1500:]
         assert racy.returncode == 66 and b"data race" in racy.stdout, racy.stdout.decode()[-1500:]
-    procs = [subprocess.Popen([exe], env=dict(os.environ, EMU_CUS=cus, EMU_SEED=seed), stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
-             for cus, seed in (("8", "0"), ("2", "7"))]
+    procs = [subprocess.Popen([exe], env=dict(os.environ, EMU_CUS=cus, EMU_SEED=seed, EMU_TILE_ORDER=order), stdout=subprocess.PIPE,
+                              stderr=subprocess.STDOUT)
+             for cus, seed, order in (("8", "0", "0"), ("2", "7", "1"))]
     # long tile sequences in one workgroup: split tails, row pieces of the last round, short and empty experts
     shapes = [("bf16", "512", "128", "1", "0", ["530", "300", "0", "70"]), ("swiglu", "256", "128", "2", "5", ["833", "64", "257"]),
               ("gather", "128", "128", "2", "3", ["530", "1", "300"]),
               ("fp8block", "384", "256", "1", "0", ["577", "33", "320"]), ("fp8row", "256", "128", "3", "9", ["129", "768", "1"]),
               ("f16", "384", "256", "2", "0", ["321", "511"]), ("bwd", "256", "128", "3", "4", ["300", "0", "41", "513"])]
-    for op, N, K, cus, seed, sizes in shapes:
-        procs.append(subprocess.Popen([exe, "shape", op, N, K] + sizes, env=dict(os.environ, EMU_CUS=cus, EMU_SEED=seed),
-                                      stdout=subprocess.PIPE, stderr=subprocess.STDOUT))
+    for i, (op, N, K, cus, seed, sizes) in enumerate(shapes):
+        for order in ("0", "1"):
+            procs.append(subprocess.Popen([exe, "shape", op, N, K] + sizes,
+                                          env=dict(os.environ, EMU_CUS=cus, EMU_SEED=seed, EMU_TILE_ORDER=order),
+                                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT))
     for p in procs:
         log = p.communicate()[0].decode()
         assert p.returncode == 0 and "data race" not in log and " rc 0" in log, log[-3000:]

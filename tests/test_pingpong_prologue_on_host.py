@@ -29,7 +29,7 @@ constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, 
               OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7, OP_F16_SWIGLU = 8, OP_BF16_SWIGLU_GATHER = 9, OP_F16_SWIGLU_GATHER = 10;
 constexpr bool op_gather(int op) { return op == OP_BF16_SWIGLU_GATHER || op == OP_F16_SWIGLU_GATHER; }
 constexpr bool op_swiglu(int op) { return op == OP_BF16_SWIGLU || op == OP_F16_SWIGLU || op_gather(op); }
-struct GgParams { const int32_t* m_sizes; int G, M, N, K, skip_rows, tails_apart, xcds; };
+struct GgParams { const int32_t* m_sizes; int G, M, N, K, skip_rows, tails_apart, xcds, split_tails; };
 struct Dim { int x; };
 static Dim blockIdx, threadIdx, gridDim;
 static int uni(int v) { return v; }
@@ -61,8 +61,8 @@ HARNESS_TAIL = r'''
 }
 
 extern "C" int emu_prologue(int op, const int32_t* m_sizes, int G, int M, int N, int K, int skip_rows, int tails_apart,
-                            int nwg, int xcds, int32_t* out, int cap) {
-  GgParams p{m_sizes, G, M, N, K, skip_rows, tails_apart, xcds};
+                            int nwg, int xcds, int split_tails, int32_t* out, int cap) {
+  GgParams p{m_sizes, G, M, N, K, skip_rows, tails_apart, xcds, split_tails};
   gridDim.x = nwg;
   static int32_t seq[2 * MOE_GG_SEQ_CAP];
   int written = 0;
@@ -105,15 +105,25 @@ def emu(tmp_path_factory):
     subprocess.run(["g++", "-O1", "-std=c++17", "-shared", "-fPIC", "-I", CSRC, "-o", str(so), str(cpp)], check=True)
     lib = ctypes.CDLL(str(so))
     lib.emu_prologue.restype = ctypes.c_int
-    lib.emu_prologue.argtypes = [ctypes.c_int, I32P] + [ctypes.c_int] * 8 + [I32P, ctypes.c_int]
+    lib.emu_prologue.argtypes = [ctypes.c_int, I32P] + [ctypes.c_int] * 9 + [I32P, ctypes.c_int]
     return lib
 
 
-def device_tiles(emu, op, sizes, N, K, nwg, skip=0, tails=0, M=None):
+@pytest.fixture(params=[0, 1], ids=["two_lists", "split_tails"])
+def split(lib, request):
+    """Tile order for one test: the host mirror is pinned to it, the device prologue gets it as p.split_tails."""
+    assert lib.moe_gg_set_variant(2, request.param) == 0     # MOE_GG_OP_TILE_ORDER
+    try:
+        yield request.param
+    finally:
+        lib.moe_gg_set_variant(2, -1)
+
+
+def device_tiles(emu, op, sizes, N, K, nwg, skip=0, tails=0, M=None, split=0):
     ms = np.ascontiguousarray(sizes, dtype=np.int32)
     out = np.zeros((CAP, 6), dtype=np.int32)
     n = emu.emu_prologue(op, ms.ctypes.data_as(I32P), len(ms), int(ms.sum()) if M is None else M, N, K, skip, tails, nwg, 8,
-                         out.ctypes.data_as(I32P), CAP)
+                         split, out.ctypes.data_as(I32P), CAP)
     assert 0 <= n < CAP
     return out[:n]
 
@@ -142,15 +152,15 @@ def shape_sets():
     return cases
 
 
-def test_device_prologue_equals_the_host_mirror(emu, lib):
+def test_device_prologue_equals_the_host_mirror(emu, lib, split):
     for sizes, N, nwg in shape_sets():
         h = host_tiles(lib, sizes, N, 256, nwg)
-        d = device_tiles(emu, 0, sizes, N, 4096, nwg).copy()
+        d = device_tiles(emu, 0, sizes, N, 4096, nwg, split=split).copy()
         assert h.shape == d.shape and (h == d).all(), ("bf16", sizes[:8], N, nwg)
         n_out = max(128, N // 2 // 128 * 128)       # fused gate/up kernel: p.N = 2 n, tiles of 128 output columns
         h = host_tiles(lib, sizes, n_out, 128, nwg)
         for op in (4, 9):   # the fused gate/up kernel and its form with the row gather
-            d = device_tiles(emu, op, sizes, 2 * n_out, 4096, nwg)
+            d = device_tiles(emu, op, sizes, 2 * n_out, 4096, nwg, split=split)
             assert h.shape == d.shape and (h == d).all(), ("swiglu", op, sizes[:8], n_out, nwg)
 
 
@@ -163,14 +173,14 @@ def cover(tiles, sizes, N):
     return c
 
 
-def test_low_tiles_left_to_the_small_m_kernel_are_exactly_the_rows_it_computes(emu, lib):
+def test_low_tiles_left_to_the_small_m_kernel_are_exactly_the_rows_it_computes(emu, lib, split):
     """p.tails_apart set (bf16, K >= 8192, few experts): when the decision (the host mirror's) is 'apart', the table
     holds every row up to each tall expert's last full tile and nothing of the few rows behind it; otherwise all rows."""
     for sizes, N in (([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], 4096), ([1151] + [1024] * 6 + [897], 4096),
                      ([1124] * 4 + [1024] * 4, 4096), ([40, 2008, 2000, 2000, 2048, 0, 48, 48], 4096), ([1039, 700] + [0] * 6, 4096)):
         ms = np.ascontiguousarray(sizes, dtype=np.int32)
         apart = lib.moe_gg_host_tails_apart(ms.ctypes.data_as(I32P), len(ms), int(ms.sum()), N, 14336, 256)
-        c = cover(device_tiles(emu, 0, sizes, N, 14336, 256, tails=256), sizes, N)
+        c = cover(device_tiles(emu, 0, sizes, N, 14336, 256, tails=256, split=split), sizes, N)
         for g, m in enumerate(sizes):
             full, rem = divmod(m, 256)
             low = 0 < rem < 128 and (full >= 2 or full == 0)
@@ -178,22 +188,22 @@ def test_low_tiles_left_to_the_small_m_kernel_are_exactly_the_rows_it_computes(e
             assert (c[g][:keep] == 1).all() and (c[g][keep:] == 0).all(), (sizes, g, apart)
 
 
-def test_fp8_prologue_skips_the_streaming_kernels_experts(emu):
+def test_fp8_prologue_skips_the_streaming_kernels_experts(emu, lib, split):
     rng = np.random.default_rng(9)
     for _ in range(40):
         G = int(rng.integers(1, 60))
         sizes = [int(rng.integers(0, 90)) if rng.random() < 0.5 else int(rng.integers(0, 1400)) for _ in range(G)]
         N, nwg = int(rng.choice([128, 256, 512, 1024, 4096])), int(rng.choice([8, 64, 256]))
         for skip in (0, 64):
-            c = cover(device_tiles(emu, 2, sizes, N, 7168, nwg, skip=skip), sizes, N)
+            c = cover(device_tiles(emu, 2, sizes, N, 7168, nwg, skip=skip, split=split), sizes, N)
             for g, m in enumerate(sizes):
                 assert (c[g] == (0 if m <= skip else 1)).all(), (sizes[:6], g, m, skip)
 
 
-def test_corrupt_sizes_are_clamped_in_the_prologue(emu):
+def test_corrupt_sizes_are_clamped_in_the_prologue(emu, lib, split):
     # a negative entry counts as empty and the running sum is cut at M: no tile starts past its group's rows
     sizes = [300, -5, 700, 90]
-    d = device_tiles(emu, 0, sizes, 512, 4096, 16, M=800)
+    d = device_tiles(emu, 0, sizes, 512, 4096, 16, M=800, split=split)
     eff = [300, 0, 500, 0]
     c = [np.zeros((m, 2), dtype=np.int32) for m in eff]
     for wg, g, m0, h, n0, nc in d.tolist():
