@@ -1,11 +1,16 @@
 """Benchmark of the MoE grouped-GEMM hot path on one MI355X.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu-baseline] [--no-moe-sweep]
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu-baseline] [--moe-sweep] [--budget-s S]
 
 A step is one pass of the hot path over one batch of synthetic, HBM-resident input. The headline workload is the
 configuration the metric is quoted on: Mixtral 8x7B w1 grouped GEMM, bf16, T=4096 tokens top-2 (8192 expert-sorted
 rows), K=4096, N=14336, 8 experts. Prints ONE JSON line; the other benchmark configurations (decode, W4A16, fp8)
 are measured in the same run and reported under "secondary" with their own rooflines.
+
+Order of work: every GPU measurement first (headline, the vendor library's dense GEMM, the secondary workloads), then
+the CPU baselines (headline first). A wall-clock budget (--budget-s, default 480 s) is checked before every secondary
+workload and every CPU baseline; what does not fit is reported as {"skipped": "time budget"}, so the line is printed
+within minutes whatever the host's speed. SIGTERM / SIGINT print the line with what has been measured so far.
 """
 import argparse
 import ctypes
@@ -35,6 +40,23 @@ def load_traffic():
 
 
 TRAFFIC, TRAFFIC_COMMIT = load_traffic()
+
+
+class Budget:
+    """Wall-clock budget of the whole run, started when main() starts."""
+
+    def __init__(self, seconds):
+        self.t0 = time.perf_counter()
+        self.seconds = float(seconds)
+
+    def elapsed(self):
+        return time.perf_counter() - self.t0
+
+    def spent(self):
+        return self.elapsed() >= self.seconds
+
+
+SKIPPED = {"skipped": "time budget"}
 
 
 def cpu_info():
@@ -140,14 +162,14 @@ def cpu_baseline_w4a16(M, K, N):
             "sample": "the whole workload, dequantisation inside the timed region + torch.matmul, 1 warm-up + 3 repetitions, median"}
 
 
-def cpu_baseline_fp8_block(xq, wq, xs, ws, m_sizes, N, K, n_experts=32):
+def cpu_baseline_fp8_block(xq, wq, xs, ws, m_sizes, N, K, n_experts=32, defer=False):
     """Config 5 on the host cores: the first `n_experts` non-empty experts (the most popular ones under the Zipf
     routing come first), dequantisation with the block scales inside the timed per-expert loop, scaled to the whole
-    workload by FLOPs. xq / wq / xs / ws are the GPU tensors of the timed launch; only the sample is copied."""
+    workload by FLOPs. xq / wq / xs / ws are the GPU tensors of the timed launch; only the sample is copied. With
+    defer the copy is made now and a function is returned that does the timing later (the GPU tensors can be freed)."""
     import torch
     from oracle import oracle as O
 
-    threads = cpu_threads()
     sizes = [int(m) for m in m_sizes]
     take, seen = 0, 0
     for m in sizes:
@@ -161,14 +183,102 @@ def cpu_baseline_fp8_block(xq, wq, xs, ws, m_sizes, N, K, n_experts=32):
     xs_h = xs[:rows].cpu()
     wq_h = wq[:take * N].view(torch.uint8).cpu()
     ws_h = ws[:take * N // 128].cpu()
-    t = cpu_median_seconds(lambda: O.grouped_gemm_fp8_block_torch_loop(xq_h, wq_h, xs_h, ws_h, sample, N))
-    flop_sample = 2.0 * rows * N * K
-    flop_all = 2.0 * sum(sizes) * N * K
+
+    def timed():
+        threads = cpu_threads()
+        t = cpu_median_seconds(lambda: O.grouped_gemm_fp8_block_torch_loop(xq_h, wq_h, xs_h, ws_h, sample, N))
+        flop_sample = 2.0 * rows * N * K
+        flop_all = 2.0 * sum(sizes) * N * K
+        return {"value": round(flop_sample / t / 1e12, 3), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "seconds": round(t, 3), "extrapolated": True,
+                "seconds_whole_workload_by_flops": round(t * flop_all / flop_sample, 3),
+                "sample": f"first {seen} non-empty experts of {len(sizes)} ({rows} of {sum(sizes)} rows, {100.0 * flop_sample / flop_all:.0f} % of the FLOPs), "
+                          "per-expert dequantise + torch.matmul, 1 warm-up + 3 repetitions, median"}
+
+    return timed if defer else timed()
+
+
+def cpu_baseline_w4a16_grouped(m_sizes, K, N, n_experts=2):
+    """The grouped W4A16 call on the host cores: the first `n_experts` experts that have rows, dequantisation inside
+    the timed per-expert loop, scaled to all experts with rows by the weight bytes they stream."""
+    import torch
+    from oracle import oracle as O
+
+    threads = cpu_threads()
+    sizes = [int(m) for m in m_sizes]
+    take, seen = 0, 0
+    for m in sizes:
+        if seen == n_experts:
+            break
+        take += 1
+        seen += m > 0
+    sample = sizes[:take]
+    active = sum(1 for m in sizes if m > 0)
+    gen = torch.Generator().manual_seed(5)
+    qw = torch.randint(-2**31, 2**31 - 1, (take, K // 8, N), dtype=torch.int32, generator=gen)
+    sc = torch.rand(take, K // 128, N, generator=gen) * 0.015 + 0.005
+    qz = torch.randint(-2**31, 2**31 - 1, (take, K // 128, N // 8), dtype=torch.int32, generator=gen)
+    a = torch.randn(sum(sample), K, generator=gen)
+    t = cpu_median_seconds(lambda: O.w4a16_grouped_torch_loop(a, qw, sc, qz, sample, 128, 0))
+    per_expert = K * N // 2 + (K // 128) * N * 2 + (K // 128) * N // 2
+    byt = seen * per_expert + sum(sample) * (K + N) * 2
+    return {"value": round(byt / t / 1e9, 3), "unit": "GB/s", "bytes": "the GPU path's algorithmic bytes", "cores": threads,
+            "kind": "port", "seconds": round(t, 4), "extrapolated": True,
+            "seconds_whole_workload_by_bytes": round(t * active / max(seen, 1), 4),
+            "sample": f"first {seen} of the {active} experts that have rows, per-expert dequantise + torch.matmul, "
+                      "1 warm-up + 3 repetitions, median"}
+
+
+def cpu_baseline_moe_layer(T, K, n, E, topk, sample_tokens=1024):
+    """The MoE layer on the host cores as the reference's torch_moe states it (test_moe_gemm.py:16-30; per-expert fp32
+    torch.matmul loop): the first `sample_tokens` tokens against all experts' weights, scaled to T tokens by FLOPs."""
+    import torch
+    from oracle import oracle as O
+
+    threads = cpu_threads()
+    Ts = min(T, sample_tokens)
+    gen = torch.Generator().manual_seed(6)
+    a = torch.randn(Ts, K, generator=gen) / 10
+    w1 = torch.empty(E, 2 * n, K)
+    w2 = torch.empty(E, K, n)
+    b1 = torch.randn(2 * n, K, generator=gen) * 0.02     # one draw, a distinct scaled copy per expert: timing only
+    b2 = torch.randn(K, n, generator=gen) * 0.02
+    for ex in range(E):
+        torch.mul(b1, 1.0 + 0.01 * ex, out=w1[ex])
+        torch.mul(b2, 1.0 + 0.01 * ex, out=w2[ex])
+    del b1, b2
+    score = torch.softmax(torch.randn(Ts, E, generator=gen), dim=-1)
+    tw, ids = torch.topk(score, topk)
+    t = cpu_median_seconds(lambda: O.fused_moe_torch(a, w1, w2, tw, ids))
+    flop_sample = 2.0 * Ts * topk * (2 * n * K + K * n)
     return {"value": round(flop_sample / t / 1e12, 3), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "seconds": round(t, 3), "extrapolated": True,
+            "seconds": round(t, 3), "extrapolated": Ts < T, "seconds_whole_workload_by_flops": round(t * T / Ts, 3),
+            "sample": f"{Ts} of {T} tokens through all {E} experts (per-expert fp32 torch.matmul loop, SiLU-and-mul and "
+                      "top-k combine in torch), 1 warm-up + 3 repetitions, median"}
+
+
+def cpu_baseline_backward(m_sizes, N, K, n_experts=2):
+    """Both gradients on the host cores (per-expert fp32 torch.matmul loop, pytorch_reference_backwards.py:165-197):
+    the first `n_experts` experts, scaled to the whole workload by FLOPs."""
+    import torch
+    from oracle import oracle as O
+
+    threads = cpu_threads()
+    sizes = [int(m) for m in m_sizes]
+    sample = sizes[:n_experts]
+    rows = sum(sample)
+    gen = torch.Generator().manual_seed(7)
+    x = torch.randn(rows, K, generator=gen) / 8
+    w = torch.randn(len(sample) * N, K, generator=gen) * 0.02
+    go = torch.randn(rows, N, generator=gen) / 8
+    t = cpu_median_seconds(lambda: O.grouped_gemm_backward_torch_loop(go, x, w, sample))
+    flop_sample = 4.0 * rows * N * K
+    flop_all = 4.0 * sum(sizes) * N * K
+    return {"value": round(flop_sample / t / 1e12, 3), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "seconds": round(t, 3), "extrapolated": len(sample) < len(sizes),
             "seconds_whole_workload_by_flops": round(t * flop_all / flop_sample, 3),
-            "sample": f"first {seen} non-empty experts of {len(sizes)} ({rows} of {sum(sizes)} rows, {100.0 * flop_sample / flop_all:.0f} % of the FLOPs), "
-                      "per-expert dequantise + torch.matmul, 1 warm-up + 3 repetitions, median"}
+            "sample": f"first {len(sample)} experts of {len(sizes)} ({rows} of {sum(sizes)} rows), grad_x and grad_w by "
+                      "per-expert fp32 torch.matmul, 1 warm-up + 3 repetitions, median"}
 
 
 # After a change of load the GPU's power management overshoots and settles again: the first launch of the prefill
@@ -263,7 +373,7 @@ def wl_decode(torch, A, dev, lib, stream, cpu):
         e.update({"value": round(byt / ms / 1e6, 1), "unit": "GB/s", "roofline": hbm_roofline("gg_bf16_decode", byt, ms, key)})
         del ws
         if cpu:
-            e["cpu_baseline"] = cpu_baseline_decode(m_sizes, K, N)
+            e["_cpu"] = lambda m_sizes=m_sizes, K=K, N=N: cpu_baseline_decode(m_sizes, K, N)
         out.append(e)
     return out
 
@@ -297,7 +407,7 @@ def wl_w4a16(torch, A, dev, lib, stream, cpu):
         e.update({"cache_hot_us_per_launch": round(ms_hot * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
                   "roofline": hbm_roofline("w4a16_splitk_g128", byt, ms, f"w4a16_m{M}")})
         if cpu:
-            e["cpu_baseline"] = cpu_baseline_w4a16(M, K, N)
+            e["_cpu"] = lambda M=M: cpu_baseline_w4a16(M, K, N)
         out.append(e)
     return out
 
@@ -330,6 +440,9 @@ def wl_w4a16_grouped(torch, A, dev, lib, stream, cpu):
     e.update(timing_fields(st, "us"))
     e.update({"value": round(byt / ms / 1e6, 1), "unit": "GB/s",
               "roofline": hbm_roofline("w4a16_splitk_g128 (grid.y = experts)", byt, ms, "w4a16_grouped")})
+    if cpu:
+        sizes3 = c3["m_sizes"].tolist()
+        e["_cpu"] = lambda: cpu_baseline_w4a16_grouped(sizes3, K, N)
     out.append(e)
 
     # the same call with the 1 x 128 fp8 quantiser as its epilogue, beside the two launches it replaces
@@ -393,7 +506,7 @@ def wl_fp8_cfg5(torch, A, dev, lib, stream, cpu):
     e.update({"value": round(byt / ms / 1e6, 1), "unit": "GB/s", "tflops": round(flop / ms / 1e9, 1),
               "roofline": hbm_roofline("gg_fp8_pingpong_block", byt, ms, "fp8_block_cfg5")})
     if cpu:
-        e["cpu_baseline"] = cpu_baseline_fp8_block(xq, wq, xs, ws, m5.tolist(), N, K)
+        e["_cpu"] = cpu_baseline_fp8_block(xq, wq, xs, ws, m5.tolist(), N, K, defer=True)
     return [e]
 
 
@@ -419,6 +532,8 @@ def wl_moe_layer(torch, A, dev, lib, stream, cpu):
               "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong (two launches) + glue kernels", "achieved": round(flop / ms / 1e9, 1),
                            "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
                            "traffic": None}})
+    if cpu:
+        e["_cpu"] = lambda: cpu_baseline_moe_layer(T, K, n, E, topk)
     return [e]
 
 
@@ -449,6 +564,9 @@ def wl_backward(torch, A, dev, lib, stream, cpu):
               "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong_nt + gg_bf16_pingpong_wgrad_direct",
                            "achieved": round(flop / ms / 1e9, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None}})
+    if cpu:
+        sizes = ms_dev.tolist()
+        e["_cpu"] = lambda: cpu_baseline_backward(sizes, N, K)
     return [e]
 
 
@@ -476,21 +594,57 @@ def wl_moe_sweep(torch, A, dev, lib, stream, cpu):
 
 
 SECONDARY = (wl_decode, wl_w4a16, wl_w4a16_grouped, wl_fp8_cfg5, wl_moe_layer, wl_backward)
-# Context entries (left out with --no-moe-sweep).
+# Context entries (only with --moe-sweep).
 OPTIONAL = (wl_moe_sweep,)
 
 
-def secondary_workloads(torch, A, dev, cpu=True, optional=False):
+def secondary_workloads(torch, A, dev, cpu=True, optional=False, budget=None, out=None):
+    """The GPU legs of the secondary workloads, appended to `out` as they finish. With cpu, an entry may carry its CPU
+    baseline as a function under "_cpu": run_cpu_baselines() calls it once every GPU leg is done."""
     lib = A._lib.lib()
     stream = torch.cuda.current_stream().cuda_stream
-    out = []
+    out = [] if out is None else out
     for wl in SECONDARY + (OPTIONAL if optional else ()):
+        if budget is not None and budget.spent():
+            out.append({"workload": wl.__name__, **SKIPPED})
+            continue
         try:
             out.extend(wl(torch, A, dev, lib, stream, cpu))
         except Exception as exc:  # one workload failing must not lose the line
             out.append({"workload": wl.__name__, "error": f"{type(exc).__name__}: {exc}"})
         torch.cuda.empty_cache()
     return out
+
+
+def run_cpu_baselines(entries, budget=None):
+    """Replaces the "_cpu" function of every entry by its result under "cpu_baseline", in order; once the budget is
+    spent the remaining ones are marked skipped."""
+    for e in entries:
+        fn = e.pop("_cpu", None)
+        if fn is None:
+            continue
+        if budget is not None and budget.spent():
+            e["cpu_baseline"] = dict(SKIPPED)
+            continue
+        try:
+            e["cpu_baseline"] = fn()
+        except Exception as exc:
+            e["cpu_baseline"] = {"error": f"{type(exc).__name__}: {exc}"}
+
+
+def printable(out):
+    """The JSON line for `out`: baselines that have not run yet are marked as such."""
+    def clean(e):
+        if isinstance(e, dict):
+            d = {k: clean(v) for k, v in e.items() if k != "_cpu"}
+            if "_cpu" in e:
+                d["cpu_baseline"] = {"skipped": "interrupted before it ran"}
+            return d
+        if isinstance(e, list):
+            return [clean(v) for v in e]
+        return e
+
+    return json.dumps(clean(out))
 
 
 def main():
@@ -500,18 +654,36 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true")
-    ap.add_argument("--no-moe-sweep", action="store_true",
-                    help="skip the fused_moe sweep over m = 1 ... 512 (the shape of the reference's published sweep; context only)")
+    ap.add_argument("--moe-sweep", action="store_true",
+                    help="also run the fused_moe sweep over m = 1 ... 512 (the shape of the reference's published sweep; context only)")
+    ap.add_argument("--no-moe-sweep", action="store_true", help="accepted for compatibility: the sweep is off unless --moe-sweep is given")
+    ap.add_argument("--budget-s", type=float, default=480.0,
+                    help="wall-clock budget: secondary workloads and CPU baselines that would start after it are reported as skipped")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, so that a rocprofv3 --pmc run of this command sees a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
+    budget = Budget(args.budget_s)
+
+    import signal
+
     import torch
 
     import applied_ai_amd as A
     from applied_ai_amd import configs
+
+    out = {}
+
+    def on_signal(signum, frame):  # a driver's time limit: print what has been measured, then leave
+        if out:
+            out["interrupted_by_signal"] = signum
+            print(printable(out), flush=True)
+        os._exit(128 + signum)
+
+    signal.signal(signal.SIGTERM, on_signal)
+    signal.signal(signal.SIGINT, on_signal)
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -546,7 +718,7 @@ def main():
     value = flop / (ms_per_step * 1e-3) / 1e12
     achieved = flop / (avg_kernel_ms * 1e-3) / 1e12
 
-    out = {
+    out.update({
         "metric": "grouped-GEMM TFLOP/s + % MFMA peak, Mixtral 8x7B bf16 T=4096 top-2",
         "value": round(value, 2),
         "unit": "TFLOP/s",
@@ -576,7 +748,7 @@ def main():
             "kernel_ms": {"avg": round(avg_kernel_ms, 4), "p20": round(kern_ms[len(kern_ms) // 5], 4),
                           "p50": round(kern_ms[len(kern_ms) // 2], 4), "p80": round(kern_ms[(len(kern_ms) * 4) // 5], 4)},
         },
-    }
+    })
     # Context for the roofline fraction: the vendor library's dense bf16 GEMM of the same FLOP count and data
     # (one [8192, 4096] x [4096, 14336] product through torch.matmul -> hipBLASLt), timed the same way. With
     # random operands the MFMA clock is power-limited well below the 2.5 PFLOP/s figure, for the library too.
@@ -596,14 +768,17 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     out["traffic_measured_at"] = TRAFFIC_COMMIT
-    if not args.no_cpu_baseline:
-        try:
-            out["cpu_baseline"] = cpu_baseline_prefill(c)
-        except Exception as exc:
-            out["cpu_baseline"] = {"error": f"{type(exc).__name__}: {exc}"}
+    cpu = not args.no_cpu_baseline
+    if cpu:
+        out["_cpu"] = lambda: cpu_baseline_prefill(c)
     if not args.no_secondary:
-        out["secondary"] = secondary_workloads(torch, A, dev, cpu=not args.no_cpu_baseline, optional=not args.no_moe_sweep)
-    print(json.dumps(out))
+        out["secondary"] = []
+        secondary_workloads(torch, A, dev, cpu=cpu, optional=args.moe_sweep, budget=budget, out=out["secondary"])
+    # every GPU number is in `out` now: the CPU baselines follow, the headline's first
+    run_cpu_baselines([out] + out.get("secondary", []), budget)
+    out["wall_s"] = round(budget.elapsed(), 1)
+    out["budget_s"] = args.budget_s
+    print(printable(out))
 
 
 if __name__ == "__main__":

@@ -231,6 +231,48 @@ def grouped_gemm_torch_loop(x, w, m_sizes):
     return y
 
 
+def grouped_gemm_backward_torch_loop(grad_output, x, w, m_sizes):
+    """Both gradients of the grouped GEMM as a per-expert loop of fp32 torch matmuls on the host cores
+    (grad_x_g = dY_g @ w_g, grad_w_g = dY_g^T @ x_g; kernels/MoE/group_GEMM/triton/testing/
+    pytorch_reference_backwards.py:165-197). grad_output [M, N], x [M, K], w [G*N, K] float tensors; only the experts
+    listed in m_sizes are computed (a prefix of all experts is allowed). bench.py times it as the CPU baseline of the
+    backward workload; tests check it against the scalar C form."""
+    import torch
+
+    G = len(m_sizes)
+    N = grad_output.shape[1]
+    K = x.shape[1]
+    rows = int(sum(int(m) for m in m_sizes))
+    gx = torch.zeros((rows, K), dtype=torch.float32)
+    gw = torch.zeros((G * N, K), dtype=torch.float32)
+    start = 0
+    for g in range(G):
+        m = int(m_sizes[g])
+        if m > 0:
+            dy = grad_output[start:start + m]
+            gx[start:start + m] = dy @ w[g * N:(g + 1) * N]
+            gw[g * N:(g + 1) * N] = dy.T @ x[start:start + m]
+        start += m
+    return gx, gw
+
+
+def w4a16_grouped_torch_loop(a, qweight, scales, qzeros, m_sizes, group_size=128, zero_offset=1):
+    """Per-expert W4A16 product over expert-sorted rows on the host cores: w4a16_torch (dequantisation included) for
+    every expert of m_sizes that has rows (the GEMM of gptq/mixtral/w4a16_fused_dequant_gemm.py:49-149). qweight
+    [E', K/8, N], scales [E', K/g, N], qzeros [E', K/g, N/8] with E' >= len(m_sizes). fp32 tensor out [sum m, N]."""
+    import torch
+
+    rows = int(sum(int(m) for m in m_sizes))
+    out = torch.zeros((rows, qweight.shape[2]), dtype=torch.float32)
+    start = 0
+    for e, m in enumerate(m_sizes):
+        m = int(m)
+        if m > 0:
+            out[start:start + m] = w4a16_torch(a[start:start + m], qweight[e], scales[e], qzeros[e], group_size, zero_offset)
+        start += m
+    return out
+
+
 def w4a16_torch(a, qweight, scales, qzeros, group_size=128, zero_offset=1):
     """W4A16 on the host cores the way the reference's path states it: dequantise the GPTQ-packed weights with the
     closed form of kernels/triton/inference/gptq/splitk_dequant_gemm.py:56-77 (vectorised torch ops, fp32), then

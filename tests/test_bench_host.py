@@ -88,3 +88,90 @@ def test_a_failing_secondary_workload_is_reported_not_raised(monkeypatch):
     t.cuda.current_stream = lambda: types.SimpleNamespace(cuda_stream=0)
     out = bench.secondary_workloads(t, fake_a, torch.device("cpu"))
     assert out == [{"workload": "boom", "error": "RuntimeError: no device"}]
+
+
+def test_cpu_baselines_run_after_the_gpu_legs_and_stop_at_the_budget():
+    order = []
+    entries = [{"workload": "a", "_cpu": lambda: order.append("a") or {"value": 1}},
+               {"workload": "b"},
+               {"workload": "c", "_cpu": lambda: 1 / 0},
+               {"workload": "d", "_cpu": lambda: order.append("d") or {"value": 4}}]
+    bench.run_cpu_baselines(entries, bench.Budget(1000.0))
+    assert order == ["a", "d"] and entries[0]["cpu_baseline"] == {"value": 1} and "cpu_baseline" not in entries[1]
+    assert entries[2]["cpu_baseline"]["error"].startswith("ZeroDivisionError")
+    assert all("_cpu" not in e for e in entries)
+    # a spent budget: nothing runs, every pending baseline is marked
+    late = [{"workload": "x", "_cpu": lambda: order.append("x")}]
+    bench.run_cpu_baselines(late, bench.Budget(0.0))
+    assert late == [{"workload": "x", "cpu_baseline": {"skipped": "time budget"}}] and "x" not in order
+    # and the secondary GPU legs are not started either
+    fake_a = types.SimpleNamespace(_lib=types.SimpleNamespace(lib=lambda: None))
+    t = _Torch()
+    t.cuda.current_stream = lambda: types.SimpleNamespace(cuda_stream=0)
+    out = bench.secondary_workloads(t, fake_a, torch.device("cpu"), budget=bench.Budget(0.0))
+    assert [e["workload"] for e in out] == [w.__name__ for w in bench.SECONDARY] and all(e["skipped"] == "time budget" for e in out)
+
+
+def test_the_line_printed_on_a_signal_marks_baselines_that_have_not_run():
+    out = {"value": 1.0, "_cpu": lambda: None, "secondary": [{"workload": "w", "_cpu": lambda: None}, {"workload": "v", "cpu_baseline": {"value": 2}}]}
+    d = json.loads(bench.printable(out))
+    assert d["cpu_baseline"] == {"skipped": "interrupted before it ran"} and d["secondary"][0]["cpu_baseline"]["skipped"]
+    assert d["secondary"][1]["cpu_baseline"] == {"value": 2} and "_cpu" in out      # the original is untouched
+
+
+def test_new_cpu_baselines_on_small_shapes():
+    b = bench.cpu_baseline_w4a16_grouped([3, 0, 5, 2], 256, 128, n_experts=2)
+    assert b["unit"] == "GB/s" and b["extrapolated"] is True and "first 2 of the 3 experts" in b["sample"]
+    assert b["seconds_whole_workload_by_bytes"] >= b["seconds"]
+    b = bench.cpu_baseline_moe_layer(64, 128, 64, 4, 2, sample_tokens=16)
+    assert b["unit"] == "TFLOP/s" and b["extrapolated"] is True and "16 of 64 tokens" in b["sample"]
+    b = bench.cpu_baseline_backward([5, 0, 7, 4], 64, 128, n_experts=2)
+    assert b["extrapolated"] is True and "first 2 experts of 4 (5 of 16 rows)" in b["sample"]
+
+
+def test_main_prints_one_line_with_the_gpu_numbers_first(monkeypatch, capsys):
+    """main() end to end with the device stubbed (CPU tensors, host-clock events, a stand-in for the GEMM): the flow of
+    the run - GPU legs, then CPU baselines, one JSON line with the fields the contract names."""
+    import sys
+
+    import applied_ai_amd as A
+    from applied_ai_amd import configs
+
+    import signal
+
+    monkeypatch.setattr(signal, "signal", lambda *a: None)       # main() installs handlers: not in the test process
+    monkeypatch.setattr(bench, "SETTLE_SECONDS", 0.0)
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--steps", "3", "--warmup", "1"])
+    monkeypatch.setattr(torch.cuda, "is_available", lambda: True)
+    monkeypatch.setattr(torch.cuda, "set_device", lambda d: None)
+    monkeypatch.setattr(torch.cuda, "synchronize", lambda *a: None)
+    monkeypatch.setattr(torch.cuda, "Event", _Event)
+    monkeypatch.setattr(torch.cuda, "empty_cache", lambda: None)
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda *a: types.SimpleNamespace(cuda_stream=0))
+    real_device = torch.device
+    monkeypatch.setattr(torch, "device", lambda *a: real_device("cpu"))
+    G, N, K, M = 2, 64, 32, 24
+    small = {"x_sorted": torch.zeros(M, K, dtype=torch.bfloat16), "w": torch.zeros(G * N, K, dtype=torch.bfloat16),
+             "m_sizes": torch.tensor([10, 14], dtype=torch.int32)}
+    monkeypatch.setattr(configs, "cfg2", lambda: small)
+    monkeypatch.setattr(A, "grouped_gemm", lambda x, w, ms: torch.zeros(x.shape[0], w.shape[0] // ms.shape[0]))
+    seen = []
+
+    def wl(torch_, A_, dev, lib, stream, cpu):
+        seen.append("gpu leg")
+        return [{"workload": "w", "value": 1.0, "_cpu": lambda: seen.append("cpu leg") or {"value": 0.5}}]
+
+    monkeypatch.setattr(bench, "SECONDARY", (wl,))
+    monkeypatch.setattr(A._lib, "lib", lambda: None)
+    monkeypatch.setattr(bench, "cpu_baseline_prefill", lambda c: seen.append("headline cpu") or {"value": 0.1, "cores": 1})
+    bench.main()
+    lines = [ln for ln in capsys.readouterr().out.splitlines() if ln.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    assert seen == ["gpu leg", "headline cpu", "cpu leg"]
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline", "secondary", "wall_s"):
+        assert key in d, key
+    assert d["steps"] == 3 and d["n_gpus"] == 1 and d["vs_baseline"] is None and d["config"]["m_sizes"] == [10, 14]
+    assert d["roofline"]["bound"] == "mfma" and d["cpu_baseline"] == {"value": 0.1, "cores": 1}
+    assert d["secondary"] == [{"workload": "w", "value": 1.0, "cpu_baseline": {"value": 0.5}}]

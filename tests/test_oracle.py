@@ -536,3 +536,36 @@ def test_fp8_block_torch_loop_equals_the_c_form():
     got2 = O.grouped_gemm_fp8_block_torch_loop(torch.from_numpy(xq), torch.from_numpy(wq), torch.from_numpy(xs),
                                                torch.from_numpy(ws), m_sizes[:1], N)
     np.testing.assert_allclose(got2.numpy(), ref[:4], rtol=1e-4, atol=1e-5)
+
+
+def test_backward_torch_loop_equals_the_c_form():
+    rng = np.random.default_rng(33)
+    G, N, K = 3, 24, 40
+    m_sizes = [5, 0, 7]
+    M = sum(m_sizes)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = rng.standard_normal((G * N, K)).astype(np.float32)
+    go = rng.standard_normal((M, N)).astype(np.float32)
+    gx, gw = O.grouped_gemm_backward(go, x, w, m_sizes)
+    tx, tw = O.grouped_gemm_backward_torch_loop(torch.from_numpy(go), torch.from_numpy(x), torch.from_numpy(w), m_sizes)
+    np.testing.assert_allclose(tx.numpy(), gx, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(tw.numpy(), gw, rtol=1e-4, atol=1e-4)
+    # a prefix of the experts (the bounded baseline sample): their rows and weight gradients only
+    tx1, tw1 = O.grouped_gemm_backward_torch_loop(torch.from_numpy(go), torch.from_numpy(x), torch.from_numpy(w), m_sizes[:1])
+    np.testing.assert_allclose(tx1.numpy(), gx[:5], rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(tw1.numpy(), gw[:N], rtol=1e-4, atol=1e-4)
+
+
+def test_w4a16_grouped_torch_loop_equals_the_c_form():
+    rng = np.random.default_rng(34)
+    E, K, N, g = 3, 256, 64, 128
+    m_sizes = [4, 0, 3]
+    q = rng.integers(0, 16, size=(E, K, N)).astype(np.uint8)
+    z = rng.integers(0, 16, size=(E, K // g, N)).astype(np.uint8)
+    sc = rng.uniform(0.005, 0.02, size=(E, K // g, N)).astype(np.float32)
+    a = rng.standard_normal((sum(m_sizes), K)).astype(np.float32)
+    qw = np.stack([O.pack_int4_along_k(q[e]) for e in range(E)])
+    qz = np.stack([O.pack_int4_along_n(z[e]) for e in range(E)])
+    ref = O.w4a16_grouped(a, qw, sc, qz, m_sizes, g, 0)
+    got = O.w4a16_grouped_torch_loop(torch.from_numpy(a), torch.from_numpy(qw), torch.from_numpy(sc), torch.from_numpy(qz), m_sizes, g, 0)
+    np.testing.assert_allclose(got.numpy(), ref, rtol=1e-4, atol=1e-4)
