@@ -28,7 +28,13 @@ int current_device_info(const DeviceInfo** out) {
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return;
     g_dev[dev].cus = prop.multiProcessorCount;
-    g_dev[dev].xcds = 8;  // MI355X: 8 XCDs x 32 CUs, workgroups dealt round-robin over XCDs
+    // Workgroups are dealt round-robin over the XCDs (MI355X: 8 XCDs x 32 CUs); a partitioned device reports fewer.
+    int xccs = 0;
+    if (hipDeviceGetAttribute(&xccs, hipDeviceAttributeNumberOfXccs, dev) != hipSuccess) {
+      (void)hipGetLastError();  // not a launch error: do not leave it for the next hipGetLastError()
+      xccs = 0;
+    }
+    g_dev[dev].xcds = (xccs >= 1 && xccs <= 16) ? xccs : 8;
     g_dev[dev].ok = prop.multiProcessorCount > 0;
   });
   if (!g_dev[dev].ok) return MOE_GG_EDEVICE;

@@ -8,6 +8,7 @@
 // is what the execution mask does on the GPU.
 //
 // Environment: EMU_CUS   number of compute units hipGetDeviceProperties reports (default 8)
+//              EMU_XCDS  number of XCDs hipDeviceGetAttribute reports (default 8)
 //              EMU_DMA   "late" (default): a global->LDS load writes LDS when its wave's counter wait retires it,
 //                        the latest moment the hardware allows; "early": at issue, the earliest
 //              EMU_SEED  non-zero: fibers are resumed in a shuffled order (changes which wave runs ahead)
@@ -554,6 +555,12 @@ int cvt_pk_fp8_f32(float a, float b, int old, bool hi) {
 hipError_t hipGetDeviceProperties(hipDeviceProp_t* p, int) {
   const char* c = getenv("EMU_CUS");
   p->multiProcessorCount = c ? atoi(c) : 8;
+  return hipSuccess;
+}
+
+hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t, int) {
+  const char* c = getenv("EMU_XCDS");
+  *value = c ? atoi(c) : 8;
   return hipSuccess;
 }
 

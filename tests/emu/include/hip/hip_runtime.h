@@ -87,6 +87,8 @@ inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
 inline const char* hipGetErrorString(hipError_t) { return "emulated HIP error"; }
 hipError_t hipGetDeviceProperties(hipDeviceProp_t* p, int dev);
+enum hipDeviceAttribute_t { hipDeviceAttributeNumberOfXccs };
+hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t attr, int dev);
 template <class T> inline hipError_t hipGetSymbolAddress(void** p, T* sym) { *p = (void*)sym; return hipSuccess; }
 
 inline void __syncthreads() { emu::syncthreads(); }
