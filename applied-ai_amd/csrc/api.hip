@@ -42,6 +42,12 @@ int current_device_info(const DeviceInfo** out) {
   return MOE_GG_OK;
 }
 
+// Variant bits of the W4A16 kernels (MOE_GG_OP_W4A16): 0 unless pinned.
+int w4_variant() {
+  const int v = g_variant[MOE_GG_OP_W4A16].load();
+  return v < 0 ? 0 : v & 3;
+}
+
 // Tile order of the forward ping-pong kernels (MOE_GG_OP_TILE_ORDER): the split-tail order only when it is pinned.
 int split_tails_on() { return g_variant[MOE_GG_OP_TILE_ORDER].load() == MOE_GG_ORDER_SPLIT_TAILS ? 1 : 0; }
 
@@ -267,7 +273,7 @@ int moe_gg_w4a16_splitk(const void* a, const int32_t* qweight, const void* scale
   int rc = current_device_info(&di);
   if (rc != MOE_GG_OK) return rc;
   W4Params p{a, qweight, scales, qzeros, c, M, N, K, group_size, zero_offset};
-  return (int)w4a16_splitk_launch(p, dtype == MOE_GG_DTYPE_FP16, (hipStream_t)stream);
+  return (int)w4a16_splitk_launch(p, dtype == MOE_GG_DTYPE_FP16, w4_variant(), (hipStream_t)stream);
 }
 
 static int w4a16_grouped_any(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros, void* c,
@@ -292,7 +298,7 @@ static int w4a16_grouped_any(const void* a, const int32_t* qweight, const void* 
     p.cq = c_q;
     p.cscale = c_scale;
   }
-  return (int)w4a16_splitk_launch(p, dtype == MOE_GG_DTYPE_FP16, (hipStream_t)stream);
+  return (int)w4a16_splitk_launch(p, dtype == MOE_GG_DTYPE_FP16, w4_variant(), (hipStream_t)stream);
 }
 
 int moe_gg_w4a16_grouped(const void* a, const int32_t* qweight, const void* scales, const int32_t* qzeros, void* c,

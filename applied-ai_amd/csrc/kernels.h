@@ -72,7 +72,11 @@ struct W4Params {
   void* cq = nullptr;
   float* cscale = nullptr;
 };
-hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream);
+// variant: bits of MOE_GG_OP_W4A16's variant (0 = the kernels chosen by default), group size 128 and 16-bit output only:
+// 1: more than 32 rows (per expert, on average): passes of four activation fragments on four waves;
+// 2: up to 16 rows: two extra waves per workgroup that request every line of its weight strip ahead of the
+//    consumer waves, and lanes of activation rows that do not exist issue no loads.
+hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, int variant, hipStream_t stream);
 
 // fp8 e4m3 grouped GEMM (gg_fp8.hip). scale_mode 0: x_scale [M], w_scale [G*N]; 1: x_scale [M, K/128],
 // w_scale [G*N/128, K/128]. Needs K % 128 == 0 (and N % 128 == 0 in block mode), 16-byte aligned x, w.

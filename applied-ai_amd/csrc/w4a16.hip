@@ -144,13 +144,13 @@ DEVINL W4View w4_view(const W4Params& p) {
 // wave (two per lane) and quantises them as fp8_groupwise_quant_kernel (quant.hip) does.
 template <bool FP16, bool QOUT, int MF, int NW>
 DEVINL void w4_reduce_store(const float (&red)[NW][MF][16 * 64], const W4View& v, int N, int mb, int n0, int cb,
-                            float (&keep)[2 * MF]) {
+                            float (&keep)[16 * MF / NW]) {
   using E = Elem<FP16>;
-  static_assert(NW == 8, "one row per wave and pass: 16 MF rows in 2 MF passes");
+  static_assert(16 % NW == 0, "one row per wave and pass: 16 MF rows in 16 MF / NW passes");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rows_here = min(v.M - mb, 16 * MF);
 #pragma unroll
-  for (int k = 0; k < 2 * MF; ++k) {
+  for (int k = 0; k < 16 * MF / NW; ++k) {
     const int ml = wave + NW * k;
     if (ml >= rows_here) continue;  // the same for all lanes of a wave
     const int i = ml / 16, rem = (ml % 16) * 64 + lane;
@@ -182,6 +182,23 @@ DEVINL void w4_reduce_store(const float (&red)[NW][MF][16 * 64], const W4View& v
 constexpr int WAVES = 8;
 constexpr int DEPTH = 8;  // K steps of qweight loads in flight per wave
 
+// 64 lanes x 4 B from global memory straight into LDS (lane l's dword lands at lds_addr + 4 l): a load without a
+// register destination, used where only the request matters. Completion is tracked by hand with vmcnt.
+DEVINL void dma4(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory");
+}
+template <int N>
+DEVINL void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+DEVINL const char* uni_ptr(const char* q) {
+  const uint64_t v = (uint64_t)q;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const char*)(((uint64_t)hi << 32) | lo);
+}
+
 // Any group size that is a multiple of 32; scales / zeros are loaded where they are used.
 template <bool FP16, int MF, bool QOUT>
 __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) {
@@ -209,7 +226,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
   // step t of this wave -> absolute K step
   auto kstep = [&](int t) { return ((t / spg) * WAVES + wave) * spg + t % spg; };
 
-  float keep[2 * MF];
+  float keep[16 * MF / WAVES];
   for (int mb = 0; mb < M; mb += 16 * MF)
   for (int cb = 0; cb < CB; ++cb) {
     const int n0 = (blockIdx.x * CB + cb) * 64;
@@ -319,11 +336,20 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
 // 4 * (lane / 16) + r of the four adjacent columns n0 + 4 * (lane % 16) + j of its own qweight words. It
 // then needs just four scales and four zero points per group (one 8-byte and one 4-byte load), and the
 // fold costs a quarter of the vector instructions of the 16-columns-per-lane layout.
-template <bool FP16, int MF, int GA, int NWAVES, bool QOUT>  // GA = groups kept in flight
-__global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
+//
+// WARM > 0: the workgroup has WARM more waves that compute nothing. They request one dword of every 128-byte line
+// of the workgroup's weight strip (64 columns = two lines per k-word row), in K order, as fast as the memory system
+// takes the requests, so that the consumer waves, whose queues are a group deep, find their lines in the L2 or on
+// the way there: a launch of this size is bound by how early its bytes are requested, not by bandwidth. The
+// requests are loads into a scrap LDS area (no register destination). With WARM the consumer lanes of activation
+// rows beyond M also issue no loads (their fragment is zero) instead of re-reading the last row.
+template <bool FP16, int MF, int GA, int NWAVES, bool QOUT, int WARM = 0>  // GA = groups kept in flight
+__global__ __launch_bounds__(64 * (NWAVES + WARM)) void w4a16_splitk_g128(W4Params p) {
   using E = Elem<FP16>;
   constexpr int SPG = 4, D = SPG * GA;
+  constexpr bool MASK = WARM > 0;
   __shared__ __attribute__((aligned(16))) float red[NWAVES][MF][16 * 64];
+  __shared__ __attribute__((aligned(256))) uint32_t scrap[WARM > 0 ? WARM : 1][64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -349,17 +375,41 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
   // before the cross-wave reduction of the current one, so the load queue does not run dry between passes.
   const int passes = (M + 16 * MF - 1) / (16 * MF) * CB;
   if (passes == 0) return;  // an expert without rows (the same for the whole workgroup)
+  if (WARM > 0 && wave >= NWAVES) {
+    // A warm-up wave: lines 2 r and 2 r + 1 are the two halves of k-word row r of the strip (256 bytes at
+    // qweight[r][n0]); the WARM waves take blocks of 64 lines in turn. The last block repeats its last line.
+    const int ww = wave - NWAVES;
+    const uint32_t scrap_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)scrap[ww];
+    const int lines = (K / 8) * 2;
+    for (int cb = 0; cb < CB; ++cb) {
+      const char* base = uni_ptr((const char*)(v.qweight + (blockIdx.x * CB + cb) * 64));
+      for (int l0 = ww * 64; l0 < lines; l0 += WARM * 64) {
+        const int line = min(l0 + lane, lines - 1);
+        dma4(base, (uint32_t)(line >> 1) * (uint32_t)N * 4u + (uint32_t)(line & 1) * 128u, scrap_addr);
+      }
+    }
+    wait_vm<0>();
+    for (int pass = 0; pass < passes; ++pass) {  // the barriers of the consumer waves' passes
+      __syncthreads();
+      __syncthreads();
+    }
+    return;
+  }
   const int32_t* qw;        // k-word row 4 * step + fq, columns n0 + 4 fr .. + 3
   const uint16_t* sc;
   const int32_t* zp;
   const uint16_t* arow[MF];
+  bool row_ok[MF];          // MASK: the lane's row of fragment i exists
   auto setup = [&](int pass) {
     const int mb = pass / CB * (16 * MF), n0 = (blockIdx.x * CB + pass % CB) * 64;
     qw = v.qweight + n0 + 4 * fr;
     sc = v.scales + n0 + 4 * fr;
     zp = v.qzeros + (n0 + 4 * fr) / 8;
 #pragma unroll
-    for (int i = 0; i < MF; ++i) arow[i] = v.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
+    for (int i = 0; i < MF; ++i) {
+      arow[i] = v.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
+      row_ok[i] = mb + i * 16 + fr < M;
+    }
   };
   u32x4_t wb[D], xr[D][MF];
   u32x2_t sg[GA];
@@ -368,7 +418,14 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
     const int ks = kstep(t);
     wb[d] = *(const u32x4_t*)(qw + (int64_t)(ks * 4 + fq) * N);
 #pragma unroll
-    for (int i = 0; i < MF; ++i) xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
+    for (int i = 0; i < MF; ++i) {
+      if (MASK) {
+        xr[d][i] = u32x4_t{0u, 0u, 0u, 0u};
+        if (row_ok[i]) xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
+      } else {
+        xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
+      }
+    }
   };
   auto load_group = [&](int q, int gi) {  // gi = index among this wave's groups
     const int64_t g = (int64_t)gi * NWAVES + wave;
@@ -387,7 +444,7 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
   setup(0);
   first_loads();
 
-  float keep[2 * MF];
+  float keep[16 * MF / NWAVES];
   for (int pass = 0; pass < passes; ++pass) {
     const int mb = pass / CB * (16 * MF), cb = pass % CB, n0 = (blockIdx.x * CB + cb) * 64;
     f32x4_t total[MF][4];  // [row fragment i][column j]: rows mb + 16 i + 4 fq + r
@@ -470,12 +527,26 @@ __global__ __launch_bounds__(64 * NWAVES) void w4a16_splitk_g128(W4Params p) {
 }
 
 template <bool FP16, bool QOUT>
-hipError_t launch(const W4Params& p, hipStream_t stream) {
+hipError_t launch(const W4Params& p, int variant, hipStream_t stream) {
   // Grouped call: one grid row per expert; the kernel variant follows the average rows per expert (an
   // expert with more rows than one pass covers is done in several passes over its weights).
   // (fp8 output: 128 columns per workgroup, N % 128 == 0 checked by the caller.)
   dim3 grid(QOUT ? p.N / 128 : (p.N + 63) / 64, p.m_sizes ? p.G : 1), block(64 * WAVES);
   const int M = p.m_sizes ? (p.M + p.G - 1) / p.G : p.M;
+  if constexpr (!QOUT) {
+    // Selectable variants (MOE_GG_OP_W4A16), group size 128: never chosen by default. The warm-up waves go with the
+    // one-fragment kernel only: ten waves leave a wave 168 registers, which the two-fragment kernel (232) does not
+    // fit, and the four-fragment kernel needs a four-wave workgroup for its 430.
+    constexpr int WARM = 2;
+    if (p.group_size == 128 && (variant & 1) && M > 32) {
+      hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 4, 1, 4, false>), grid, dim3(64 * 4), 0, stream, p);
+      return hipGetLastError();
+    }
+    if (p.group_size == 128 && (variant & 2) && M <= 16) {
+      hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES, false, WARM>), grid, dim3(64 * (WAVES + WARM)), 0, stream, p);
+      return hipGetLastError();
+    }
+  }
   // Group size 128: one activation fragment per pass for M <= 16, two for more rows (32 rows per pass over the
   // weights; four fragments do not fit the registers), all loads issued one group ahead (deeper queues and
   // more waves measured slower). Other group sizes: up to four activation fragments per pass (two with fp8
@@ -490,7 +561,7 @@ hipError_t launch(const W4Params& p, hipStream_t stream) {
 
 }  // namespace
 
-hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, hipStream_t stream) {
-  if (p.cq) return fp16 ? launch<true, true>(p, stream) : launch<false, true>(p, stream);
-  return fp16 ? launch<true, false>(p, stream) : launch<false, false>(p, stream);
+hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, int variant, hipStream_t stream) {
+  if (p.cq) return fp16 ? launch<true, true>(p, variant, stream) : launch<false, true>(p, variant, stream);
+  return fp16 ? launch<true, false>(p, variant, stream) : launch<false, false>(p, variant, stream);
 }

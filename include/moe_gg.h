@@ -328,6 +328,13 @@ int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scale
 #define MOE_GG_ORDER_TWO_LISTS 0   /* long tiles, then low tiles; last round cut by its fill alone */
 #define MOE_GG_ORDER_SPLIT_TAILS 1 /* + a tall expert's last full tile and few rows become two half tiles; row
                                       pieces of the last round chosen with the second list in view */
+#define MOE_GG_OP_W4A16 3
+/* variants of MOE_GG_OP_W4A16 (bits, group size 128 and 16-bit output only; -1 and 0 are the default kernels) */
+#define MOE_GG_W4_ONE_PASS 1 /* 33-64 rows per expert: one pass of four activation fragments on four waves instead of
+                                two passes of two fragments on eight (the weights are read and unpacked once) */
+#define MOE_GG_W4_WARMUP 2   /* up to 16 rows per expert: two extra waves per workgroup request the workgroup's weight
+                                lines ahead of the consumer waves; lanes of activation rows that do not exist issue
+                                no loads */
 int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,

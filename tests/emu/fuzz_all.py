@@ -114,13 +114,14 @@ def c_w4a16(rng):
     sc = (2.0 ** rng.integers(-3, 1, (E, K // gs, N))).astype(np.float32)
     a = ints(rng, (M, K), -2, 3)
     a16, s16 = H.to16(a, fp16), H.to16(sc, fp16)
-    what = ("w4a16", kind, M if sizes is None else sizes, N, K, gs, fp16, zero_offset)
+    variant = int(rng.choice([-1, 1, 2, 3]))       # MOE_GG_OP_W4A16: the selectable kernels too
+    what = ("w4a16", kind, M if sizes is None else sizes, N, K, gs, fp16, zero_offset, variant)
     if sizes is None:
-        c = H.w4a16(a16, qw[0], s16[0], qz[0], gs, zero_offset, fp16)
+        c = H.w4a16(a16, qw[0], s16[0], qz[0], gs, zero_offset, fp16, variant=variant)
         return exact16(c, O.w4a16_gemm(a, qw[0], sc[0], qz[0], gs, zero_offset), fp16), what
     want = O.w4a16_grouped(a, qw, sc, qz, sizes, gs, zero_offset)
     if kind == "grouped":
-        return exact16(H.w4a16(a16, qw, s16, qz, gs, zero_offset, fp16, sizes), want, fp16), what
+        return exact16(H.w4a16(a16, qw, s16, qz, gs, zero_offset, fp16, sizes, variant=variant), want, fp16), what
     cq, cs = H.w4a16(a16, qw, s16, qz, gs, zero_offset, fp16, sizes, fp8out=True)
     oq, os_ = O.fp8_groupwise_quant(H.from16(H.to16(want, fp16), fp16))
     return bool((cq == oq).all() and (cs == os_).all()), what

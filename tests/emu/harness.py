@@ -24,7 +24,7 @@ _keep = []
 _libc = ctypes.CDLL(None, use_errno=True)
 _libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
 BF16, FP16, FP32 = 0, 1, 2
-OP_BF16, OP_FP8, OP_TILE_ORDER = 0, 1, 2
+OP_BF16, OP_FP8, OP_TILE_ORDER, OP_W4A16 = 0, 1, 2, 3
 
 
 def lib():
@@ -187,8 +187,16 @@ def backward(go16, x16, w16, m_sizes, N, block_layout=False, static=False):
     return gx, gw
 
 
-def w4a16(a16, qweight, scales16, qzeros, group_size=128, zero_offset=1, fp16=False, m_sizes=None, fp8out=False):
+def w4a16(a16, qweight, scales16, qzeros, group_size=128, zero_offset=1, fp16=False, m_sizes=None, fp8out=False, variant=-1):
     L = lib()
+    L.moe_gg_set_variant(OP_W4A16, variant)
+    try:
+        return _w4a16(L, a16, qweight, scales16, qzeros, group_size, zero_offset, fp16, m_sizes, fp8out)
+    finally:
+        L.moe_gg_set_variant(OP_W4A16, -1)
+
+
+def _w4a16(L, a16, qweight, scales16, qzeros, group_size, zero_offset, fp16, m_sizes, fp8out):
     M, K = a16.shape
     dt = FP16 if fp16 else BF16
     if m_sizes is None:

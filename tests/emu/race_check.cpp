@@ -169,13 +169,20 @@ int main(int argc, char** argv) {
     auto a = bf16_small((size_t)80 * K);
     Buf<uint16_t> c((size_t)80 * N);
     const int Ms[] = {1, 16, 33, 70};
-    for (int M : Ms)
-      check(moe_gg_w4a16_splitk(a.p(), qw.p(), sc.p(), qz.p(), c.p(), M, N, K, 128, 1, MOE_GG_DTYPE_BF16, nullptr), "w4a16_splitk (M = 1, 16, 33, 70)");
+    for (int variant = 0; variant <= 3; ++variant) {  // the default kernels, then the selectable ones
+      moe_gg_set_variant(MOE_GG_OP_W4A16, variant);
+      for (int M : Ms)
+        check(moe_gg_w4a16_splitk(a.p(), qw.p(), sc.p(), qz.p(), c.p(), M, N, K, 128, 1, MOE_GG_DTYPE_BF16, nullptr), "w4a16_splitk (M = 1, 16, 33, 70; every variant)");
+    }
+    moe_gg_set_variant(MOE_GG_OP_W4A16, -1);
     check(moe_gg_w4a16_splitk(a.p(), qw.p(), sc.p(), qz.p(), c.p(), 20, N, K, 64, 0, MOE_GG_DTYPE_FP16, nullptr), "w4a16_splitk group 64 fp16");
     const int sizes[] = {3, 0, 40, 12};
     Buf<int32_t> ms(E);
     std::memcpy(ms.p(), sizes, sizeof(sizes));
     check(moe_gg_w4a16_grouped(a.p(), qw.p(), sc.p(), qz.p(), c.p(), ms.p(), E, 55, N, K, 128, 1, MOE_GG_DTYPE_BF16, nullptr), "w4a16_grouped");
+    moe_gg_set_variant(MOE_GG_OP_W4A16, MOE_GG_W4_WARMUP);
+    check(moe_gg_w4a16_grouped(a.p(), qw.p(), sc.p(), qz.p(), c.p(), ms.p(), E, 55, N, K, 128, 1, MOE_GG_DTYPE_BF16, nullptr), "w4a16_grouped with warm-up waves");
+    moe_gg_set_variant(MOE_GG_OP_W4A16, -1);
     Buf<uint8_t> cq((size_t)80 * N);
     Buf<float> cs((size_t)80 * (N / 128));
     check(moe_gg_w4a16_grouped_fp8out(a.p(), qw.p(), sc.p(), qz.p(), cq.p(), cs.p(), ms.p(), E, 55, N, K, 128, 1, MOE_GG_DTYPE_BF16, nullptr), "w4a16_grouped_fp8out");
