@@ -378,7 +378,7 @@ __global__ __launch_bounds__(64 * (NWAVES + WARM)) void w4a16_splitk_g128(W4Para
   if (WARM > 0 && wave >= NWAVES) {
     // A warm-up wave: lines 2 r and 2 r + 1 are the two halves of k-word row r of the strip (256 bytes at
     // qweight[r][n0]); the WARM waves take blocks of 64 lines in turn. The last block repeats its last line.
-    const int ww = wave - NWAVES;
+    const int ww = __builtin_amdgcn_readfirstlane(wave) - NWAVES;  // the same in every lane: scalar registers below
     const uint32_t scrap_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t*)scrap[ww];
     const int lines = (K / 8) * 2;
     for (int cb = 0; cb < CB; ++cb) {
