@@ -185,6 +185,58 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
     __syncthreads();
     read_frags(0, 0, wf0, xf0);
 
+    if constexpr (C::NW == 4 && C::FM == 8 && C::FN == 8) {
+      // Four waves of 128 x 128 outputs: a wave is alone on its SIMD, so nothing else fills the issue slots an
+      // instruction block without MFMAs leaves empty. The order is therefore written out, one MFMA at a time
+      // (64 per 32-wide half step; an MFMA occupies the matrix pipe for four issue slots, so up to three other
+      // instructions fit behind each): the 16 fragment reads of the next half step and, in a K step's second half,
+      // the 16 slab loads of the step after next each follow an MFMA, and a scheduling barrier after every such pair
+      // keeps the compiler from collecting them into blocks. Same loads, reads, waits and barrier as the loop below.
+      auto read_one = [&](int buf, int kk, int r, bf16x8_t (&wf)[C::FN], bf16x8_t (&xf)[C::FM]) {
+        // read r of a half step's 16: the activation fragments first (the first eight MFMAs use all of them)
+        const char* xs = lds + buf * C::STAGE + wm * (C::FM * 16 * 128);
+        const char* ws = lds + buf * C::STAGE + C::X_BYTES + wn * (C::FN * 16 * 128);
+        const int ro = kk ? (rd0 ^ 64) : rd0;
+        if (r < C::FM) xf[r] = *(const bf16x8_t*)(xs + r * 2048 + ro);
+        else wf[r - C::FM] = *(const bf16x8_t*)(ws + (r - C::FM) * 2048 + ro);
+      };
+      // Load r of a slab's 16 of this wave (x rows first). `keep` is all ones, or zero for the loads behind the tile's
+      // last slab: there is one loop body for every K step (no branch around a load: a lone wave pays for every
+      // branch), so the last two steps issue their loads too, with every lane's offset zero (one line per
+      // instruction, of slab KT - 1) and into the buffer that nobody reads again in this tile.
+      auto dma_one = [&](int kt, int buf, int r, uint32_t keep) {
+        const uint32_t lb = lds_wave + buf * C::STAGE;
+        if (r < C::XI) dma16(xg + kt * 128, xoff[r] & keep, lb + r * NW * 1024);
+        else dma16(wg + kt * 128, woff[r - C::XI] & keep, lb + C::X_BYTES + (r - C::XI) * NW * 1024);
+      };
+      for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        // First half: MFMAs on F0, F1 <- (slab kt, half 1), one read behind every fourth MFMA.
+#pragma unroll
+        for (int u = 0; u < 64; ++u) {
+          const int j = u >> 3, i = u & 7;
+          acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf0[j]), __builtin_bit_cast(u32x4_t, xf0[i]), acc[j][i]);
+          if ((u & 3) == 0) read_one(cur, 1, u >> 2, wf1, xf1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave has read all of slab kt
+        wait_vmcnt<0>();                                     // this wave's share of slab kt+1 has landed
+        __syncthreads();
+        // Second half: MFMAs on F1; slab kt+2 into the buffer slab kt left, one load behind every second MFMA of the
+        // first 32 (a K step and a half ahead of the wait that covers it), then F0 <- (slab kt+1, half 0; behind the
+        // last slab these reads return stale data that nothing uses).
+        const uint32_t keep = kt + 2 < KT ? ~0u : 0u;
+        const int kt2 = min(kt + 2, KT - 1);
+#pragma unroll
+        for (int u = 0; u < 64; ++u) {
+          const int j = u >> 3, i = u & 7;
+          acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf1[j]), __builtin_bit_cast(u32x4_t, xf1[i]), acc[j][i]);
+          if (u < 32 && (u & 1) == 0) dma_one(kt2, cur, u >> 1, keep);
+          else if (u >= 32 && (u & 1) == 0) read_one(cur ^ 1, 0, (u - 32) >> 1, wf0, xf0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else {
     for (int kt = 0; kt < KT; ++kt) {
       const int cur = kt & 1;
       read_frags(cur, 1, wf1, xf1);
@@ -200,6 +252,7 @@ __global__ __launch_bounds__(C::NT) void gg_bf16_persistent(GgParams p) {
       mma(wf1, xf1);
       interleave();
       __builtin_amdgcn_sched_barrier(0);
+    }
     }
     // All LDS reads of this tile were consumed by the MFMAs above; the next tile's prologue may
     // overwrite both buffers only after every wave got here.
