@@ -185,6 +185,9 @@ static int grouped_gemm_16(const void* x, const void* w, void* y, const int32_t*
       if (e != hipSuccess || !tails) return (int)e;
       return (int)gg_bf16_decode_tails_launch(p, s);
     }
+    case MOE_GG_GG_FOURWAVE_256:
+      if (!pingpong_ok) return MOE_GG_EUNSUPPORTED;
+      return (int)gg_bf16_fourwave_launch(p, num_wg, s);
     case MOE_GG_GG_TILED_256: return (int)gg_bf16_tiled_launch(p, 256, num_wg, s);
     case MOE_GG_GG_TILED_256_W4: return (int)gg_bf16_tiled_launch(p, GG_TILED_256_FOUR_WAVES, num_wg, s);
     case MOE_GG_GG_TILED_128: return (int)gg_bf16_tiled_launch(p, 128, num_wg, s);

@@ -677,8 +677,224 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
   wait_vm<0>();                   // trailing (never read) slab loads must land before the LDS is released
 }
 
+
+// ---- Four waves, 128 x 128 outputs each ------------------------------------------------------------------------
+// The same 256 x 256 tile, LDS stages, slab loads and tile order on a workgroup of four waves, one per SIMD. Wave
+// (wm, wn) owns the activation fragments i = 0 .. 7 of tile rows (2 i + wm) * 16 .. + 15 and the weight fragments
+// j = 0 .. 7 of tile columns (8 wn + j) * 16 .. + 15: 64 accumulators of four registers (all 256 accumulation
+// registers), and per 32-wide half step 16 fragment reads feed 64 MFMAs where a wave of the eight-wave kernel reads
+// 12 for 32: a third fewer LDS bytes per MFMA. A wave alone on its SIMD has nobody to fill the issue slots that an
+// instruction block without MFMAs leaves empty, so the order is written out one MFMA at a time (an MFMA holds the
+// matrix pipe for four issue slots: up to three other instructions fit behind it): in the first half of a K step
+// the 16 reads of the second half's fragments follow every fourth MFMA; then the wave waits for its reads and for
+// its loads of the next slab, and the workgroup's one barrier per K step publishes that slab and frees the buffer of
+// the present one; in the second half the 16 loads of the slab after next go into that buffer, one behind every
+// second MFMA of the first 32 (a K step and a half ahead of the wait that covers them), and the 16 reads of the
+// next step's first half follow every second MFMA of the last 32. A scheduling barrier after every such pair keeps
+// the compiler from collecting reads or loads into blocks. The slab stream runs through tile boundaries (the loads
+// and the reads for a tile's first step are issued in the last step of the tile before, and land during its
+// epilogue); behind the last tile the loads are still issued, with every lane's offset zero (one line per
+// instruction) into a buffer nobody reads again: one loop body, no branch around a load.
+constexpr int W4_NW = 4, W4_NT = 64 * W4_NW, W4_FM = 8, W4_FN = 8;
+
 template <int OP>
+DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
+  static_assert(OP == OP_BF16 || OP == OP_F16, "forward product on 16-bit floats");
+  constexpr bool F16 = op_f16(OP);
+  constexpr int FMW = W4_FM, FNW = W4_FN;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  const int N = p.N;
+  const uint32_t KROW = (uint32_t)p.K * 2u;  // bytes per operand row
+  const int KT = (int)(KROW / 128u);         // K steps of every tile
+
+  struct Tile { int g, row0, m0, h, n0, nc; };
+  auto tile_at = [&](int seq) {
+    // As decoded in the prologue: group | rows << 16 | columns / 32 << 26, first row / 64 | first column / 32 << 16.
+    const int gh = uni(sh.seq_tab[2 * seq]), mn = uni(sh.seq_tab[2 * seq + 1]);
+    Tile t;
+    t.g = gh & 0xFFFF;
+    t.h = (gh >> 16) & 0x3FF;
+    t.nc = (int)((uint32_t)gh >> 26) * 32;
+    t.m0 = (mn & 0xFFFF) * 64;
+    t.n0 = (int)((uint32_t)mn >> 16) * 32;
+    t.row0 = uni(sh.row_off[t.g]);
+    return t;
+  };
+
+  // Slab loads: an instruction fills 8 rows (1 KB of LDS): lane -> row lane / 8, physical 16-byte slot lane % 8, which
+  // must hold logical chunk slot ^ ((row >> 1) & 7). Instruction r of wave w fills the 8-row block 4 r + w.
+  const int d_r = lane >> 3;
+  const uint32_t d_c16 = (uint32_t)(((lane & 7) ^ (((wave & 1) << 2) | (lane >> 4))) << 4);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)sh.lds;
+  // Fragment reads: row = fragment * 16 + lane % 16, chunk = half * 4 + lane / 16 (swizzled).
+  const int fr = lane & 15, fq = lane >> 4;
+  const int rd0 = fr * 128 + ((fq ^ (fr >> 1)) << 4);  // first half; the second is rd0 ^ 64
+
+  const char* xp = (const char*)p.x;
+  const char* wp = (const char*)p.w;
+  bf16_t* __restrict__ yp = (bf16_t*)p.y;
+
+  // Load cursor: the slab (tile of the sequence, K step) that the next 16 load instructions of this wave fetch.
+  const char* c_xg = xp;
+  const char* c_wg = wp;
+  uint32_t c_xoff[8], c_woff[8];
+  uint32_t c_keep = ~0u;  // zero behind the last tile
+  int c_seq = 0, c_kt = 0;
+  auto cursor_tile = [&](int seq) {
+    c_seq = seq;
+    c_kt = 0;
+    if (seq >= sh.n_my) {  // behind the last tile: the pointers stay at the last tile's (in bounds), offsets zero
+      c_keep = 0u;
+      return;
+    }
+    const Tile t = tile_at(seq);
+    const int x_last = max(t.h, 1) - 1, w_last = max(min(N - t.n0, t.nc), 1) - 1;
+    c_xg = uni_ptr(xp + (int64_t)(t.row0 + t.m0) * KROW);
+    c_wg = uni_ptr(wp + ((int64_t)t.g * N + t.n0) * KROW);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      // rows beyond the tile's last one re-read it (the loads stay inside the tensors)
+      c_xoff[r] = (uint32_t)min((r * W4_NW + wave) * 8 + d_r, x_last) * KROW + d_c16;
+      c_woff[r] = (uint32_t)min((r * W4_NW + wave) * 8 + d_r, w_last) * KROW + d_c16;
+    }
+  };
+  auto cursor_next = [&]() {
+    if (c_keep != 0u && ++c_kt == KT) cursor_tile(c_seq + 1);
+  };
+  auto load_one = [&](int r, int buf) {  // load r of the cursor slab's 16 (activation rows first) into stage buf
+    const uint32_t lb = lds_base + buf * STAGE + wave * 1024;
+    if (r < 8) dma16(c_xg + c_kt * 128, c_xoff[r] & c_keep, lb + r * W4_NW * 1024);
+    else dma16(c_wg + c_kt * 128, c_woff[r - 8] & c_keep, lb + X_BYTES + (r - 8) * W4_NW * 1024);
+  };
+
+  bf16x8_t wf0[FNW], xf0[FMW], wf1[FNW], xf1[FMW];
+  auto read_one = [&](int buf, int half, int r, bf16x8_t (&wf)[FNW], bf16x8_t (&xf)[FMW]) {
+    // read r of a half step's 16: the activation fragments first (the first eight MFMAs use all of them)
+    const char* st = sh.lds + buf * STAGE;
+    const int ro = half ? (rd0 ^ 64) : rd0;
+    if (r < FMW) xf[r] = *(const bf16x8_t*)(st + (r * 2 + wm) * 2048 + ro);
+    else wf[r - FMW] = *(const bf16x8_t*)(st + X_BYTES + (wn * FNW + r - FMW) * 2048 + ro);
+  };
+
+  f32x4_t acc[FNW][FMW];
+
+  // Stream start: slabs 0 and 1 in flight, first fragments read.
+  cursor_tile(0);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) load_one(r, 0);
+  cursor_next();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) load_one(r, 1);
+  cursor_next();
+  wait_vm<16>();  // slab 0 (loads return in order)
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) read_one(0, 0, r, wf0, xf0);
+
+  int step = 0;  // K steps done, over all tiles: slab `step` sits in stage step & 1
+  for (int seq = 0; seq < sh.n_my; ++seq) {
+    // The lanes of a wave leave the epilogue's row-masked store blocks at different points and are together again
+    // here (no instruction; it also keeps the compiler from moving memory operations across the tile boundary).
+    __builtin_amdgcn_wave_barrier();
+    const Tile t = tile_at(seq);
+#pragma unroll
+    for (int j = 0; j < FNW; ++j)
+#pragma unroll
+      for (int i = 0; i < FMW; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int kt = 0; kt < KT; ++kt, ++step) {
+      const int cur = step & 1;
+      // First half: MFMAs on (wf0, xf0); (wf1, xf1) <- second half of the slab, one read behind every fourth MFMA.
+#pragma unroll
+      for (int u = 0; u < 64; ++u) {
+        const int j = u >> 3, i = u & 7;
+        acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf0[j]), __builtin_bit_cast(u32x4_t, xf0[i]), acc[j][i]);
+        if ((u & 3) == 0) read_one(cur, 1, u >> 2, wf1, xf1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      wait_lgkm0();   // this wave has read all it needs of the slab
+      wait_vm<0>();   // its share of the next slab has landed
+      __syncthreads();
+      // Second half: MFMAs on (wf1, xf1); the slab after next into the stage that is free now; (wf0, xf0) <- first
+      // half of the next slab.
+#pragma unroll
+      for (int u = 0; u < 64; ++u) {
+        const int j = u >> 3, i = u & 7;
+        acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf1[j]), __builtin_bit_cast(u32x4_t, xf1[i]), acc[j][i]);
+        if (u < 32 && (u & 1) == 0) load_one(u >> 1, cur);
+        else if (u >= 32 && (u & 1) == 0) read_one(cur ^ 1, 0, (u - 32) >> 1, wf0, xf0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      cursor_next();
+    }
+
+    // Epilogue: lane holds y[m][n .. n + 3] for m = (2 i + wm) * 16 + lane % 16, n = (8 wn + j) * 16 + 4 (lane / 16).
+    const int rows_valid = t.h, cols_valid = min(N - t.n0, t.nc);
+    bf16_t* yg = yp + (int64_t)(t.row0 + t.m0) * p.ldy + (int64_t)t.g * p.col_block + t.n0;
+    if (p.vec_store && cols_valid == BN && p.ldy < (1 << 24)) {
+      const uint32_t voff = (uint32_t)fr * (uint32_t)p.ldy + (uint32_t)(wn * FNW * 16 + fq * 4);
+#pragma unroll
+      for (int i = 0; i < FMW; ++i) {
+        const int mrow = (i * 2 + wm) * 16;
+        bf16_t* ybase = yg + (int64_t)mrow * p.ldy;  // uniform
+        if (mrow + fr < rows_valid) {
+          if (p.vec_store == 2) {
+            // Lanes l and l ^ 16 (column quarters 2 q, 2 q + 1 of the same row) trade halves so that each stores 16
+            // bytes: the even one columns 8 q' .. + 7 of fragment j, the odd one those of fragment j + 1.
+#pragma unroll
+            for (int j = 0; j < FNW; j += 2) {
+              const f32x4_t v0 = acc[j][i], v1 = acc[j + 1][i];
+              const uint32_t a0 = pack_16x2<F16>(v0[0], v0[1]), a1 = pack_16x2<F16>(v0[2], v0[3]);
+              const uint32_t b0 = pack_16x2<F16>(v1[0], v1[1]), b1 = pack_16x2<F16>(v1[2], v1[3]);
+              const bool odd = fq & 1;
+              const uint32_t s0 = odd ? a0 : b0, s1 = odd ? a1 : b1;   // what the partner stores
+              const uint32_t r0 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)s0, 0x401F);  // lane ^ 16
+              const uint32_t r1 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)s1, 0x401F);
+              u32x4_t o;
+              if (odd) o = u32x4_t{r0, r1, b0, b1}; else o = u32x4_t{a0, a1, r0, r1};
+              *(u32x4_t*)(ybase + voff + (odd ? (j + 1) * 16 - 4 : j * 16)) = o;
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < FNW; ++j) {
+              const f32x4_t v = acc[j][i];
+              u32x2_t o;
+              o[0] = pack_16x2<F16>(v[0], v[1]);
+              o[1] = pack_16x2<F16>(v[2], v[3]);
+              *(u32x2_t*)(ybase + voff + j * 16) = o;
+            }
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < FMW; ++i) {
+        const int m = (i * 2 + wm) * 16 + fr;
+        if (m < rows_valid) {
+          bf16_t* yrow = yg + (int64_t)m * p.ldy;
+#pragma unroll
+          for (int j = 0; j < FNW; ++j) {
+            const int n = (wn * FNW + j) * 16 + fq * 4;
+            const f32x4_t v = acc[j][i];
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr)
+              if (n + rr < cols_valid) ((uint16_t*)yrow)[n + rr] = cvt_16<F16>(v[rr]);
+          }
+        }
+      }
+    }
+  }
+  wait_vm<0>();  // the trailing (never read) slab loads must land before the LDS is released
+}
+
+// FOURWAVE: the workgroup is four waves running run_fourwave (one wave per SIMD, 128 x 128 outputs each) instead of the
+// two groups of four above; tables, tile order and LDS stages are the same.
+template <int OP, bool FOURWAVE = false>
 DEVINL void pingpong_body(const GgParams& p) {
+  constexpr int NTB = FOURWAVE ? W4_NT : NT;  // threads of the workgroup
   __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + (OP == OP_FP8_BLOCK ? 2 * SCALE_BYTES : 0)];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t tile_off[MOE_GG_MAX_GROUPS + 1];
@@ -739,7 +955,7 @@ DEVINL void pingpong_body(const GgParams& p) {
   // dealt to the workgroups round-robin: every workgroup gets the same number (+- 1) of long tiles, and the second
   // list goes on where the long ones stopped.
   const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
-  for (int i = threadIdx.x; i < n_my; i += NT) {
+  for (int i = threadIdx.x; i < n_my; i += NTB) {
     int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
     constexpr int TC = op_swiglu(OP) ? BN / 2 : BN;  // output columns of a tile
     int g, m0, h, n0, nc = TC;  // group, first row inside the group, rows, first column, columns
@@ -769,13 +985,19 @@ DEVINL void pingpong_body(const GgParams& p) {
   __syncthreads();
 
   Shared sh{row_off, tile_off, part_off, seq_tab, lds, n_my};
-  const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
-  if (grp == 0) run_group<0, OP>(p, sh);
-  else run_group<1, OP>(p, sh);
+  if constexpr (FOURWAVE) {
+    run_fourwave<OP>(p, sh);
+  } else {
+    const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
+    if (grp == 0) run_group<0, OP>(p, sh);
+    else run_group<1, OP>(p, sh);
+  }
 }
 
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_body<OP_BF16>(p); }
 __global__ __launch_bounds__(NT) void gg_f16_pingpong(GgParams p) { pingpong_body<OP_F16>(p); }
+__global__ __launch_bounds__(W4_NT) void gg_bf16_fourwave(GgParams p) { pingpong_body<OP_BF16, true>(p); }
+__global__ __launch_bounds__(W4_NT) void gg_f16_fourwave(GgParams p) { pingpong_body<OP_F16, true>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
 __global__ __launch_bounds__(NT) void gg_f16_pingpong_swiglu(GgParams p) { pingpong_body<OP_F16_SWIGLU>(p); }
@@ -791,6 +1013,12 @@ __global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpo
 hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream) {
   if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
   else hipLaunchKernelGGL(gg_bf16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t gg_bf16_fourwave_launch(const GgParams& p, int num_wg, hipStream_t stream) {
+  if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+  else hipLaunchKernelGGL(gg_bf16_fourwave, dim3(num_wg), dim3(W4_NT), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -315,6 +315,9 @@ int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scale
 #define MOE_GG_GG_GENERIC 4      /* one thread per output element, any shape / alignment */
 #define MOE_GG_GG_DECODE 5       /* small-M path: weights streamed once, split-K inside the workgroup */
 #define MOE_GG_GG_TILED_256_W4 6 /* 256x256 tiles on four waves of 128x128 outputs each (never chosen automatically) */
+#define MOE_GG_GG_FOURWAVE_256 7 /* the ping-pong kernel's tiles, tile order and slab stream on four waves of 128x128
+                                    outputs each, loads and LDS reads placed behind single MFMAs (never chosen
+                                    automatically) */
 #define MOE_GG_OP_GG_FP8 1
 /* variants of MOE_GG_OP_GG_FP8 */
 #define MOE_GG_FP8_TILED_128 0       /* 128x128 tiles for every expert */

@@ -87,6 +87,7 @@ struct Fiber {
 struct Wave {
   int alive, waiting;
   bool wait[64];
+  bool join[64];                 // the lane waits at a join point (wave_join): for every live lane of the wave
   const void* site[64];          // where the lane waits (the call that started the exchange, or its end)
   uint64_t epoch[64];            // how often the lane has moved backwards in the code (loop iterations, roughly)
   unsigned long long mask[64];   // lanes of the exchange the lane was released from last
@@ -129,11 +130,18 @@ uint64_t g_divergent = 0;
 // in the program go first and meet the others further down, as the hardware runs a branch to its join point.
 // "Behind" is judged by (epoch, code address): a lane's epoch goes up whenever its next exchange lies at a lower
 // address than its last one (a loop's back edge); lanes released together continue with the same epoch.
+// That guess fails where a divergent region ends a loop body (the lanes that skipped it wait at the top of the next
+// iteration, at a lower address and the same epoch as the lanes inside it). A kernel marks such a place with
+// __builtin_amdgcn_wave_barrier() (wave_join below): lanes that wait there are released only when every live lane of
+// the wave has arrived, so lanes still inside a divergent region always go first.
 void try_release(Wave& w, bool force) {
   if (w.waiting == 0 || (!force && w.waiting < w.alive)) return;
+  bool other = false;  // some lane waits at an ordinary exchange
+  for (int l = 0; l < 64; ++l) other |= w.wait[l] && !w.join[l];
   int pick = -1;
   for (int l = 0; l < 64; ++l)
-    if (w.wait[l] && (pick < 0 || w.epoch[l] < w.epoch[pick] || (w.epoch[l] == w.epoch[pick] && w.site[l] < w.site[pick]))) pick = l;
+    if (w.wait[l] && !(other && w.join[l]) &&
+        (pick < 0 || w.epoch[l] < w.epoch[pick] || (w.epoch[l] == w.epoch[pick] && w.site[l] < w.site[pick]))) pick = l;
   unsigned long long m = 0;
   uint64_t top = 0;
   for (int l = 0; l < 64; ++l)
@@ -175,11 +183,12 @@ void fiber_main() {
   fail("a finished fiber was resumed");
 }
 
-void wave_sync(const void* site) {
+void wave_sync(const void* site, bool join = false) {
   Fiber* f = g_cur;
   Wave& w = g_w[f->tid >> 6];
   const int l = f->tid & 63;
   w.wait[l] = true;
+  w.join[l] = join;
   if (site < w.site[l]) ++w.epoch[l];
   w.site[l] = site;
   ++w.waiting;
@@ -226,6 +235,7 @@ void run_workgroup(unsigned order_seed) {
     g_w[w].alive = std::min(64, nt - 64 * w);
     g_w[w].waiting = 0;
     memset(g_w[w].wait, 0, sizeof(g_w[w].wait));
+    memset(g_w[w].join, 0, sizeof(g_w[w].join));
     memset(g_w[w].site, 0, sizeof(g_w[w].site));
     memset(g_w[w].epoch, 0, sizeof(g_w[w].epoch));
   }
@@ -354,6 +364,9 @@ __attribute__((noinline)) void exchange_done(const void* site) {
   if (!site) site = __builtin_return_address(0);
   wave_sync((const char*)site + 1);
 }
+
+// A place where the whole wave is together again (the top of a loop whose body ends in a divergent region).
+__attribute__((noinline)) void wave_join() { wave_sync(__builtin_return_address(0), true); }
 
 __attribute__((noinline)) int readfirstlane(int v) {
   const void* site = __builtin_return_address(0);

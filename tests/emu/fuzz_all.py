@@ -46,7 +46,7 @@ def c_gemm(rng):
         N, K, variant = int(rng.integers(1, 200)), int(rng.integers(1, 200)), -1
     else:
         N, K = int(rng.choice([16, 64, 100, 128, 256, 264, 512])), int(rng.choice([64, 128, 192, 256]))
-        variant = int(rng.choice([-1, 0, 1, 2, 3, 4, 5, 6]))
+        variant = int(rng.choice([-1, 0, 1, 2, 3, 4, 5, 6, 7, 7]))
         if variant == 5 and K % 128:
             K = 128
     G, M = len(sizes), sum(sizes)

@@ -25,12 +25,12 @@ def one_case(rng):
     M = sum(sizes)
     N = int(rng.choice([64, 256, 320, 512, 768]))
     K = int(rng.choice([64, 128, 192]))
-    op = str(rng.choice(["bf16", "f16", "swiglu", "gather", "fp8row", "fp8block"]))
-    if op in ("bf16", "f16"):
-        fp16 = op == "f16"
+    op = str(rng.choice(["bf16", "f16", "bf16w4", "f16w4", "swiglu", "gather", "fp8row", "fp8block"]))
+    if op in ("bf16", "f16", "bf16w4", "f16w4"):     # ...w4: the same tiles and order on the four-wave kernel
+        fp16 = op.startswith("f16")
         x = rng.integers(-4, 5, (M, K)).astype(np.float32)
         w = rng.integers(-4, 5, (G * N, K)).astype(np.float32)
-        y = H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), sizes, N, fp16=fp16, variant=0)
+        y = H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), sizes, N, fp16=fp16, variant=7 if op.endswith("w4") else 0)
         good = (H.from16(y, fp16) == H.from16(H.to16(O.grouped_gemm(x, w, sizes), fp16), fp16)).all()
     elif op == "gather":   # the fused activation kernel reading its rows through a permutation: same bits as gather + kernel
         n, k = max(64, N // 2 // 4 * 4), int(rng.integers(1, 4))

@@ -70,6 +70,7 @@ template <class T> inline T get_lane(T v, int src, const void* site = nullptr) {
   return r;
 }
 int readfirstlane(int v);
+void wave_join();
 unsigned long long ballot(int pred);
 f32x4 mfma_16x16x32_bf16(bf16x8 a, bf16x8 b, f32x4 c);
 f32x4 mfma_16x16x32_f16(f16x8 a, f16x8 b, f32x4 c);
@@ -103,6 +104,7 @@ template <class T> inline T atomicAdd(T* p, T v) { return __atomic_fetch_add(p, 
 // Fast-math exponential of the device library: the host's expf (results differ in the last bits).
 #define __expf(x) expf(x)
 #define __builtin_amdgcn_readfirstlane(v) emu::readfirstlane((int)(v))
+#define __builtin_amdgcn_wave_barrier() emu::wave_join()
 #define __builtin_amdgcn_sched_barrier(m) ((void)0)
 #define __builtin_amdgcn_sched_group_barrier(a, b, c) ((void)0)
 #define __builtin_amdgcn_s_setprio(p) ((void)0)

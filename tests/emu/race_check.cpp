@@ -87,10 +87,11 @@ static int one_shape(const char* op, int N, int K, int G, char** sizes) {
     for (int i = M - 1; i > 0; --i) std::swap(perm.v[i], perm.v[rnd() % (i + 1)]);
     check(moe_gg_grouped_gemm_swiglu_gather(x.p(), T, perm.p(), 2, w.p(), y.p(), ms.p(), G, M, N, K, N, MOE_GG_DTYPE_BF16, nullptr), op);
   } else {
-    const bool f16 = !std::strcmp(op, "f16");
+    const bool f16 = !std::strcmp(op, "f16") || !std::strcmp(op, "f16w4");
+    const bool fourwave = !std::strcmp(op, "bf16w4") || !std::strcmp(op, "f16w4");
     auto x = f16 ? f16_small((size_t)M * K) : bf16_small((size_t)M * K);
     auto w = f16 ? f16_small((size_t)G * N * K) : bf16_small((size_t)G * N * K);
-    moe_gg_set_variant(MOE_GG_OP_GG_BF16, MOE_GG_GG_PINGPONG_256);
+    moe_gg_set_variant(MOE_GG_OP_GG_BF16, fourwave ? MOE_GG_GG_FOURWAVE_256 : MOE_GG_GG_PINGPONG_256);
     check((f16 ? moe_gg_grouped_gemm_f16 : moe_gg_grouped_gemm_bf16)(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, MOE_GG_OUT_MN, nullptr), op);
   }
   return failures ? 1 : 0;
@@ -114,7 +115,7 @@ int main(int argc, char** argv) {
     std::memcpy(ms.p(), sizes, sizeof(sizes));
     auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * N * K);
     Buf<uint16_t> y((size_t)M * N * G);
-    for (int variant = -1; variant <= 6; ++variant) {
+    for (int variant = -1; variant <= 7; ++variant) {
       moe_gg_set_variant(MOE_GG_OP_GG_BF16, variant);
       check(moe_gg_grouped_gemm_bf16(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, MOE_GG_OUT_MN, nullptr), "grouped_gemm_bf16 (every variant)");
     }

@@ -55,7 +55,7 @@ def tile_order(request):
 SIZES = [300, 0, 70, 530]   # a full tile + a low tile, an empty expert, a short one, a tall one whose tail is split
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, -1])
 def test_bf16_every_kernel_variant(variant, tile_order):
     rng = np.random.default_rng(variant + 1)
     x, w = ints(rng, (sum(SIZES), 128)), ints(rng, (4 * 512, 128))
@@ -65,15 +65,17 @@ def test_bf16_every_kernel_variant(variant, tile_order):
 
 @pytest.mark.parametrize("K", [64, 128, 192, 320])
 @pytest.mark.parametrize("sizes,N", [([300, 0, 70, 530], 512), ([257, 1], 300), ([40], 64)])
-def test_four_wave_tiled_kernel_over_k_steps(sizes, N, K):
-    """MOE_GG_GG_TILED_256_W4 with 1, 2, 3 and 5 K steps per tile: its loop issues the slab loads behind the last slab
-    too (masked to one line, into the buffer nobody reads again), so the short reductions are the cases to see."""
+@pytest.mark.parametrize("variant", [6, 7])
+def test_four_wave_kernels_over_k_steps(sizes, N, K, variant):
+    """MOE_GG_GG_TILED_256_W4 and MOE_GG_GG_FOURWAVE_256 with 1, 2, 3 and 5 K steps per tile: their loops issue the
+    slab loads behind the last slab too (masked to one line, into the buffer nobody reads again), and the second one
+    streams slabs through tile boundaries, so the short reductions are the cases to see."""
     rng = np.random.default_rng(K + N)
     G = len(sizes)
     x, w = ints(rng, (sum(sizes), K)), ints(rng, (G * N, K))
-    for fp16 in (False, True):
-        y = H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), sizes, N, fp16=fp16, variant=6)
-        assert exact16(y, O.grouped_gemm(x, w, sizes), fp16)
+    for fp16, block in ((False, False), (True, True)):
+        y = H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), sizes, N, fp16=fp16, block_layout=block, variant=variant)
+        assert exact16(y, O.grouped_gemm(x, w, sizes, block_layout=block), fp16)
 
 
 @pytest.mark.parametrize("fp16,block", [(True, False), (False, True), (True, True)])
@@ -431,7 +433,8 @@ def test_no_data_race_between_the_waves_of_a_workgroup():
     shapes = [("bf16", "512", "128", "1", "0", ["530", "300", "0", "70"]), ("swiglu", "256", "128", "2", "5", ["833", "64", "257"]),
               ("gather", "128", "128", "2", "3", ["530", "1", "300"]),
               ("fp8block", "384", "256", "1", "0", ["577", "33", "320"]), ("fp8row", "256", "128", "3", "9", ["129", "768", "1"]),
-              ("f16", "384", "256", "2", "0", ["321", "511"]), ("bwd", "256", "128", "3", "4", ["300", "0", "41", "513"])]
+              ("f16", "384", "256", "2", "0", ["321", "511"]), ("bwd", "256", "128", "3", "4", ["300", "0", "41", "513"]),
+              ("bf16w4", "512", "192", "1", "0", ["530", "300", "0", "70"]), ("f16w4", "384", "64", "2", "6", ["321", "511", "1"])]
     for i, (op, N, K, cus, seed, sizes) in enumerate(shapes):
         for order in ("0", "1"):
             procs.append(subprocess.Popen([exe, "shape", op, N, K] + sizes,

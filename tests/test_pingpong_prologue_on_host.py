@@ -24,7 +24,7 @@ HARNESS_HEAD = r'''
 #include "tile_sched.h"
 #define MOE_GG_MAX_GROUPS 1024
 using std::min; using std::max;
-constexpr int BM = 256, BN = 256, NT = 512;
+constexpr int BM = 256, BN = 256, NT = 512, NTB = NT;
 constexpr int OP_BF16 = 0, OP_FP8_ROW = 1, OP_FP8_BLOCK = 2, OP_BF16_WGRAD = 3, OP_BF16_SWIGLU = 4, OP_BF16_NT = 5,
               OP_BF16_WGRAD_DIRECT = 6, OP_F16 = 7, OP_F16_SWIGLU = 8, OP_BF16_SWIGLU_GATHER = 9, OP_F16_SWIGLU_GATHER = 10;
 constexpr bool op_gather(int op) { return op == OP_BF16_SWIGLU_GATHER || op == OP_F16_SWIGLU_GATHER; }
