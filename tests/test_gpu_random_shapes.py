@@ -1,7 +1,8 @@
-"""NOT an oracle comparison: every fast kernel against the generic HIP kernel of the same library, a self-comparison
-that earns parity credit only through the chain generic kernel -> oracle (tests/test_gpu_grouped_gemm_bf16.py pins
-the generic kernel, variant 4, against the CPU oracle). Random shapes and expert-size distributions; the generic
-kernel is one thread per output element with fp32 accumulation in k order. Covers what the fixed oracle cases miss:
+"""Random shapes and expert-size distributions. The forward product of the generic HIP kernel (one thread per output
+element, fp32 accumulation in k order) is checked against the oracle's per-expert fp32 matmul loop on the CPU
+(dev/triton_groupGEMM/testing/unit_tests.py:49-55) for every case, and every fast kernel against the generic one; the
+fused SiLU-and-mul GEMM and the backward pass are compared with the generic kernel's path only (their oracle tests are
+tests/test_gpu_moe_layer.py and tests/test_gpu_backward.py). Covers what the fixed oracle cases miss:
 tile tables with many experts, empty experts, sizes around the tile edges, N and K that are not multiples of the
 tiles. Bar: the grouped-GEMM bar of the parity tests, 1e-2 + 1e-2 |ref| on bf16 results (the two sides round the
 same fp32 sums, accumulated in different orders)."""
@@ -9,6 +10,8 @@ import random
 
 import pytest
 import torch
+
+from oracle import oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -60,6 +63,10 @@ def test_fast_paths_against_the_generic_kernel(seed):
             m = torch.tensor(ms, dtype=torch.int32, device="cuda")
             L.moe_gg_set_variant(0, GENERIC)
             ref = A.grouped_gemm(x, w, m)[:R]
+            if R > 0:
+                cpu = O.grouped_gemm_torch_loop(x[:R].float().cpu(), w.float().cpu(), ms)
+                ok, worst = close(ref.cpu(), cpu)
+                assert ok, ("generic kernel against the oracle", G, R, N, K, worst)
             for variant in (PINGPONG, AUTO):
                 L.moe_gg_set_variant(0, variant)
                 ok, worst = close(A.grouped_gemm(x, w, m)[:R], ref)
