@@ -486,7 +486,7 @@ def wl_fp8_cfg5(torch, A, dev, lib, stream, cpu):
     ws = torch.empty(G * N // 128, K // 128, dtype=torch.float32, device=dev)
     for g in range(G):
         q, sc = A.float8_blockwise_quantize_weight(torch.randn(N, K, generator=gen, device=dev) * 0.02)
-        wq[g * N:(g + 1) * N] = q
+        wq.view(torch.uint8)[g * N:(g + 1) * N] = q.view(torch.uint8)     # a byte copy: no fp8 copy kernel needed
         ws[g * N // 128:(g + 1) * N // 128] = sc
     y = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
     ms_dev = m5.to(torch.int32).to(dev)
