@@ -686,7 +686,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
 // 12 for 32: a third fewer LDS bytes per MFMA. A wave alone on its SIMD has nobody to fill the issue slots that an
 // instruction block without MFMAs leaves empty, so the order is written out one MFMA at a time (an MFMA holds the
 // matrix pipe for four issue slots: up to three other instructions fit behind it): in the first half of a K step
-// the 16 reads of the second half's fragments follow every fourth MFMA; then the wave waits for its reads and for
+// the 16 reads of the second half's fragments follow every third MFMA; then the wave waits for its reads and for
 // its loads of the next slab, and the workgroup's one barrier per K step publishes that slab and frees the buffer of
 // the present one; in the second half the 16 loads of the slab after next go into that buffer, one behind every
 // second MFMA of the first 32 (a K step and a half ahead of the wait that covers them), and the 16 reads of the
@@ -807,12 +807,13 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
 
     for (int kt = 0; kt < KT; ++kt, ++step) {
       const int cur = step & 1;
-      // First half: MFMAs on (wf0, xf0); (wf1, xf1) <- second half of the slab, one read behind every fourth MFMA.
+      // First half: MFMAs on (wf0, xf0); (wf1, xf1) <- second half of the slab, one read behind every third MFMA, so
+      // that the last one is 18 MFMAs old when the wave waits for its reads.
 #pragma unroll
       for (int u = 0; u < 64; ++u) {
         const int j = u >> 3, i = u & 7;
         acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf0[j]), __builtin_bit_cast(u32x4_t, xf0[i]), acc[j][i]);
-        if ((u & 3) == 0) read_one(cur, 1, u >> 2, wf1, xf1);
+        if (u % 3 == 0 && u / 3 < 16) read_one(cur, 1, u / 3, wf1, xf1);
         __builtin_amdgcn_sched_barrier(0);
       }
       wait_lgkm0();   // this wave has read all it needs of the slab
