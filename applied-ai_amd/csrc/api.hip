@@ -393,6 +393,9 @@ static int grouped_gemm_swiglu_16(const void* x, const void* w, void* y, const i
   p.gather_perm = perm;
   p.gather_k = k;
   p.gather_rows = (int)T;
+  // The four-wave form when that kernel is pinned for the grouped GEMM (it has no row gather).
+  if (!perm && g_variant[MOE_GG_OP_GG_BF16].load() == MOE_GG_GG_FOURWAVE_256)
+    return (int)gg_bf16_fourwave_swiglu_launch(p, num_wg, (hipStream_t)stream);
   return (int)gg_bf16_pingpong_swiglu_launch(p, num_wg, (hipStream_t)stream);
 }
 

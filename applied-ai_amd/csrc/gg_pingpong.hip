@@ -699,14 +699,18 @@ constexpr int W4_NW = 4, W4_NT = 64 * W4_NW, W4_FM = 8, W4_FN = 8;
 
 template <int OP>
 DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
-  static_assert(OP == OP_BF16 || OP == OP_F16, "forward product on 16-bit floats");
+  static_assert(OP == OP_BF16 || OP == OP_F16 || OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU,
+                "forward product on 16-bit floats, plain or with SiLU-and-mul in the epilogue");
   constexpr bool F16 = op_f16(OP);
+  constexpr bool SWIGLU = op_swiglu(OP);
   constexpr int FMW = W4_FM, FNW = W4_FN;
+  constexpr int TILE_COLS = SWIGLU ? BN / 2 : BN;  // output columns of a tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
   const int N = p.N;
+  const int NCOLS = SWIGLU ? N / 2 : N;      // output columns of a group
   const uint32_t KROW = (uint32_t)p.K * 2u;  // bytes per operand row
   const int KT = (int)(KROW / 128u);         // K steps of every tile
 
@@ -751,14 +755,20 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
       return;
     }
     const Tile t = tile_at(seq);
-    const int x_last = max(t.h, 1) - 1, w_last = max(min(N - t.n0, t.nc), 1) - 1;
+    // w_last: last valid weight row of the tile; SWIGLU: last valid output column (a gate row and an up row each)
+    const int x_last = max(t.h, 1) - 1, w_last = max(min(NCOLS - t.n0, t.nc), 1) - 1;
     c_xg = uni_ptr(xp + (int64_t)(t.row0 + t.m0) * KROW);
     c_wg = uni_ptr(wp + ((int64_t)t.g * N + t.n0) * KROW);
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       // rows beyond the tile's last one re-read it (the loads stay inside the tensors)
-      c_xoff[r] = (uint32_t)min((r * W4_NW + wave) * 8 + d_r, x_last) * KROW + d_c16;
-      c_woff[r] = (uint32_t)min((r * W4_NW + wave) * 8 + d_r, w_last) * KROW + d_c16;
+      const int b = r * W4_NW + wave;  // 8-row block of the slab
+      c_xoff[r] = (uint32_t)min(b * 8 + d_r, x_last) * KROW + d_c16;
+      // SWIGLU: LDS weight row 128 wn + 64 h + c (h = 0 gate, 1 up) holds output column 64 wn + c of the tile, so that
+      // a wave has the gate and the up value of its own 64 columns: block b -> wn = b >> 4, h = (b >> 3) & 1.
+      const uint32_t wrow = SWIGLU ? (uint32_t)min((b >> 4) * 64 + (b & 7) * 8 + d_r, w_last) + (((b >> 3) & 1) ? (uint32_t)NCOLS : 0u)
+                                   : (uint32_t)min(b * 8 + d_r, w_last);
+      c_woff[r] = wrow * KROW + d_c16;
     }
   };
   auto cursor_next = [&]() {
@@ -833,9 +843,62 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
     }
 
     // Epilogue: lane holds y[m][n .. n + 3] for m = (2 i + wm) * 16 + lane % 16, n = (8 wn + j) * 16 + 4 (lane / 16).
-    const int rows_valid = t.h, cols_valid = min(N - t.n0, t.nc);
+    const int rows_valid = t.h, cols_valid = min(NCOLS - t.n0, t.nc);
     bf16_t* yg = yp + (int64_t)(t.row0 + t.m0) * p.ldy + (int64_t)t.g * p.col_block + t.n0;
-    if (p.vec_store && cols_valid == BN && p.ldy < (1 << 24)) {
+    if constexpr (SWIGLU) {
+      // acc[j][i], j = 0 .. 3: gate of output columns 64 wn + 16 j + 4 fq .. + 3; acc[j + 4][i]: up of the same columns.
+#pragma unroll
+      for (int i = 0; i < FMW; ++i) {
+        const int m = (i * 2 + wm) * 16 + fr;
+        if (m < rows_valid) {
+          bf16_t* yrow = yg + (int64_t)m * p.ldy;
+          u32x2_t q[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const f32x4_t gv = acc[j][i], uv = acc[j + 4][i];
+            // both products rounded to the 16-bit type first, as they are when the GEMM output is stored
+            const uint32_t g01 = pack_16x2<F16>(gv[0], gv[1]), g23 = pack_16x2<F16>(gv[2], gv[3]);
+            const uint32_t u01 = pack_16x2<F16>(uv[0], uv[1]), u23 = pack_16x2<F16>(uv[2], uv[3]);
+            const float g[4] = {f32_of_16<F16>((uint16_t)g01), f32_of_16<F16>((uint16_t)(g01 >> 16)),
+                                f32_of_16<F16>((uint16_t)g23), f32_of_16<F16>((uint16_t)(g23 >> 16))};
+            const float u[4] = {f32_of_16<F16>((uint16_t)u01), f32_of_16<F16>((uint16_t)(u01 >> 16)),
+                                f32_of_16<F16>((uint16_t)u23), f32_of_16<F16>((uint16_t)(u23 >> 16))};
+            float o[4];
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) o[rr] = g[rr] / (1.f + __expf(-g[rr])) * u[rr];
+            q[j][0] = pack_16x2<F16>(o[0], o[1]);
+            q[j][1] = pack_16x2<F16>(o[2], o[3]);
+          }
+          if (p.vec_store == 2 && cols_valid == TILE_COLS) {
+            // 16-byte stores: lanes l and l ^ 16 trade halves as in the plain epilogue below.
+            const bool odd = fq & 1;
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+              const uint32_t r0 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)(odd ? q[j][0] : q[j + 1][0]), 0x401F);
+              const uint32_t r1 = (uint32_t)__builtin_amdgcn_ds_swizzle((int)(odd ? q[j][1] : q[j + 1][1]), 0x401F);
+              u32x4_t o4;
+              if (odd) o4 = u32x4_t{r0, r1, q[j + 1][0], q[j + 1][1]}; else o4 = u32x4_t{q[j][0], q[j][1], r0, r1};
+              *(u32x4_t*)(yrow + wn * 64 + j * 16 + fq * 4 + (odd ? 16 - 4 : 0)) = o4;
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int n = wn * 64 + j * 16 + fq * 4;
+              if (p.vec_store && n + 3 < cols_valid) {
+                *(u32x2_t*)(yrow + n) = q[j];
+              } else {
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr)
+                  if (n + rr < cols_valid) {
+                    const uint32_t w2 = q[j][rr >> 1];
+                    ((uint16_t*)yrow)[n + rr] = (uint16_t)((rr & 1) ? (w2 >> 16) : (w2 & 0xFFFFu));
+                  }
+              }
+            }
+          }
+        }
+      }
+    } else if (p.vec_store && cols_valid == BN && p.ldy < (1 << 24)) {
       const uint32_t voff = (uint32_t)fr * (uint32_t)p.ldy + (uint32_t)(wn * FNW * 16 + fq * 4);
 #pragma unroll
       for (int i = 0; i < FMW; ++i) {
@@ -999,6 +1062,8 @@ __global__ __launch_bounds__(NT) void gg_bf16_pingpong(GgParams p) { pingpong_bo
 __global__ __launch_bounds__(NT) void gg_f16_pingpong(GgParams p) { pingpong_body<OP_F16>(p); }
 __global__ __launch_bounds__(W4_NT) void gg_bf16_fourwave(GgParams p) { pingpong_body<OP_BF16, true>(p); }
 __global__ __launch_bounds__(W4_NT) void gg_f16_fourwave(GgParams p) { pingpong_body<OP_F16, true>(p); }
+__global__ __launch_bounds__(W4_NT) void gg_bf16_fourwave_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU, true>(p); }
+__global__ __launch_bounds__(W4_NT) void gg_f16_fourwave_swiglu(GgParams p) { pingpong_body<OP_F16_SWIGLU, true>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
 __global__ __launch_bounds__(NT) void gg_f16_pingpong_swiglu(GgParams p) { pingpong_body<OP_F16_SWIGLU>(p); }
@@ -1020,6 +1085,12 @@ hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t st
 hipError_t gg_bf16_fourwave_launch(const GgParams& p, int num_wg, hipStream_t stream) {
   if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave, dim3(num_wg), dim3(W4_NT), 0, stream, p);
   else hipLaunchKernelGGL(gg_bf16_fourwave, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t gg_bf16_fourwave_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream) {
+  if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave_swiglu, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+  else hipLaunchKernelGGL(gg_bf16_fourwave_swiglu, dim3(num_wg), dim3(W4_NT), 0, stream, p);
   return hipGetLastError();
 }
 

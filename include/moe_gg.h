@@ -317,7 +317,8 @@ int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scale
 #define MOE_GG_GG_TILED_256_W4 6 /* 256x256 tiles on four waves of 128x128 outputs each (never chosen automatically) */
 #define MOE_GG_GG_FOURWAVE_256 7 /* the ping-pong kernel's tiles, tile order and slab stream on four waves of 128x128
                                     outputs each, loads and LDS reads placed behind single MFMAs (never chosen
-                                    automatically) */
+                                    automatically); while pinned, moe_gg_grouped_gemm_swiglu_bf16 / _f16 run their
+                                    four-wave form too */
 #define MOE_GG_OP_GG_FP8 1
 /* variants of MOE_GG_OP_GG_FP8 */
 #define MOE_GG_FP8_TILED_128 0       /* 128x128 tiles for every expert */

@@ -25,7 +25,7 @@ def one_case(rng):
     M = sum(sizes)
     N = int(rng.choice([64, 256, 320, 512, 768]))
     K = int(rng.choice([64, 128, 192]))
-    op = str(rng.choice(["bf16", "f16", "bf16w4", "f16w4", "swiglu", "gather", "fp8row", "fp8block"]))
+    op = str(rng.choice(["bf16", "f16", "bf16w4", "f16w4", "swiglu", "swigluw4", "gather", "fp8row", "fp8block"]))
     if op in ("bf16", "f16", "bf16w4", "f16w4"):     # ...w4: the same tiles and order on the four-wave kernel
         fp16 = op.startswith("f16")
         x = rng.integers(-4, 5, (M, K)).astype(np.float32)
@@ -44,11 +44,11 @@ def one_case(rng):
         good = (ms == np.array(sizes)).all()
         two_step = H.grouped_gemm_swiglu(H.gather_rows(tok, perm, k, n_valid=M), w, ms, n)
         good = bool(good and (H.grouped_gemm_swiglu_gather(tok, perm, k, w, ms, n)[:M] == two_step[:M]).all())
-    elif op == "swiglu":
+    elif op in ("swiglu", "swigluw4"):
         n = max(64, N // 2 // 4 * 4)
         x = rng.integers(-2, 3, (M, K)).astype(np.float32)
         w = (rng.integers(-2, 3, (G * 2 * n, K)) * 0.125).astype(np.float32)
-        got = H.from_bf16(H.grouped_gemm_swiglu(H.to_bf16(x), H.to_bf16(w), sizes, n))
+        got = H.from_bf16(H.grouped_gemm_swiglu(H.to_bf16(x), H.to_bf16(w), sizes, n, variant=7 if op == "swigluw4" else -1))
         want = O.silu_and_mul(O.grouped_gemm(x, w, sizes))
         good = not np.isnan(got).any() and np.abs(got - want).max() <= 1e-2 * max(1.0, np.abs(want).max())
     else:

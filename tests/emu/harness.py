@@ -149,13 +149,18 @@ def grouped_gemm_fp8(xq, wq, x_scale, w_scale, mode, m_sizes, N, variant=-1):
     return y
 
 
-def grouped_gemm_swiglu(x16, w16, m_sizes, n, fp16=False):
+def grouped_gemm_swiglu(x16, w16, m_sizes, n, fp16=False, variant=-1):
+    """variant 7 (MOE_GG_GG_FOURWAVE_256 pinned for the grouped GEMM) selects the four-wave form of the fused kernel."""
     L = lib()
     ms = i32(m_sizes)
     G, (M, K) = len(ms), x16.shape
     y = _full((M, n), NAN16, dtype=np.uint16)
     fn = L.moe_gg_grouped_gemm_swiglu_f16 if fp16 else L.moe_gg_grouped_gemm_swiglu_bf16
-    ok(fn(P(x16), P(w16), P(y), P(ms), G, M, n, K, n, None))
+    L.moe_gg_set_variant(OP_BF16, variant)
+    try:
+        ok(fn(P(x16), P(w16), P(y), P(ms), G, M, n, K, n, None))
+    finally:
+        L.moe_gg_set_variant(OP_BF16, -1)
     return y
 
 

@@ -76,6 +76,11 @@ static int one_shape(const char* op, int N, int K, int G, char** sizes) {
     Buf<uint8_t> ws(wsb + 512);
     uint8_t* wsp = ws.p() + ((256 - ((uintptr_t)ws.p() & 255)) & 255);
     check(moe_gg_grouped_gemm_backward_bf16(go.p(), N, 0, x.p(), w.p(), ms.p(), G, M, N, K, gx.p(), gw.p(), wsp, wsb, nullptr), op);
+  } else if (!std::strcmp(op, "swigluw4")) {  // the fused kernel on four waves (N = output columns n, w [G, 2 n, K])
+    auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * 2 * N * K);
+    moe_gg_set_variant(MOE_GG_OP_GG_BF16, MOE_GG_GG_FOURWAVE_256);
+    check(moe_gg_grouped_gemm_swiglu_bf16(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, nullptr), op);
+    moe_gg_set_variant(MOE_GG_OP_GG_BF16, -1);
   } else if (!std::strcmp(op, "swiglu")) {
     auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * 2 * N * K);
     check(moe_gg_grouped_gemm_swiglu_bf16(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, nullptr), op);

@@ -125,15 +125,21 @@ def test_fp8_every_kernel_variant(mode, variant, tile_order):
 
 
 @pytest.mark.parametrize("fp16", [False, True])
-def test_fused_silu_and_mul_gemm(fp16, tile_order):
+@pytest.mark.parametrize("variant", [-1, 7])
+@pytest.mark.parametrize("n,K", [(192, 128), (64, 64), (328, 192)])
+def test_fused_silu_and_mul_gemm(fp16, variant, n, K, tile_order):
+    """The eight-wave kernel and (variant 7) its four-wave form: against the oracle, and the two against each other
+    bit for bit (the same products in the same order, the same roundings)."""
     rng = np.random.default_rng(5)
-    n, K = 192, 128
     x = (rng.standard_normal((sum(SIZES), K)) * 0.5).astype(np.float32)
     w = (rng.standard_normal((4 * 2 * n, K)) * 0.1).astype(np.float32)
     x16, w16 = H.to16(x, fp16), H.to16(w, fp16)
-    got = H.from16(H.grouped_gemm_swiglu(x16, w16, SIZES, n, fp16), fp16)
+    got16 = H.grouped_gemm_swiglu(x16, w16, SIZES, n, fp16, variant=variant)
+    got = H.from16(got16, fp16)
     want = O.silu_and_mul(O.grouped_gemm(H.from16(x16, fp16), H.from16(w16, fp16), SIZES))
     np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2)
+    if variant == 7:
+        assert (got16 == H.grouped_gemm_swiglu(x16, w16, SIZES, n, fp16)).all()
 
 
 @pytest.mark.parametrize("fp16", [False, True])
@@ -434,7 +440,8 @@ def test_no_data_race_between_the_waves_of_a_workgroup():
               ("gather", "128", "128", "2", "3", ["530", "1", "300"]),
               ("fp8block", "384", "256", "1", "0", ["577", "33", "320"]), ("fp8row", "256", "128", "3", "9", ["129", "768", "1"]),
               ("f16", "384", "256", "2", "0", ["321", "511"]), ("bwd", "256", "128", "3", "4", ["300", "0", "41", "513"]),
-              ("bf16w4", "512", "192", "1", "0", ["530", "300", "0", "70"]), ("f16w4", "384", "64", "2", "6", ["321", "511", "1"])]
+              ("bf16w4", "512", "192", "1", "0", ["530", "300", "0", "70"]), ("f16w4", "384", "64", "2", "6", ["321", "511", "1"]),
+              ("swigluw4", "192", "128", "2", "1", ["300", "70", "0", "257"])]
     for i, (op, N, K, cus, seed, sizes) in enumerate(shapes):
         for order in ("0", "1"):
             procs.append(subprocess.Popen([exe, "shape", op, N, K] + sizes,

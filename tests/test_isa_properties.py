@@ -104,10 +104,10 @@ def test_hot_kernels_do_not_touch_scratch(asm):
 
 
 def test_four_wave_k_loop_is_what_the_source_spells_out(asm):
-    """gg_bf16_fourwave / gg_f16_fourwave: one K-step loop of 128 MFMAs with 32 fragment reads and 16 slab loads
+    """gg_bf16_fourwave / gg_f16_fourwave and their SiLU-and-mul forms: one K-step loop of 128 MFMAs with 32 fragment reads and 16 slab loads
     between them, no accumulator moves, no scratch access, no branch but the back edge (and the one around the load
     cursor's tile change), and never more than five other instructions between two MFMAs of a half step."""
-    for want in ("gg_bf16_fourwaveE", "gg_f16_fourwaveE"):
+    for want in ("gg_bf16_fourwaveE", "gg_f16_fourwaveE", "gg_bf16_fourwave_swigluE", "gg_f16_fourwave_swigluE"):
         (name, (lines, meta)), = [(n, v) for n, v in kernels(asm["gg_pingpong.hip"]).items() if want in n]
         main = [seg for seg in loops(lines) if count(seg, "v_mfma") == 128 and count(seg, "global_load_lds_dwordx4") == 16]
         assert main, name
