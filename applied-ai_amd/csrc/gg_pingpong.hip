@@ -685,13 +685,15 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
 // registers), and per 32-wide half step 16 fragment reads feed 64 MFMAs where a wave of the eight-wave kernel reads
 // 12 for 32: a third fewer LDS bytes per MFMA. A wave alone on its SIMD has nobody to fill the issue slots that an
 // instruction block without MFMAs leaves empty, so the order is written out one MFMA at a time (an MFMA holds the
-// matrix pipe for four issue slots: up to three other instructions fit behind it): in the first half of a K step
-// the 16 reads of the second half's fragments follow every third MFMA; then the wave waits for its reads and for
-// its loads of the next slab, and the workgroup's one barrier per K step publishes that slab and frees the buffer of
-// the present one; in the second half the 16 loads of the slab after next go into that buffer, one behind every
-// second MFMA of the first 32 (a K step and a half ahead of the wait that covers them), and the 16 reads of the
-// next step's first half follow every second MFMA of the last 32. A scheduling barrier after every such pair keeps
-// the compiler from collecting reads or loads into blocks. The slab stream runs through tile boundaries (the loads
+// matrix pipe for four issue slots: up to three other instructions fit behind it). Each half of a K step is two
+// blocks of 32 MFMAs: first those of the activation fragments 0 .. 3, which carry the other instructions, then those
+// of fragments 4 .. 7, which one uniform branch skips for a tile of at most 128 rows (low tiles, row pieces). First
+// half: the 16 reads of the second half's fragments follow every second MFMA of the first block; then the wave
+// waits for its reads and for its loads of the next slab, and the workgroup's one barrier per K step publishes that
+// slab and frees the buffer of the present one. Second half: behind the MFMAs of the first block alternate the 16
+// loads of the slab after next (into that buffer, more than a K step ahead of the wait that covers them) and the 16
+// reads of the next step's first half. A scheduling barrier after every such pair keeps the compiler from
+// collecting reads or loads into blocks. The slab stream runs through tile boundaries (the loads
 // and the reads for a tile's first step are issued in the last step of the tile before, and land during its
 // epilogue); behind the last tile the loads are still issued, with every lane's offset zero (one line per
 // instruction) into a buffer nobody reads again: one loop body, no branch around a load.
@@ -815,30 +817,52 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
 #pragma unroll
       for (int i = 0; i < FMW; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
+    // Activation fragments of this wave that hold rows of the tile: i with (2 i + wm) * 16 < t.h. A tile of at most
+    // 128 rows (low tile, row piece) has none beyond i = 3: the MFMAs of fragments 4 .. 7 form a block of their own
+    // in each half step, behind the block that carries the reads and loads, and one uniform branch skips it.
+    const bool upper = (moe_gg_cdiv(t.h, 16) - wm + 1) / 2 > 4;
     for (int kt = 0; kt < KT; ++kt, ++step) {
       const int cur = step & 1;
-      // First half: MFMAs on (wf0, xf0); (wf1, xf1) <- second half of the slab, one read behind every third MFMA, so
-      // that the last one is 18 MFMAs old when the wave waits for its reads.
+      // First half: MFMAs on (wf0, xf0); (wf1, xf1) <- second half of the slab, one read behind every second MFMA of
+      // the first block.
 #pragma unroll
-      for (int u = 0; u < 64; ++u) {
-        const int j = u >> 3, i = u & 7;
+      for (int u = 0; u < 32; ++u) {
+        const int j = u >> 2, i = u & 3;
         acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf0[j]), __builtin_bit_cast(u32x4_t, xf0[i]), acc[j][i]);
-        if (u % 3 == 0 && u / 3 < 16) read_one(cur, 1, u / 3, wf1, xf1);
+        if ((u & 1) == 0) read_one(cur, 1, u >> 1, wf1, xf1);
         __builtin_amdgcn_sched_barrier(0);
       }
+      if (upper) {
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+          const int j = u >> 2, i = 4 + (u & 3);
+          acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf0[j]), __builtin_bit_cast(u32x4_t, xf0[i]), acc[j][i]);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
       wait_lgkm0();   // this wave has read all it needs of the slab
       wait_vm<0>();   // its share of the next slab has landed
       __syncthreads();
-      // Second half: MFMAs on (wf1, xf1); the slab after next into the stage that is free now; (wf0, xf0) <- first
-      // half of the next slab.
+      // Second half: MFMAs on (wf1, xf1); behind the MFMAs of the first block, alternately, one of the 16 loads of the
+      // slab after next (into the stage that is free now; more than a K step ahead of the wait that covers them) and
+      // one of the 16 reads (wf0, xf0) <- first half of the next slab.
 #pragma unroll
-      for (int u = 0; u < 64; ++u) {
-        const int j = u >> 3, i = u & 7;
+      for (int u = 0; u < 32; ++u) {
+        const int j = u >> 2, i = u & 3;
         acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf1[j]), __builtin_bit_cast(u32x4_t, xf1[i]), acc[j][i]);
-        if (u < 32 && (u & 1) == 0) load_one(u >> 1, cur);
-        else if (u >= 32 && (u & 1) == 0) read_one(cur ^ 1, 0, (u - 32) >> 1, wf0, xf0);
+        __builtin_amdgcn_sched_barrier(0);           // the MFMA first, then what rides in its shadow
+        if ((u & 1) == 0) load_one(u >> 1, cur);   // five instructions with its offset mask and M0 write
+        else read_one(cur ^ 1, 0, u >> 1, wf0, xf0);   // one: three per MFMA on average, the slots an MFMA leaves
         __builtin_amdgcn_sched_barrier(0);
       }
+      if (upper) {
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+          const int j = u >> 2, i = 4 + (u & 3);
+          acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf1[j]), __builtin_bit_cast(u32x4_t, xf1[i]), acc[j][i]);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
       cursor_next();
     }
 
