@@ -8,7 +8,7 @@ rows), K=4096, N=14336, 8 experts. Prints ONE JSON line; the other benchmark con
 are measured in the same run and reported under "secondary" with their own rooflines.
 
 Order of work: every GPU measurement first (headline, the vendor library's dense GEMM, the secondary workloads), then
-the CPU baselines (headline first). A wall-clock budget (--budget-s, default 480 s) is checked before every secondary
+the CPU baselines (headline first). A wall-clock budget (--budget-s, default 300 s) is checked before every secondary
 workload and every CPU baseline; what does not fit is reported as {"skipped": "time budget"}, so the line is printed
 within minutes whatever the host's speed. SIGTERM / SIGINT print the line with what has been measured so far.
 """
@@ -657,7 +657,7 @@ def main():
     ap.add_argument("--moe-sweep", action="store_true",
                     help="also run the fused_moe sweep over m = 1 ... 512 (the shape of the reference's published sweep; context only)")
     ap.add_argument("--no-moe-sweep", action="store_true", help="accepted for compatibility: the sweep is off unless --moe-sweep is given")
-    ap.add_argument("--budget-s", type=float, default=480.0,
+    ap.add_argument("--budget-s", type=float, default=300.0,
                     help="wall-clock budget: secondary workloads and CPU baselines that would start after it are reported as skipped")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, so that a rocprofv3 --pmc run of this command sees a kernel of known traffic")
