@@ -446,3 +446,58 @@ def test_bench_refuses_more_than_one_gpu():
                        timeout=300)
     assert r.returncode != 0
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def _lockstep_traffic(lib, m_sizes, n_out, K, nwg=256, xcds=8, fused_gate_up=False, elem=2):
+    """Bytes that cross from the fabric into the XCDs' L2 caches when the workgroups of an XCD run their tiles in step
+    (sequence position by sequence position) and a slab is fetched once per XCD and position: the traffic that the
+    tile order itself implies, before any drift between workgroups. Returns (x bytes, w bytes, y bytes)."""
+    ms = np.ascontiguousarray(m_sizes, dtype=np.int32)
+    M = int(ms.sum())
+    bn = 128 if fused_gate_up else 256
+    cap = 1 << 18
+    out = np.zeros((cap, 6), dtype=np.int32)
+    n = lib.moe_gg_host_enumerate_tiles_two_lists(ms.ctypes.data_as(I32P), len(ms), M, n_out, 256, bn, nwg, xcds,
+                                                  out.ctypes.data_as(I32P), cap)
+    assert 0 < n < cap
+    seqs = {}
+    for wg, g, m0, h, n0, nc in out[:n].tolist():
+        seqs.setdefault(wg, []).append((g, m0, h, n0))
+    xb = wb = 0
+    for x in range(xcds):
+        for pos in range(max(len(v) for v in seqs.values())):
+            xs, ws = set(), set()
+            for wg, v in seqs.items():
+                if wg % xcds == x and pos < len(v):
+                    g, m0, h, n0 = v[pos]
+                    xs.add((g, m0, h))
+                    ws.add((g, n0))
+            xb += sum(h for _, _, h in xs) * K * elem
+            wb += sum(min(bn, n_out - n0) for _, n0 in ws) * K * elem * (2 if fused_gate_up else 1)
+    return xb, wb, M * n_out * 2
+
+
+def test_traffic_implied_by_the_tile_order(lib):
+    """What the two-list order costs in L2-side traffic at the benchmark shapes, from the host mirror alone. Mixtral
+    prefill (config 2): every weight tile once (0.94 GB) plus once more for the 224 low tiles of the four experts
+    that end 12-24 rows past a tile edge (0.47 GB), the activations once per XCD and round (7 x 67 MB), the output:
+    2.11 GB = 1.70 times the algorithmic 1.24 GB. (The counters read 2.18 GB per launch: the traffic above the
+    algorithmic bytes is the order's own, not workgroups drifting apart.)"""
+    cfg2 = [1012, 1039, 1048, 1036, 998, 1023, 1040, 996]
+    xb, wb, yb = _lockstep_traffic(lib, cfg2, 14336, 4096)
+    alg = 8192 * 4096 * 2 + 8 * 14336 * 4096 * 2 + yb
+    assert abs(wb - (8 + 4) * 14336 * 4096 * 2) < 0.01 * wb          # all weights once + four experts' a second time
+    assert abs(xb - 7 * 8192 * 4096 * 2) < 0.02 * xb                  # activations: once per XCD round of 8 column tiles
+    assert 1.65 < (xb + wb + yb) / alg < 1.75
+    # the fused gate/up GEMM of the layer: 128 output columns per tile, so twice the rounds and activation reads
+    xb, wb, yb = _lockstep_traffic(lib, cfg2, 14336, 4096, fused_gate_up=True)
+    alg = 8192 * 4096 * 2 + 8 * 2 * 14336 * 4096 * 2 + yb
+    assert abs(xb - 14 * 8192 * 4096 * 2) < 0.02 * xb and 1.75 < (xb + wb + yb) / alg < 1.9
+    # config 5 (fp8, 256 experts): dominated by weights that are read once; the order adds 7 %
+    from applied_ai_amd import configs
+
+    m5 = configs.cfg5_routing()[3].tolist()
+    xb, wb, yb = _lockstep_traffic(lib, m5, 4096, 7168, elem=1)
+    act = sum(1 for m in m5 if m > 0)
+    alg = 32768 * 7168 + act * 4096 * 7168 + yb
+    assert 1.03 < (xb + wb + yb) / alg < 1.10
