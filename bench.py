@@ -346,29 +346,32 @@ def hbm_roofline(kernel, byt, ms, traffic_key):
 # straight through the C ABI so that the ~10 us kernels are not timed through Python allocation overhead. Every
 # workload is a function of its own returning a list of JSON entries; one that raises is reported as an "error" entry
 # and the others still run.
-def wl_decode(torch, A, dev, lib, stream, cpu):
+def wl_decode(torch, A, dev, lib, stream, cpu, shapes=((4096, 14336), (14336, 4096))):
+    """shapes: (K, N) of the up- and the down-projection (the benchmark's by default; tests pass small ones)."""
     from applied_ai_amd import configs
 
     out = []
     c3 = configs.cfg3()
     m_sizes = c3["m_sizes"].tolist()
     ms_dev = c3["m_sizes"].to(dev)
+    G, R = len(m_sizes), sum(m_sizes)
     active = sum(1 for m in m_sizes if m > 0)
-    for name, key, K, N in (("up-proj K=4096 N=14336", "decode_up", 4096, 14336), ("down-proj K=14336 N=4096", "decode_down", 14336, 4096)):
-        x = torch.randn(64, K, device=dev).to(torch.bfloat16)
-        ws = [(torch.randn(8 * N, K, device=dev) * 0.02).to(torch.bfloat16) for _ in range(2)]
-        y = torch.empty(64, N, device=dev, dtype=torch.bfloat16)
+    for (name, key), (K, N) in zip((("up-proj", "decode_up"), ("down-proj", "decode_down")), shapes):
+        name = f"{name} K={K} N={N}"
+        x = torch.randn(R, K, device=dev).to(torch.bfloat16)
+        ws = [(torch.randn(G * N, K, device=dev) * 0.02).to(torch.bfloat16) for _ in range(2)]
+        y = torch.empty(R, N, device=dev, dtype=torch.bfloat16)
         state = {"i": 0}
 
         def call():
             w = ws[state["i"] & 1]
             state["i"] += 1
-            lib.moe_gg_grouped_gemm_bf16(x.data_ptr(), w.data_ptr(), y.data_ptr(), ms_dev.data_ptr(), 8, 64, N, K, N, 0, stream)
+            lib.moe_gg_grouped_gemm_bf16(x.data_ptr(), w.data_ptr(), y.data_ptr(), ms_dev.data_ptr(), G, R, N, K, N, 0, stream)
 
         st = event_stats(torch, call, 40, 6)
         ms = st["p50"]
-        byt = active * N * K * 2 + 64 * K * 2 + 64 * N * 2
-        e = {"workload": f"Mixtral decode bf16, T=32 top-2 (64 rows, m_sizes {m_sizes}), {name}"}
+        byt = active * N * K * 2 + R * K * 2 + R * N * 2
+        e = {"workload": f"Mixtral decode bf16, T=32 top-2 ({R} rows, m_sizes {m_sizes}), {name}"}
         e.update(timing_fields(st, "us"))
         e.update({"value": round(byt / ms / 1e6, 1), "unit": "GB/s", "roofline": hbm_roofline("gg_bf16_decode", byt, ms, key)})
         del ws
@@ -378,9 +381,8 @@ def wl_decode(torch, A, dev, lib, stream, cpu):
     return out
 
 
-def wl_w4a16(torch, A, dev, lib, stream, cpu):
+def wl_w4a16(torch, A, dev, lib, stream, cpu, K=4096, N=14336, copies=12):
     out = []
-    K, N, copies = 4096, 14336, 12
     qws = [torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device=dev) for _ in range(copies)]
     sc = (torch.rand(K // 128, N, device=dev) * 0.015 + 0.005).to(torch.bfloat16)
     qz = torch.randint(-2**31, 2**31 - 1, (K // 128, N // 8), dtype=torch.int32, device=dev)
@@ -402,7 +404,7 @@ def wl_w4a16(torch, A, dev, lib, stream, cpu):
 
         ms_hot = event_stats(torch, call_hot, 120, 24)["p50"]
         byt = K * N // 2 + (K // 128) * N * 2 + (K // 128) * N // 2 + M * K * 2 + M * N * 2
-        e = {"workload": f"W4A16 split-K M={M} K=4096 N=14336 group 128"}
+        e = {"workload": f"W4A16 split-K M={M} K={K} N={N} group 128"}
         e.update(timing_fields(st, "us"))
         e.update({"cache_hot_us_per_launch": round(ms_hot * 1e3, 2), "value": round(byt / ms / 1e6, 1), "unit": "GB/s",
                   "roofline": hbm_roofline("w4a16_splitk_g128", byt, ms, f"w4a16_m{M}")})
@@ -412,11 +414,11 @@ def wl_w4a16(torch, A, dev, lib, stream, cpu):
     return out
 
 
-def wl_w4a16_grouped(torch, A, dev, lib, stream, cpu):
+def wl_w4a16_grouped(torch, A, dev, lib, stream, cpu, K=4096, N=14336):
     from applied_ai_amd import configs
 
     out = []
-    K, N, E = 4096, 14336, 8
+    E = 8
     c3 = configs.cfg3()
     qwe = [torch.randint(-2**31, 2**31 - 1, (E, K // 8, N), dtype=torch.int32, device=dev) for _ in range(2)]
     sce = (torch.rand(E, K // 128, N, device=dev) * 0.015 + 0.005).to(torch.bfloat16)
@@ -471,13 +473,15 @@ def wl_w4a16_grouped(torch, A, dev, lib, stream, cpu):
     return out
 
 
-def wl_fp8_cfg5(torch, A, dev, lib, stream, cpu):
+def wl_fp8_cfg5(torch, A, dev, lib, stream, cpu, m5=None, N=4096, K=7168):
     """Config 5 with the inputs its definition states: x ~ N(0, 1) through the 1 x 128 quantiser, weights ~ N(0, 0.02)
-    through the 128 x 128 block quantiser (drawn and quantised expert by expert to bound memory)."""
+    through the 128 x 128 block quantiser (drawn and quantised expert by expert to bound memory). m5 / N / K: the
+    benchmark's routing and shape by default (tests pass small ones)."""
     from applied_ai_amd import configs
 
-    _, _, _, m5 = configs.cfg5_routing()
-    G, N, K = 256, 4096, 7168
+    if m5 is None:
+        _, _, _, m5 = configs.cfg5_routing()
+    G = int(m5.shape[0])
     M = int(m5.sum())
     f8 = torch.float8_e4m3fn
     gen = torch.Generator(device=dev).manual_seed(1005)
@@ -500,7 +504,7 @@ def wl_fp8_cfg5(torch, A, dev, lib, stream, cpu):
     active = int((m5 > 0).sum())
     byt = M * K + active * N * K + M * N * 2 + M * (K // 128) * 4 + active * (N // 128) * (K // 128) * 4
     flop = 2.0 * M * N * K
-    e = {"workload": "DeepSeek-V3-style fp8 e4m3 block-scaled grouped GEMM: 256 experts top-8, T=4096 (32768 rows, Zipf 1.1), K=7168, N=4096; "
+    e = {"workload": f"DeepSeek-V3-style fp8 e4m3 block-scaled grouped GEMM: {G} experts top-8, T=4096 ({M} rows, Zipf 1.1), K={K}, N={N}; "
                      "x ~ N(0,1) through the 1x128 quantiser, w ~ N(0,0.02) through the 128x128 block quantiser"}
     e.update(timing_fields(st, "ms"))
     e.update({"value": round(byt / ms / 1e6, 1), "unit": "GB/s", "tflops": round(flop / ms / 1e9, 1),
@@ -510,8 +514,8 @@ def wl_fp8_cfg5(torch, A, dev, lib, stream, cpu):
     return [e]
 
 
-def wl_moe_layer(torch, A, dev, lib, stream, cpu):
-    T, K, n, E, topk = 4096, 4096, 14336, 8, 2
+def wl_moe_layer(torch, A, dev, lib, stream, cpu, T=4096, K=4096, n=14336):
+    E, topk = 8, 2
     gen = torch.Generator(device=dev).manual_seed(1002)
     h = (torch.randn(T, K, device=dev, generator=gen) / 10).to(torch.bfloat16)
     w1 = torch.empty(E, 2 * n, K, device=dev, dtype=torch.bfloat16)
@@ -525,7 +529,7 @@ def wl_moe_layer(torch, A, dev, lib, stream, cpu):
     st = event_stats(torch, lambda: A.fused_moe(h, w1, w2, tw, ids), 10, 3, batches=5)
     ms = st["p50"]
     flop = 2.0 * T * topk * (2 * n * K + K * n)
-    e = {"workload": "Mixtral 8x7B MoE layer (fused_moe: group, gather, w1 GEMM, SiLU-and-mul, w2 GEMM, top-2 combine), T=4096, bf16",
+    e = {"workload": f"Mixtral 8x7B MoE layer (fused_moe: group, gather, w1 GEMM, SiLU-and-mul, w2 GEMM, top-2 combine), T={T}, K={K}, n={n}, bf16",
          "m_sizes": torch.bincount(ids.flatten().long(), minlength=E).tolist()}
     e.update(timing_fields(st, "ms"))
     e.update({"value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
@@ -537,10 +541,11 @@ def wl_moe_layer(torch, A, dev, lib, stream, cpu):
     return [e]
 
 
-def wl_backward(torch, A, dev, lib, stream, cpu):
-    G, M, N, K = 8, 8192, 14336, 4096
+def wl_backward(torch, A, dev, lib, stream, cpu, sizes=(1012, 1039, 1048, 1036, 998, 1023, 1040, 996), N=14336, K=4096):
+    """sizes: rows per expert (config 2's routing by default; tests pass small ones)."""
+    G, M = len(sizes), sum(sizes)
     gen = torch.Generator(device=dev).manual_seed(1002)
-    ms_dev = torch.tensor([1012, 1039, 1048, 1036, 998, 1023, 1040, 996], dtype=torch.int32, device=dev)  # config 2's routing
+    ms_dev = torch.tensor(list(sizes), dtype=torch.int32, device=dev)
     x = (torch.randn(M, K, device=dev, generator=gen) / 8).to(torch.bfloat16)
     w = torch.empty(G * N, K, device=dev, dtype=torch.bfloat16)
     for g in range(G):
@@ -558,36 +563,35 @@ def wl_backward(torch, A, dev, lib, stream, cpu):
     st = event_stats(torch, call, 10, 2, batches=5)
     ms = st["p50"]
     flop = 4.0 * M * N * K
-    e = {"workload": "grouped GEMM backward (grad_x and grad_w), Mixtral 8x7B w1 shape: 8192 rows, K=4096, N=14336, 8 experts, bf16"}
+    e = {"workload": f"grouped GEMM backward (grad_x and grad_w), Mixtral 8x7B w1 shape: {M} rows, K={K}, N={N}, {G} experts, bf16"}
     e.update(timing_fields(st, "ms"))
     e.update({"value": round(flop / ms / 1e9, 1), "unit": "TFLOP/s",
               "roofline": {"bound": "mfma", "kernel": "gg_bf16_pingpong_nt + gg_bf16_pingpong_wgrad_direct",
                            "achieved": round(flop / ms / 1e9, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None}})
     if cpu:
-        sizes = ms_dev.tolist()
-        e["_cpu"] = lambda: cpu_baseline_backward(sizes, N, K)
+        e["_cpu"] = lambda: cpu_baseline_backward(list(sizes), N, K)
     return [e]
 
 
-def wl_moe_sweep(torch, A, dev, lib, stream, cpu):
+def wl_moe_sweep(torch, A, dev, lib, stream, cpu, n=7168, k=4096, tokens=(1, 2, 4, 8, 16, 32, 64, 128, 256, 512)):
     """Context only, not a target: the sweep behind the one table of numbers the reference publishes for a
     neighbouring kernel (kernels/triton/inference/col_major_moe_gemm/test.csv:1-11): the fused MoE layer at
     m = 1 ... 512 tokens, n = 7168, k = 4096, 8 experts, top-2, fp16, reported with the reference's own formula
     2 m n k / t (perf_test_moe.py:123), which counts one m x n x k GEMM for the whole two-GEMM layer."""
-    n, k, E, topk = 7168, 4096, 8, 2
+    E, topk = 8, 2
     gen = torch.Generator(device=dev).manual_seed(3227)
     w1 = (torch.randn(E, 2 * n, k, device=dev, generator=gen) / 10).to(torch.float16)
     w2 = (torch.randn(E, k, n, device=dev, generator=gen) / 10).to(torch.float16)
     rows = []
-    for m in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512):
+    for m in tokens:
         a = (torch.randn(m, k, device=dev, generator=gen) / 10).to(torch.float16)
         score = torch.softmax(torch.randn(m, E, device=dev, generator=gen), dim=-1)
         tw, ids = torch.topk(score, topk)
         ids = ids.to(torch.int32)
         st = event_stats(torch, lambda: A.fused_moe(a, w1, w2, tw, ids), 40, 8)
         rows.append({"m": m, "us": round(st["p50"] * 1e3, 1), "tflops_reference_formula": round(2.0 * m * n * k / st["p50"] / 1e9, 3)})
-    return [{"workload": "fused_moe sweep as the reference's perf_test_moe.py runs it: n=7168, k=4096, 8 experts, top-2, fp16; "
+    return [{"workload": f"fused_moe sweep as the reference's perf_test_moe.py runs it: n={n}, k={k}, 8 experts, top-2, fp16; "
                          "TFLOPS = 2 m n k / t (one GEMM counted for the whole layer); context for test.csv:1-11, not a target",
              "timing": "median over 5 batches of 8 back-to-back calls through the Python entry function, HIP events",
              "rows": rows}]

@@ -56,7 +56,8 @@ def test_empty_batch_gives_zero_weight_gradient():
     nbytes = lib.moe_gg_grouped_gemm_backward_workspace(G, 1, N, K, 0)
     ws = torch.full((nbytes // 2,), float("nan"), dtype=torch.bfloat16, device="cuda")
     m = torch.zeros(G, dtype=torch.int32, device="cuda")
-    rc = lib.moe_gg_grouped_gemm_backward_bf16(None, N, 0, None, w.cuda().data_ptr(), m.data_ptr(), G, 0, N, K, None,
+    wd = w.cuda()     # bound to a name: the device copy must outlive the launch
+    rc = lib.moe_gg_grouped_gemm_backward_bf16(None, N, 0, None, wd.data_ptr(), m.data_ptr(), G, 0, N, K, None,
                                                gw.data_ptr(), ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()

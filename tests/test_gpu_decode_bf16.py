@@ -82,8 +82,8 @@ def test_forced_empty_experts_leave_rows_untouched():
     lib = A._lib.lib()
     lib.moe_gg_set_variant(0, DECODE)
     try:
-        rc = lib.moe_gg_grouped_gemm_bf16(x.data_ptr(), w.data_ptr(), y.data_ptr(),
-                                          torch.tensor(m_sizes, dtype=torch.int32, device="cuda").data_ptr(), G, M, N, K, N, 0,
+        ms = torch.tensor(m_sizes, dtype=torch.int32, device="cuda")   # bound to a name: it must outlive the launch
+        rc = lib.moe_gg_grouped_gemm_bf16(x.data_ptr(), w.data_ptr(), y.data_ptr(), ms.data_ptr(), G, M, N, K, N, 0,
                                           torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
     finally:

@@ -101,7 +101,8 @@ def test_fast_verification_shape_and_block_layout():
     check(x, w, m_sizes)
     ms = torch.tensor(m_sizes, dtype=torch.int32, device="cuda")
     yb = torch.full((M, N * G), float("nan"), dtype=torch.bfloat16, device="cuda")
-    rc = A._lib.lib().moe_gg_grouped_gemm_bf16(x.cuda().data_ptr(), w.cuda().data_ptr(), yb.data_ptr(), ms.data_ptr(),
+    xd, wd = x.cuda(), w.cuda()     # bound to names: the device copies must outlive the launch
+    rc = A._lib.lib().moe_gg_grouped_gemm_bf16(xd.data_ptr(), wd.data_ptr(), yb.data_ptr(), ms.data_ptr(),
                                                G, M, N, K, N * G, 1, torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
@@ -122,7 +123,8 @@ def test_rows_beyond_sum_are_untouched():
     x, w, _ = bf16_inputs(G, M, N, K, seed=14)
     ms = torch.tensor([10, 0, 30], dtype=torch.int32, device="cuda")
     y = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
-    rc = A._lib.lib().moe_gg_grouped_gemm_bf16(x.cuda().data_ptr(), w.cuda().data_ptr(), y.data_ptr(), ms.data_ptr(),
+    xd, wd = x.cuda(), w.cuda()     # bound to names: the device copies must outlive the launch
+    rc = A._lib.lib().moe_gg_grouped_gemm_bf16(xd.data_ptr(), wd.data_ptr(), y.data_ptr(), ms.data_ptr(),
                                                G, M, N, K, N, 0, torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()

@@ -1,0 +1,63 @@
+"""A selection of the `-m gpu` tests (and of the uncollected first-run tests, tests/wip_*.py) executed on the CPU:
+tests/emu/gpu_tests_on_emu.py loads the emulated build of the library in place of libmoe_gg.so and turns torch's "cuda"
+tensors into CPU tensors, so the GPU tests' own code - input construction, the Python entry functions, the ctypes
+calls, the oracle comparisons - runs end to end without a GPU. A mistake in a GPU test or in the host layer shows up
+here instead of on the GPU box. The selection is what the emulation carries in about a minute; the whole GPU suite,
+the benchmark-sized cases aside, passes the same way when given the time."""
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "tests", "emu"))
+
+import build_emu  # noqa: E402
+
+if not os.path.exists(build_emu.CXX):
+    pytest.skip("host clang++ of the ROCm toolchain not found: the emulated build needs it", allow_module_level=True)
+
+FILES = ["tests/test_gpu_routing.py", "tests/test_gpu_w4a16.py", "tests/test_gpu_w4a16_moe.py", "tests/test_gpu_decode_bf16.py",
+         "tests/test_zy_validate.py", "tests/test_gpu_moe_layer.py", "tests/wip_w4a16_variants.py"]
+# left out: benchmark-sized cases, and the tests of argument errors that need a real device to tell host from device memory
+SKIP = ("not config4 and not mixtral and not invalid and not rejects and not errors and not reference_test_shape and not 1500 "
+        "and not prefill_rows and not m_sizes5 and not sizes1-1032")
+
+
+def test_gpu_tests_pass_against_the_emulated_library():
+    build_emu.build()
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "emu", "gpu_tests_on_emu.py")] + FILES + ["-k", SKIP],
+                       cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=1500)
+    log = p.stdout.decode()
+    assert p.returncode == 0, log[-3000:]
+    m = re.search(r"(\d+) passed", log)
+    assert m and int(m.group(1)) >= 200, log[-1000:]
+
+
+def test_bench_py_runs_end_to_end_against_the_emulated_library():
+    """bench.py's main() and every secondary workload (with CPU baselines and the optional sweep) at reduced shapes,
+    through the real ctypes calls into the emulated kernels: one JSON line with the contract's fields, no workload
+    ending in an "error" entry, the baselines attached after the device legs."""
+    import json
+
+    build_emu.build()
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "emu", "bench_on_emu.py")], cwd=ROOT, stdout=subprocess.PIPE,
+                       stderr=subprocess.PIPE, timeout=1500)
+    assert p.returncode == 0, p.stderr.decode()[-3000:]
+    lines = [ln for ln in p.stdout.decode().splitlines() if ln.startswith("{")]
+    assert len(lines) == 1, p.stdout.decode()[-2000:]
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+                "dtype", "data", "config", "roofline", "cpu_baseline", "secondary", "dense_gemm_library", "wall_s"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 3 and d["unit"] == "TFLOP/s" and d["vs_baseline"] is None
+    assert {"bound", "achieved", "peak", "unit", "frac", "traffic"} <= set(d["roofline"])
+    assert {"value", "unit", "cores", "kind", "sample"} <= set(d["cpu_baseline"])
+    sec = d["secondary"]
+    assert len(sec) == 11 and not any("error" in e or "skipped" in e for e in sec), [e for e in sec if "error" in e or "skipped" in e]
+    with_roofline = [e for e in sec if "roofline" in e]
+    assert len(with_roofline) == 10 and all(e["roofline"]["bound"] in ("hbm", "mfma") for e in with_roofline)
+    assert sum("cpu_baseline" in e for e in sec) == 9          # all but the fp8-epilogue line and the sweep
+    assert sec[-1]["rows"] and sec[-1]["rows"][0]["m"] == 1
