@@ -61,3 +61,11 @@ def test_bench_py_runs_end_to_end_against_the_emulated_library():
     assert len(with_roofline) == 10 and all(e["roofline"]["bound"] in ("hbm", "mfma") for e in with_roofline)
     assert sum("cpu_baseline" in e for e in sec) == 9          # all but the fp8-epilogue line and the sweep
     assert sec[-1]["rows"] and sec[-1]["rows"][0]["m"] == 1
+
+
+def test_smoke_entry_point_against_the_emulated_library():
+    """__graft_entry__.smoke() (one small grouped GEMM through the Python entry function, checked against the oracle)."""
+    code = ("import sys; sys.path.insert(0, 'tests/emu'); sys.path.insert(0, '.'); import gpu_tests_on_emu as g; g.install(); "
+            "import __graft_entry__ as e; e.smoke()")
+    p = subprocess.run([sys.executable, "-c", code], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=600)
+    assert p.returncode == 0 and "smoke ok" in p.stdout.decode(), p.stdout.decode()[-2000:]
