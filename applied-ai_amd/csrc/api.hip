@@ -45,7 +45,7 @@ int current_device_info(const DeviceInfo** out) {
 // Variant bits of the W4A16 kernels (MOE_GG_OP_W4A16): 0 unless pinned.
 int w4_variant() {
   const int v = g_variant[MOE_GG_OP_W4A16].load();
-  return v < 0 ? 0 : v & 3;
+  return v < 0 ? 0 : v & 7;
 }
 
 // Tile order of the forward ping-pong kernels (MOE_GG_OP_TILE_ORDER): the split-tail order only when it is pinned.

@@ -79,7 +79,8 @@ struct W4Params {
 // variant: bits of MOE_GG_OP_W4A16's variant (0 = the kernels chosen by default), group size 128 and 16-bit output only:
 // 1: more than 32 rows (per expert, on average): passes of four activation fragments on four waves;
 // 2: up to 16 rows: two extra waves per workgroup that request every line of its weight strip ahead of the
-//    consumer waves, and lanes of activation rows that do not exist issue no loads.
+//    consumer waves, and lanes of activation rows that do not exist issue no loads;
+// 4: the activations of a quantisation group go through the wave's own LDS area (whole-line loads).
 hipError_t w4a16_splitk_launch(const W4Params& p, bool fp16, int variant, hipStream_t stream);
 
 // fp8 e4m3 grouped GEMM (gg_fp8.hip). scale_mode 0: x_scale [M], w_scale [G*N]; 1: x_scale [M, K/128],

@@ -343,13 +343,23 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
 // the way there: a launch of this size is bound by how early its bytes are requested, not by bandwidth. The
 // requests are loads into a scrap LDS area (no register destination). With WARM the consumer lanes of activation
 // rows beyond M also issue no loads (their fragment is zero) instead of re-reading the last row.
-template <bool FP16, int MF, int GA, int NWAVES, bool QOUT, int WARM = 0>  // GA = groups kept in flight
+//
+// STAGE: the activations of a quantisation group (16 MF rows x 256 bytes) reach the wave through its own LDS area
+// instead of as fragment loads. A fragment load takes 64 bytes of each of 16 rows (16 half lines per instruction, the
+// rows a whole K apart), and every workgroup of the launch pulls the same few rows out of the L2 that way: measured
+// 4.5 us per 16 rows, several times what the bytes cost. Staged, a load instruction takes 4 rows x 256 contiguous
+// bytes (8 whole lines), the same number of instructions and registers; the pieces are written to LDS when the group's
+// turn comes (16-byte chunks XOR-swizzled with the row, so that the fragment reads spread over all banks) and read
+// back as the MFMA fragments. The area is the wave's own: no barrier, the LDS queue of a wave is in order.
+template <bool FP16, int MF, int GA, int NWAVES, bool QOUT, int WARM = 0, bool STAGE = false>  // GA = groups kept in flight
 __global__ __launch_bounds__(64 * (NWAVES + WARM)) void w4a16_splitk_g128(W4Params p) {
   using E = Elem<FP16>;
   constexpr int SPG = 4, D = SPG * GA;
   constexpr bool MASK = WARM > 0;
+  static_assert(!STAGE || GA == 1, "the staged form keeps one group in flight");
   __shared__ __attribute__((aligned(16))) float red[NWAVES][MF][16 * 64];
   __shared__ __attribute__((aligned(256))) uint32_t scrap[WARM > 0 ? WARM : 1][64];
+  __shared__ __attribute__((aligned(16))) u32x4_t stage[STAGE ? NWAVES : 1][STAGE ? 16 * MF : 1][16];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -400,6 +410,10 @@ __global__ __launch_bounds__(64 * (NWAVES + WARM)) void w4a16_splitk_g128(W4Para
   const int32_t* zp;
   const uint16_t* arow[MF];
   bool row_ok[MF];          // MASK: the lane's row of fragment i exists
+  // STAGE: piece q (0 .. 4 MF - 1) of a group is rows 4 q + lane / 16 of the pass, 16-byte chunk lane % 16.
+  const int sr = lane >> 4, sc16 = lane & 15;
+  const uint16_t* srow = nullptr;  // row sr of the pass, chunk sc16, K offset 0
+  int srows = 0;                   // rows of the pass that exist
   auto setup = [&](int pass) {
     const int mb = pass / CB * (16 * MF), n0 = (blockIdx.x * CB + pass % CB) * 64;
     qw = v.qweight + n0 + 4 * fr;
@@ -410,20 +424,35 @@ __global__ __launch_bounds__(64 * (NWAVES + WARM)) void w4a16_splitk_g128(W4Para
       arow[i] = v.a + (int64_t)min(mb + i * 16 + fr, M - 1) * K + fq * 8;
       row_ok[i] = mb + i * 16 + fr < M;
     }
+    if constexpr (STAGE) {
+      srow = v.a + (int64_t)(mb + sr) * K + sc16 * 8;
+      srows = M - mb;
+    }
   };
   u32x4_t wb[D], xr[D][MF];
   u32x2_t sg[GA];
   uint32_t zg[GA];
+  // STAGE: all pieces of the wave's group gi (the gi-th of its own) into xr; rows that do not exist are zero.
+  auto load_pieces = [&](int gi) {
+    const int64_t koff = ((int64_t)gi * NWAVES + wave) * 128;  // first k of the group
+#pragma unroll
+    for (int q = 0; q < 4 * MF; ++q) {
+      xr[q / MF][q % MF] = u32x4_t{0u, 0u, 0u, 0u};
+      if (4 * q + sr < srows) xr[q / MF][q % MF] = *(const u32x4_t*)(srow + (int64_t)(4 * q) * K + koff);
+    }
+  };
   auto load_step = [&](int d, int t) {
     const int ks = kstep(t);
     wb[d] = *(const u32x4_t*)(qw + (int64_t)(ks * 4 + fq) * N);
+    if constexpr (!STAGE) {  // staged: the activations come group by group (load_pieces)
 #pragma unroll
-    for (int i = 0; i < MF; ++i) {
-      if (MASK) {
-        xr[d][i] = u32x4_t{0u, 0u, 0u, 0u};
-        if (row_ok[i]) xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
-      } else {
-        xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
+      for (int i = 0; i < MF; ++i) {
+        if (MASK) {
+          xr[d][i] = u32x4_t{0u, 0u, 0u, 0u};
+          if (row_ok[i]) xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
+        } else {
+          xr[d][i] = *(const u32x4_t*)(arow[i] + ks * 32);
+        }
       }
     }
   };
@@ -439,6 +468,9 @@ __global__ __launch_bounds__(64 * (NWAVES + WARM)) void w4a16_splitk_g128(W4Para
       for (int e = 0; e < SPG; ++e)
         if (q * SPG + e < steps) load_step(q * SPG + e, q * SPG + e);
       if (q < my_groups) load_group(q, q);
+      if constexpr (STAGE) {
+        if (q < my_groups) load_pieces(q);
+      }
     }
   };
   setup(0);
@@ -466,13 +498,27 @@ __global__ __launch_bounds__(64 * (NWAVES + WARM)) void w4a16_splitk_g128(W4Para
             for (int j = 0; j < 4; ++j) accg[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             accs[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
           }
+          if constexpr (STAGE) {
+            // The group's pieces from registers into the wave's LDS area (row 4 p + sr, chunk sc16 at slot
+            // sc16 ^ (row % 16)), then the registers take the next group's. The lanes of a wave read what other
+            // lanes of it wrote: LDS serves a wave's accesses in order, and the two wave barriers keep the compiler
+            // from moving the reads of one group and the writes of the next across each other.
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int pc = 0; pc < 4 * MF; ++pc) stage[wave][4 * pc + sr][sc16 ^ ((4 * pc + sr) & 15)] = xr[pc / MF][pc % MF];
+            __builtin_amdgcn_wave_barrier();
+            if (more) load_pieces(gi + GA);
+          }
 #pragma unroll
           for (int e = 0; e < SPG; ++e) {
             const int d = q * SPG + e;
             u32x4_t xb[MF];
 #pragma unroll
             for (int i = 0; i < MF; ++i) {
-              const u32x4_t xv = xr[d][i];
+              // fragment i of step e: row 16 i + fr, k chunk 4 e + fq of the group
+              u32x4_t xv;
+              if constexpr (STAGE) xv = stage[wave][16 * i + fr][(4 * e + fq) ^ fr];
+              else xv = xr[d][i];
               xb[i][0] = __builtin_amdgcn_perm(xv[2], xv[0], 0x05040100u);  // k 0, 4
               xb[i][1] = __builtin_amdgcn_perm(xv[2], xv[0], 0x07060302u);  // k 1, 5
               xb[i][2] = __builtin_amdgcn_perm(xv[3], xv[1], 0x05040100u);  // k 2, 6
@@ -536,14 +582,20 @@ hipError_t launch(const W4Params& p, int variant, hipStream_t stream) {
   if constexpr (!QOUT) {
     // Selectable variants (MOE_GG_OP_W4A16), group size 128: never chosen by default. The warm-up waves go with the
     // one-fragment kernel only: ten waves leave a wave 168 registers, which the two-fragment kernel (232) does not
-    // fit, and the four-fragment kernel needs a four-wave workgroup for its 430.
+    // fit, and the four-fragment kernel needs a four-wave workgroup for its 430. Bit 4: activations staged through LDS.
     constexpr int WARM = 2;
-    if (p.group_size == 128 && (variant & 1) && M > 32) {
-      hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 4, 1, 4, false>), grid, dim3(64 * 4), 0, stream, p);
-      return hipGetLastError();
-    }
-    if (p.group_size == 128 && (variant & 2) && M <= 16) {
-      hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES, false, WARM>), grid, dim3(64 * (WAVES + WARM)), 0, stream, p);
+    const bool one_pass = (variant & 1) && M > 32, warm = (variant & 2) && M <= 16, staged = (variant & 4) != 0;
+    if (p.group_size == 128 && (one_pass || warm || staged)) {
+      if (one_pass) {
+        if (staged) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 4, 1, 4, false, 0, true>), grid, dim3(64 * 4), 0, stream, p);
+        else hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 4, 1, 4, false>), grid, dim3(64 * 4), 0, stream, p);
+      } else if (M <= 16) {
+        if (warm && staged) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES, false, WARM, true>), grid, dim3(64 * (WAVES + WARM)), 0, stream, p);
+        else if (warm) hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES, false, WARM>), grid, dim3(64 * (WAVES + WARM)), 0, stream, p);
+        else hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 1, 1, WAVES, false, 0, true>), grid, block, 0, stream, p);
+      } else {
+        hipLaunchKernelGGL((w4a16_splitk_g128<FP16, 2, 1, WAVES, false, 0, true>), grid, block, 0, stream, p);
+      }
       return hipGetLastError();
     }
   }

@@ -339,6 +339,9 @@ int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scale
 #define MOE_GG_W4_WARMUP 2   /* up to 16 rows per expert: two extra waves per workgroup request the workgroup's weight
                                 lines ahead of the consumer waves; lanes of activation rows that do not exist issue
                                 no loads */
+#define MOE_GG_W4_STAGED 4   /* activations reach a wave through its own LDS area: loads of 4 rows x 256 contiguous bytes,
+                                written to LDS and read back as MFMA fragments, instead of fragment loads of
+                                16 rows x 64 bytes */
 int moe_gg_set_variant(int op, int variant);
 int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                 int block_n, int num_workgroups, int xcds, int32_t* out,

@@ -114,7 +114,7 @@ def c_w4a16(rng):
     sc = (2.0 ** rng.integers(-3, 1, (E, K // gs, N))).astype(np.float32)
     a = ints(rng, (M, K), -2, 3)
     a16, s16 = H.to16(a, fp16), H.to16(sc, fp16)
-    variant = int(rng.choice([-1, 1, 2, 3]))       # MOE_GG_OP_W4A16: the selectable kernels too
+    variant = int(rng.integers(-1, 8))              # MOE_GG_OP_W4A16: the selectable kernels too
     what = ("w4a16", kind, M if sizes is None else sizes, N, K, gs, fp16, zero_offset, variant)
     if sizes is None:
         c = H.w4a16(a16, qw[0], s16[0], qz[0], gs, zero_offset, fp16, variant=variant)

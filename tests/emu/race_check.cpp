@@ -175,7 +175,7 @@ int main(int argc, char** argv) {
     auto a = bf16_small((size_t)80 * K);
     Buf<uint16_t> c((size_t)80 * N);
     const int Ms[] = {1, 16, 33, 70};
-    for (int variant = 0; variant <= 3; ++variant) {  // the default kernels, then the selectable ones
+    for (int variant = 0; variant <= 7; ++variant) {  // the default kernels, then the selectable ones
       moe_gg_set_variant(MOE_GG_OP_W4A16, variant);
       for (int M : Ms)
         check(moe_gg_w4a16_splitk(a.p(), qw.p(), sc.p(), qz.p(), c.p(), M, N, K, 128, 1, MOE_GG_DTYPE_BF16, nullptr), "w4a16_splitk (M = 1, 16, 33, 70; every variant)");

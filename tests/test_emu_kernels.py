@@ -214,12 +214,13 @@ def test_w4a16_splitk(M, N, K, gs, fp16):
     assert exact16(c, O.w4a16_gemm(a, qw[0], sc[0], qz[0], gs, 1), fp16)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("M,N,K,fp16", [(1, 256, 512, False), (5, 128, 1024, True), (16, 192, 256, False), (17, 64, 512, False),
                                         (33, 128, 512, False), (64, 64, 1024, True), (70, 64, 256, False), (130, 128, 512, False)])
 def test_w4a16_selectable_variants(M, N, K, fp16, variant):
     """MOE_GG_OP_W4A16: 1 = passes of four activation fragments on four waves for more than 32 rows, 2 = warm-up waves
-    and masked activation rows for up to 16 rows; row counts outside a variant's range take the default kernels."""
+    and masked activation rows for up to 16 rows, 4 = activations staged through the wave's LDS area (every row count);
+    row counts outside the range of bits 1 and 2 take the default kernels (or their staged forms)."""
     rng = np.random.default_rng(100 * variant + M)
     qw, qz, sc = w4_inputs(rng, 1, K, N, 128)
     a = ints(rng, (M, K), -2, 3)
@@ -227,10 +228,10 @@ def test_w4a16_selectable_variants(M, N, K, fp16, variant):
     assert exact16(c, O.w4a16_gemm(a, qw[0], sc[0], qz[0], 128, 1), fp16)
 
 
-@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("variant", [1, 2, 4, 5, 6])
 def test_w4a16_grouped_selectable_variants(variant):
     rng = np.random.default_rng(40 + variant)
-    sizes = [40, 0, 70, 33, 30] if variant == 1 else [3, 0, 16, 12, 1]       # average rows per expert picks the kernel
+    sizes = [40, 0, 70, 33, 30] if variant & 1 else [3, 0, 16, 12, 1]       # average rows per expert picks the kernel
     N, K = 128, 512
     qw, qz, sc = w4_inputs(rng, len(sizes), K, N, 128)
     a = ints(rng, (sum(sizes), K), -2, 3)

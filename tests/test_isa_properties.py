@@ -99,8 +99,10 @@ def test_hot_kernels_do_not_touch_scratch(asm):
             assert scratch_bytes(meta) == 0, name
             vgpr = int(re.search(r"\.amdhsa_next_free_vgpr (\d+)", meta).group(1))
             four_waves = "ELi4ELi1ELi4E" in name        # <FP16, MF = 4, GA = 1, NWAVES = 4, ...>: one wave per SIMD
-            warm = name.endswith("ELi2EEEv8W4Params")   # ten waves: three on some SIMDs
+            warm = re.search(r"ELi2ELb[01]EEEv8W4Params$", name) is not None   # ten waves: three on some SIMDs
             assert vgpr <= (512 if four_waves else 168 if warm else 256), (name, vgpr)
+            lds = int(re.search(r"\.amdhsa_group_segment_fixed_size (\d+)", meta).group(1))
+            assert lds <= 160 << 10, (name, lds)        # the staged forms add 4 KB of LDS per wave and fragment
 
 
 def test_four_wave_k_loop_is_what_the_source_spells_out(asm):
