@@ -1,6 +1,7 @@
 """Benchmark of the MoE grouped-GEMM hot path on one MI355X.
 
 python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary] [--no-cpu-baseline] [--moe-sweep] [--budget-s S]
+                [--pin OP=VARIANT ...]
 
 A step is one pass of the hot path over one batch of synthetic, HBM-resident input. The headline workload is the
 configuration the metric is quoted on: Mixtral 8x7B w1 grouped GEMM, bf16, T=4096 tokens top-2 (8192 expert-sorted
@@ -651,6 +652,27 @@ def printable(out):
     return json.dumps(clean(out))
 
 
+# moe_gg_set_variant ops by name (include/moe_gg.h) and the headline kernel behind each MOE_GG_OP_GG_BF16 variant
+PIN_OPS = {"gg_bf16": 0, "gg_fp8": 1, "tile_order": 2, "w4a16": 3}
+HEADLINE_KERNELS = {-1: "gg_bf16_pingpong", 0: "gg_bf16_pingpong", 1: "gg_bf16_persistent<256x256>", 2: "gg_bf16_persistent<128x128>",
+                    3: "gg_bf16_persistent<64x128>", 4: "gg_bf16_generic", 5: "gg_bf16_decode",
+                    6: "gg_bf16_persistent<256x256, four waves>", 7: "gg_bf16_fourwave"}
+
+
+def parse_pins(items):
+    """{"op name": variant} from --pin OP=VARIANT arguments."""
+    pins = {}
+    for item in items:
+        op, sep, variant = item.partition("=")
+        if not sep or op not in PIN_OPS:
+            sys.exit(f"--pin {item}: expected OP=VARIANT with OP one of {', '.join(PIN_OPS)}")
+        try:
+            pins[op] = int(variant)
+        except ValueError:
+            sys.exit(f"--pin {item}: VARIANT must be an integer")
+    return pins
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -663,6 +685,9 @@ def main():
     ap.add_argument("--no-moe-sweep", action="store_true", help="accepted for compatibility: the sweep is off unless --moe-sweep is given")
     ap.add_argument("--budget-s", type=float, default=300.0,
                     help="wall-clock budget: secondary workloads and CPU baselines that would start after it are reported as skipped")
+    ap.add_argument("--pin", action="append", default=[], metavar="OP=VARIANT",
+                    help="pin a kernel variant for the whole run (moe_gg_set_variant): OP is gg_bf16, gg_fp8, tile_order or w4a16; "
+                         "for timing and profiling the selectable kernels, e.g. --pin gg_bf16=7 --pin tile_order=1. The line says what was pinned")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, so that a rocprofv3 --pmc run of this command sees a kernel of known traffic")
     args = ap.parse_args()
@@ -670,6 +695,9 @@ def main():
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
     budget = Budget(args.budget_s)
+    pins = parse_pins(args.pin)
+    if pins:
+        TRAFFIC.clear()   # the committed traffic figures were measured on the library's automatic choice of kernels
 
     import signal
 
@@ -692,6 +720,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    for op, variant in pins.items():
+        rc = A._lib.lib().moe_gg_set_variant(PIN_OPS[op], variant)
+        assert rc == 0, (op, variant, rc)
     c = configs.cfg2()
     x = c["x_sorted"].to(dev)
     w = c["w"].to(dev)
@@ -743,7 +774,7 @@ def main():
         "pct_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
         "roofline": {
             "bound": "mfma",
-            "kernel": "gg_bf16_pingpong",
+            "kernel": HEADLINE_KERNELS.get(pins.get("gg_bf16", 0), f"gg_bf16 variant {pins.get('gg_bf16')}"),
             "achieved": round(achieved, 2),
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
@@ -772,6 +803,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     out["traffic_measured_at"] = TRAFFIC_COMMIT
+    if pins:
+        # not the library's automatic choice: the figures of this line belong to the pinned kernels
+        out["pinned_variants"] = pins
     cpu = not args.no_cpu_baseline
     if cpu:
         out["_cpu"] = lambda: cpu_baseline_prefill(c)

@@ -3,7 +3,7 @@ main() with a small stand-in for the headline configuration and every secondary 
 CPU baselines included. Prints the JSON line main() printed. What it checks is bench.py's own code - tensor shapes,
 ctypes argument lists, the JSON fields - not speed. Test infrastructure only.
 
-    python tests/emu/bench_on_emu.py
+    python tests/emu/bench_on_emu.py [further bench.py arguments, e.g. --pin gg_bf16=7 --pin w4a16=7]
 """
 import functools
 import os
@@ -48,7 +48,7 @@ def main():
     bench.OPTIONAL = (functools.partial(bench.wl_moe_sweep, n=128, k=64, tokens=(1, 8)),)
     for f in bench.SECONDARY + bench.OPTIONAL:   # the error entry of a failing workload names the function
         f.__name__ = f.func.__name__
-    sys.argv = ["bench.py", "--steps", "3", "--warmup", "1", "--moe-sweep"]
+    sys.argv = ["bench.py", "--steps", "3", "--warmup", "1", "--moe-sweep"] + sys.argv[1:]   # e.g. --pin gg_bf16=7
     bench.main()
 
 

@@ -175,3 +175,16 @@ def test_main_prints_one_line_with_the_gpu_numbers_first(monkeypatch, capsys):
     assert d["steps"] == 3 and d["n_gpus"] == 1 and d["vs_baseline"] is None and d["config"]["m_sizes"] == [10, 14]
     assert d["roofline"]["bound"] == "mfma" and d["cpu_baseline"] == {"value": 0.1, "cores": 1}
     assert d["secondary"] == [{"workload": "w", "value": 1.0, "cpu_baseline": {"value": 0.5}}]
+
+
+def test_pin_arguments():
+    assert bench.parse_pins([]) == {}
+    assert bench.parse_pins(["gg_bf16=7", "tile_order=1", "w4a16=5"]) == {"gg_bf16": 7, "tile_order": 1, "w4a16": 5}
+    assert bench.HEADLINE_KERNELS[7] == "gg_bf16_fourwave" and set(bench.PIN_OPS.values()) == {0, 1, 2, 3}
+    for bad in (["nothing=1"], ["gg_bf16"], ["gg_bf16=x"]):
+        try:
+            bench.parse_pins(bad)
+        except SystemExit as e:
+            assert "--pin" in str(e)
+        else:
+            raise AssertionError(bad)
