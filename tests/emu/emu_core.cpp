@@ -9,6 +9,7 @@
 //
 // Environment: EMU_CUS   number of compute units hipGetDeviceProperties reports (default 8)
 //              EMU_XCDS  number of XCDs hipDeviceGetAttribute reports (default 8)
+//              EMU_LDS_POISON  set: every workgroup starts with LDS full of 0xFF bytes (NaN patterns)
 //              EMU_DMA   "late" (default): a global->LDS load writes LDS when its wave's counter wait retires it,
 //                        the latest moment the hardware allows; "early": at issue, the earliest
 //              EMU_SEED  non-zero: fibers are resumed in a shuffled order (changes which wave runs ahead)
@@ -324,10 +325,15 @@ void launch(dim3 grid, dim3 block, size_t dyn, const std::function<void()>& body
   TSAN(g_tsan_main = __tsan_get_current_fiber());
   TSAN(__tsan_release(&g_tsan_launch));
   unsigned wg = 0;
+  const bool poison = getenv("EMU_LDS_POISON") != nullptr;
   for (unsigned z = 0; z < grid.z; ++z)
     for (unsigned y = 0; y < grid.y; ++y)
       for (unsigned x = 0; x < grid.x; ++x, ++wg) {
         blockIdx = dim3(x, y, z);
+        // EMU_LDS_POISON: a workgroup starts with all of LDS holding 0xFF bytes (NaN as bf16, fp16 and fp32), as
+        // far from a previous workgroup's leftovers as it gets: an output that depends on LDS bytes its own
+        // workgroup never wrote comes out as NaN.
+        if (poison) memset(__start_emu_lds, 0xFF, (size_t)(__stop_emu_lds - __start_emu_lds));
         run_workgroup(g_seed ? g_seed * 2654435761u + wg * 40503u + 1u : 0u);
       }
   g_cur = nullptr;
