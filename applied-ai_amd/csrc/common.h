@@ -46,6 +46,13 @@ template <bool F16> DEVINL f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
+// A point where all lanes of a wave are known to be together again: the top of a loop whose body ends in lane-masked
+// blocks. Nothing on the GPU (no instruction, no constraint on the compiler's scheduling). A host build of the kernels
+// that runs the lanes of a wave as separate threads of control defines wave_whole() as the place where they meet.
+#ifndef wave_whole
+DEVINL void wave_whole() {}
+#endif
+
 DEVINL int lane_id() { return threadIdx.x & 63; }
 DEVINL int wave_id() { return threadIdx.x >> 6; }
 

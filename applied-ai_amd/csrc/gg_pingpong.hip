@@ -412,6 +412,7 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
 
   int step = 0;
   for (int r = 0; r < sh.n_my; ++r) {
+    wave_whole();  // the lanes left the epilogue's masked store blocks at different points
     const TileRef tr = tile_ref(r);
     const MoeGgTile& t = tr.t;
     const int KT = tr.KT;

@@ -20,6 +20,10 @@ OUT = os.environ.get("EMU_OUT") or os.path.join(HERE, "_build")
 CXX = "/opt/rocm/llvm/bin/clang++"
 FLAGS = ["-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-attributes", "-Wno-unused-value",
          "-Wno-ignored-attributes", "-I", os.path.join(HERE, "include"), "-I", CSRC]
+# EMU_UBSAN (with an EMU_OUT of its own): the kernels trap on misaligned vector accesses, out-of-range shifts, signed
+# overflow and indices beyond a fixed-size array (no sanitizer runtime needed: the checks end in a trap instruction).
+if os.environ.get("EMU_UBSAN"):
+    FLAGS += ["-fsanitize=alignment,shift,signed-integer-overflow,bounds,null", "-fsanitize-trap=all"]
 
 
 def _split_top(s, sep):

@@ -105,6 +105,7 @@ template <class T> inline T atomicAdd(T* p, T v) { return __atomic_fetch_add(p, 
 #define __expf(x) expf(x)
 #define __builtin_amdgcn_readfirstlane(v) emu::readfirstlane((int)(v))
 #define __builtin_amdgcn_wave_barrier() emu::wave_join()
+#define wave_whole() emu::wave_join()   // common.h's marker of a point where a wave's lanes are together again
 #define __builtin_amdgcn_sched_barrier(m) ((void)0)
 #define __builtin_amdgcn_sched_group_barrier(a, b, c) ((void)0)
 #define __builtin_amdgcn_s_setprio(p) ((void)0)
