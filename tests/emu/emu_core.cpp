@@ -335,6 +335,10 @@ void launch(dim3 grid, dim3 block, size_t dyn, const std::function<void()>& body
         // workgroup never wrote comes out as NaN.
         if (poison) memset(__start_emu_lds, 0xFF, (size_t)(__stop_emu_lds - __start_emu_lds));
         run_workgroup(g_seed ? g_seed * 2654435761u + wg * 40503u + 1u : 0u);
+        // ... and nothing may have been written behind the launch's dynamic LDS size (the GPU drops such writes)
+        if (poison)
+          for (size_t b = dyn; b < sizeof(g_dyn_lds); ++b)
+            if ((unsigned char)g_dyn_lds[b] != 0xFF) fail("write beyond the dynamic LDS size of the launch");
       }
   g_cur = nullptr;
 }
