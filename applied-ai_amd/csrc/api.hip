@@ -186,8 +186,9 @@ static int grouped_gemm_16(const void* x, const void* w, void* y, const int32_t*
       return (int)gg_bf16_decode_tails_launch(p, s);
     }
     case MOE_GG_GG_FOURWAVE_256:
+    case MOE_GG_GG_FOURWAVE_TALL:
       if (!pingpong_ok) return MOE_GG_EUNSUPPORTED;
-      return (int)gg_bf16_fourwave_launch(p, num_wg, s);
+      return (int)gg_bf16_fourwave_launch(p, variant == MOE_GG_GG_FOURWAVE_TALL, num_wg, s);
     case MOE_GG_GG_TILED_256: return (int)gg_bf16_tiled_launch(p, 256, num_wg, s);
     case MOE_GG_GG_TILED_256_W4: return (int)gg_bf16_tiled_launch(p, GG_TILED_256_FOUR_WAVES, num_wg, s);
     case MOE_GG_GG_TILED_128: return (int)gg_bf16_tiled_launch(p, 128, num_wg, s);
@@ -393,9 +394,10 @@ static int grouped_gemm_swiglu_16(const void* x, const void* w, void* y, const i
   p.gather_perm = perm;
   p.gather_k = k;
   p.gather_rows = (int)T;
-  // The four-wave form when that kernel is pinned for the grouped GEMM (it has no row gather).
-  if (!perm && g_variant[MOE_GG_OP_GG_BF16].load() == MOE_GG_GG_FOURWAVE_256)
-    return (int)gg_bf16_fourwave_swiglu_launch(p, num_wg, (hipStream_t)stream);
+  // The four-wave forms when one of them is pinned for the grouped GEMM (they have no row gather).
+  const int pinned = g_variant[MOE_GG_OP_GG_BF16].load();
+  if (!perm && (pinned == MOE_GG_GG_FOURWAVE_256 || pinned == MOE_GG_GG_FOURWAVE_TALL))
+    return (int)gg_bf16_fourwave_swiglu_launch(p, pinned == MOE_GG_GG_FOURWAVE_TALL, num_wg, (hipStream_t)stream);
   return (int)gg_bf16_pingpong_swiglu_launch(p, num_wg, (hipStream_t)stream);
 }
 
@@ -724,7 +726,8 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
       low_off[MOE_GG_MAX_GROUPS_ABI + 1];
   // The lists of a launch that computes its low tiles itself, in the tile order that is in force
   // (MOE_GG_OP_TILE_ORDER); the decode below is the kernels' own.
-  const bool split = split_tails_on() != 0;
+  const bool tall = g_variant[MOE_GG_OP_TILE_ORDER].load() == MOE_GG_ORDER_TALL_TILES;
+  const bool split = !tall && split_tails_on() != 0;
   const int ntn = moe_gg_cdiv(N, block_n);
   int64_t r = 0;
   int nl = 0, ns = 0;
@@ -732,8 +735,8 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
     row_off[g] = (int32_t)r; long_off[g] = nl; low_off[g] = ns;
     const int m = moe_gg_clamp_rows(m_sizes_host[g], r, M);
     r += m;
-    nl += moe_gg_long_row_tiles2(m, block_m, split) * ntn;
-    ns += moe_gg_low_row_tiles2(m, block_m, split) * ntn;
+    nl += (tall ? moe_gg_long_row_tiles_tall(m, block_m) : moe_gg_long_row_tiles2(m, block_m, split)) * ntn;
+    ns += (tall ? moe_gg_low_row_tiles_tall(m, block_m) : moe_gg_low_row_tiles2(m, block_m, split)) * ntn;
   }
   row_off[G] = (int32_t)r; long_off[G] = nl; low_off[G] = ns;
   const int tail_s = split ? moe_gg_tail_pieces_low(nl, ns, num_workgroups) : moe_gg_tail_pieces(nl, num_workgroups);
@@ -750,8 +753,10 @@ int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, in
       const int L = moe_gg_tile_of(wg, num_workgroups, xcds, moe_gg_seq_round(seq, n_my, n_low, phase));
       if (written >= max_tiles) return written;
       if (L >= total) return MOE_GG_EINVAL;  // cannot happen
-      const MoeGgListTile t = moe_gg_two_list_decode(row_off, long_off, low_off, G, L, long_ids, tail_first, tail_s,
-                                                     block_m, block_n, split);
+      const MoeGgListTile t = tall ? moe_gg_two_list_decode_tall(row_off, long_off, low_off, G, L, long_ids, tail_first,
+                                                                 tail_s, block_m, block_n)
+                                   : moe_gg_two_list_decode(row_off, long_off, low_off, G, L, long_ids, tail_first, tail_s,
+                                                            block_m, block_n, split);
       int32_t* o = out + (size_t)written * 6;
       o[0] = wg; o[1] = t.g; o[2] = t.m0; o[3] = t.h; o[4] = t.n0; o[5] = block_n;
       ++written;

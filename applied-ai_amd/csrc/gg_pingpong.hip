@@ -54,6 +54,7 @@ constexpr int WM = 2;            // wave = wm + 2 * wn; group = wave >> 2 = wn >
 constexpr int FM = 8, FN = 4;    // 16-row activation / weight fragments per wave
 constexpr int X_BYTES = BM * 128;
 constexpr int STAGE = (BM + BN) * 128;
+constexpr int TALL_BYTES = MOE_GG_TALL_ROWS * 128;  // per stage: the slab rows of a tall tile's rows 256 .. 287 (four-wave kernel)
 constexpr int SCALE_BYTES = 2048;  // per stage: 256 activation scales, then 4 x 256 B of weight-block scales
 
 // Operand kinds.
@@ -700,13 +701,20 @@ DEVINL void run_group(const GgParams& p, const Shared& sh) {
 // instruction) into a buffer nobody reads again: one loop body, no branch around a load.
 constexpr int W4_NW = 4, W4_NT = 64 * W4_NW, W4_FM = 8, W4_FN = 8;
 
-template <int OP>
+// TALL: tiles of up to BM + MOE_GG_TALL_ROWS rows (moe_gg_tall_tail: the few rows behind a group's last full row tile
+// ride along with that tile instead of streaming the weight tile a second time as a low tile). A wave then has a ninth
+// activation fragment, tile rows 256 + 16 wm .. + 15: its slab rows live in a 4 KB area per stage behind the two
+// stages (one more load instruction per wave and slab, issued only for tall tiles), its fragment reads are issued for
+// every tile (they cost two reads per K step and spare the loop a second condition), and its eight MFMAs per half step
+// form a third block that one uniform branch skips for tiles of at most 256 rows.
+template <int OP, bool TALL = false>
 DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
   static_assert(OP == OP_BF16 || OP == OP_F16 || OP == OP_BF16_SWIGLU || OP == OP_F16_SWIGLU,
                 "forward product on 16-bit floats, plain or with SiLU-and-mul in the epilogue");
   constexpr bool F16 = op_f16(OP);
   constexpr bool SWIGLU = op_swiglu(OP);
   constexpr int FMW = W4_FM, FNW = W4_FN;
+  constexpr int FMA = FMW + (TALL ? 1 : 0);  // activation fragments a wave holds accumulators for
   constexpr int TILE_COLS = SWIGLU ? BN / 2 : BN;  // output columns of a tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -748,6 +756,8 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
   const char* c_xg = xp;
   const char* c_wg = wp;
   uint32_t c_xoff[8], c_woff[8];
+  uint32_t c_xoff_tall = 0;  // TALL: the wave's 8 rows of tile rows 256 .. 287
+  bool c_tall = false;       // TALL: the cursor's tile has such rows
   uint32_t c_keep = ~0u;  // zero behind the last tile
   int c_seq = 0, c_kt = 0;
   auto cursor_tile = [&](int seq) {
@@ -755,11 +765,16 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
     c_kt = 0;
     if (seq >= sh.n_my) {  // behind the last tile: the pointers stay at the last tile's (in bounds), offsets zero
       c_keep = 0u;
+      c_tall = false;
       return;
     }
     const Tile t = tile_at(seq);
     // w_last: last valid weight row of the tile; SWIGLU: last valid output column (a gate row and an up row each)
     const int x_last = max(t.h, 1) - 1, w_last = max(min(NCOLS - t.n0, t.nc), 1) - 1;
+    if constexpr (TALL) {
+      c_tall = t.h > BM;
+      c_xoff_tall = (uint32_t)min(BM + wave * 8 + d_r, x_last) * KROW + d_c16;
+    }
     c_xg = uni_ptr(xp + (int64_t)(t.row0 + t.m0) * KROW);
     c_wg = uni_ptr(wp + ((int64_t)t.g * N + t.n0) * KROW);
 #pragma unroll
@@ -782,30 +797,52 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
     if (r < 8) dma16(c_xg + c_kt * 128, c_xoff[r] & c_keep, lb + r * W4_NW * 1024);
     else dma16(c_wg + c_kt * 128, c_woff[r - 8] & c_keep, lb + X_BYTES + (r - 8) * W4_NW * 1024);
   };
+  // TALL: the seventeenth load of a slab, rows 256 + 8 wave .. + 7 into the stage's extra area (tall tiles only)
+  auto load_tall = [&](int buf) {
+    if (c_tall) dma16(c_xg + c_kt * 128, c_xoff_tall, lds_base + 2 * STAGE + buf * TALL_BYTES + wave * 1024);
+  };
 
-  bf16x8_t wf0[FNW], xf0[FMW], wf1[FNW], xf1[FMW];
-  auto read_one = [&](int buf, int half, int r, bf16x8_t (&wf)[FNW], bf16x8_t (&xf)[FMW]) {
+  bf16x8_t wf0[FNW], xf0[FMA], wf1[FNW], xf1[FMA];
+  auto read_one = [&](int buf, int half, int r, bf16x8_t (&wf)[FNW], bf16x8_t (&xf)[FMA]) {
     // read r of a half step's 16: the activation fragments first (the first eight MFMAs use all of them)
     const char* st = sh.lds + buf * STAGE;
     const int ro = half ? (rd0 ^ 64) : rd0;
     if (r < FMW) xf[r] = *(const bf16x8_t*)(st + (r * 2 + wm) * 2048 + ro);
     else wf[r - FMW] = *(const bf16x8_t*)(st + X_BYTES + (wn * FNW + r - FMW) * 2048 + ro);
   };
+  // TALL: fragment 8 (tile rows 256 + 16 wm .. + 15) of a half step, from the stage's extra area
+  auto read_tall = [&](int buf, int half, bf16x8_t (&xf)[FMA]) {
+    xf[FMA - 1] = *(const bf16x8_t*)(sh.lds + 2 * STAGE + buf * TALL_BYTES + wm * 2048 + (half ? (rd0 ^ 64) : rd0));
+  };
 
-  f32x4_t acc[FNW][FMW];
+  f32x4_t acc[FNW][FMA];
+  // TALL: the ninth fragment's 32 accumulation registers do not fit the AGPRs, which the other 256 fill, and the
+  // compiler selects one form of MFMA for the whole function (AGPR accumulators: it would copy these 32 registers into
+  // spare AGPRs and back around every MFMA). So their MFMAs are written out with VGPR accumulators. The compiler does
+  // not know the instruction, i.e. it tracks the operands (it waits for the LDS reads behind a and b) but inserts none
+  // of the wait states an MFMA result needs before another kind of instruction reads it: a dependent MFMA on the same
+  // accumulator follows 72 MFMAs later at the earliest (no wait needed), and the epilogue's first read is kept 32
+  // issue slots away by the s_nops behind the K loop.
+  auto mfma_vgpr = [&](const bf16x8_t& a, const bf16x8_t& b, f32x4_t& c) {
+    if constexpr (F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  };
 
   // Stream start: slabs 0 and 1 in flight, first fragments read.
   cursor_tile(0);
 #pragma unroll
   for (int r = 0; r < 16; ++r) load_one(r, 0);
+  if constexpr (TALL) load_tall(0);
   cursor_next();
 #pragma unroll
   for (int r = 0; r < 16; ++r) load_one(r, 1);
+  if constexpr (TALL) load_tall(1);
   cursor_next();
-  wait_vm<16>();  // slab 0 (loads return in order)
+  wait_vm<16>();  // slab 0 (loads return in order; TALL: 16 or 17 are behind it, so at least slab 0 has landed)
   __syncthreads();
 #pragma unroll
   for (int r = 0; r < 16; ++r) read_one(0, 0, r, wf0, xf0);
+  if constexpr (TALL) read_tall(0, 0, xf0);
 
   int step = 0;  // K steps done, over all tiles: slab `step` sits in stage step & 1
   for (int seq = 0; seq < sh.n_my; ++seq) {
@@ -816,12 +853,13 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
 #pragma unroll
     for (int j = 0; j < FNW; ++j)
 #pragma unroll
-      for (int i = 0; i < FMW; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int i = 0; i < FMA; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     // Activation fragments of this wave that hold rows of the tile: i with (2 i + wm) * 16 < t.h. A tile of at most
     // 128 rows (low tile, row piece) has none beyond i = 3: the MFMAs of fragments 4 .. 7 form a block of their own
     // in each half step, behind the block that carries the reads and loads, and one uniform branch skips it.
     const bool upper = (moe_gg_cdiv(t.h, 16) - wm + 1) / 2 > 4;
+    const bool tall = TALL && t.h > BM;  // the ninth fragment has rows (for wm = 1: if more than 16)
     for (int kt = 0; kt < KT; ++kt, ++step) {
       const int cur = step & 1;
       // First half: MFMAs on (wf0, xf0); (wf1, xf1) <- second half of the slab, one read behind every second MFMA of
@@ -833,11 +871,22 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
         if ((u & 1) == 0) read_one(cur, 1, u >> 1, wf1, xf1);
         __builtin_amdgcn_sched_barrier(0);
       }
+      if constexpr (TALL) {
+        read_tall(cur, 1, xf1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (upper) {
 #pragma unroll
         for (int u = 0; u < 32; ++u) {
           const int j = u >> 2, i = 4 + (u & 3);
           acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf0[j]), __builtin_bit_cast(u32x4_t, xf0[i]), acc[j][i]);
+        }
+      }
+      if constexpr (TALL) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (tall) {
+#pragma unroll
+          for (int j = 0; j < FNW; ++j) mfma_vgpr(wf0[j], xf0[FMA - 1], acc[j][FMA - 1]);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -856,6 +905,11 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
         else read_one(cur ^ 1, 0, u >> 1, wf0, xf0);   // one: three per MFMA on average, the slots an MFMA leaves
         __builtin_amdgcn_sched_barrier(0);
       }
+      if constexpr (TALL) {
+        load_tall(cur);
+        read_tall(cur ^ 1, 0, xf0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (upper) {
 #pragma unroll
         for (int u = 0; u < 32; ++u) {
@@ -863,8 +917,19 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
           acc[j][i] = mfma_16x16x32<F16>(__builtin_bit_cast(u32x4_t, wf1[j]), __builtin_bit_cast(u32x4_t, xf1[i]), acc[j][i]);
         }
       }
+      if constexpr (TALL) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (tall) {
+#pragma unroll
+          for (int j = 0; j < FNW; ++j) mfma_vgpr(wf1[j], xf1[FMA - 1], acc[j][FMA - 1]);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
       cursor_next();
+    }
+    if constexpr (TALL) {
+      // the results of the last hand-written MFMAs must not be read before they are written (see mfma_vgpr)
+      if (tall) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     }
 
     // Epilogue: lane holds y[m][n .. n + 3] for m = (2 i + wm) * 16 + lane % 16, n = (8 wn + j) * 16 + 4 (lane / 16).
@@ -873,7 +938,7 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
     if constexpr (SWIGLU) {
       // acc[j][i], j = 0 .. 3: gate of output columns 64 wn + 16 j + 4 fq .. + 3; acc[j + 4][i]: up of the same columns.
 #pragma unroll
-      for (int i = 0; i < FMW; ++i) {
+      for (int i = 0; i < FMA; ++i) {
         const int m = (i * 2 + wm) * 16 + fr;
         if (m < rows_valid) {
           bf16_t* yrow = yg + (int64_t)m * p.ldy;
@@ -926,7 +991,7 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
     } else if (p.vec_store && cols_valid == BN && p.ldy < (1 << 24)) {
       const uint32_t voff = (uint32_t)fr * (uint32_t)p.ldy + (uint32_t)(wn * FNW * 16 + fq * 4);
 #pragma unroll
-      for (int i = 0; i < FMW; ++i) {
+      for (int i = 0; i < FMA; ++i) {
         const int mrow = (i * 2 + wm) * 16;
         bf16_t* ybase = yg + (int64_t)mrow * p.ldy;  // uniform
         if (mrow + fr < rows_valid) {
@@ -960,7 +1025,7 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < FMW; ++i) {
+      for (int i = 0; i < FMA; ++i) {
         const int m = (i * 2 + wm) * 16 + fr;
         if (m < rows_valid) {
           bf16_t* yrow = yg + (int64_t)m * p.ldy;
@@ -981,10 +1046,11 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
 
 // FOURWAVE: the workgroup is four waves running run_fourwave (one wave per SIMD, 128 x 128 outputs each) instead of the
 // two groups of four above; tables, tile order and LDS stages are the same.
-template <int OP, bool FOURWAVE = false>
+template <int OP, bool FOURWAVE = false, bool TALL = false>
 DEVINL void pingpong_body(const GgParams& p) {
+  static_assert(!TALL || FOURWAVE, "tall tiles are the four-wave kernel's");
   constexpr int NTB = FOURWAVE ? W4_NT : NT;  // threads of the workgroup
-  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + (OP == OP_FP8_BLOCK ? 2 * SCALE_BYTES : 0)];
+  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + (OP == OP_FP8_BLOCK ? 2 * SCALE_BYTES : 0) + (TALL ? 2 * TALL_BYTES : 0)];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t tile_off[MOE_GG_MAX_GROUPS + 1];
   __shared__ int32_t part_off[MOE_GG_MAX_GROUPS + 1];
@@ -1017,8 +1083,14 @@ DEVINL void pingpong_body(const GgParams& p) {
       if (apart) split = false;
       __syncthreads();  // the tables are rewritten below
     }
+    if constexpr (TALL) {
+      split = false;  // the lists of moe_gg_tall_tail
+      build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles_tall(rows, BM) * ntn : 0; });
+      build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles_tall(rows, BM) * ntn : 0; });
+    } else {
     build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles2(rows, BM, split) * ntn : 0; });
     build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles2(rows, BM, split) * ntn : 0; });
+    }
     total_low = apart ? 0 : uni(part_off[p.G]);
     total = uni(tile_off[p.G]);
   }
@@ -1028,7 +1100,7 @@ DEVINL void pingpong_body(const GgParams& p) {
   // round alone (moe_gg_tail_pieces), or, with p.split_tails, as many as make the busiest workgroup's load smallest
   // with the second list dealt behind them, moe_gg_tail_pieces_low.)
   const bool fwd = OP != OP_BF16_WGRAD && OP != OP_BF16_WGRAD_DIRECT;
-  const int tail_s = !fwd ? 1 : p.split_tails ? moe_gg_tail_pieces_low(total, total_low, nwg) : moe_gg_tail_pieces(total, nwg);
+  const int tail_s = !fwd ? 1 : (p.split_tails && !TALL) ? moe_gg_tail_pieces_low(total, total_low, nwg) : moe_gg_tail_pieces(total, nwg);
   const int tail_first = moe_gg_tail_first_s(total, nwg, tail_s);
   const int long_ids = moe_gg_long_ids_s(total, nwg, tail_s);
   const int low_ids = total_low;
@@ -1065,7 +1137,9 @@ DEVINL void pingpong_body(const GgParams& p) {
       // Long tiles (the last round cut into row pieces when it is sparsely filled), then the second list.
       // (Cutting few low tiles into column pieces for more workgroups was measured: no gain, a low tile is bound
       // by the per-step cost of the K loop, not by the bytes it streams.)
-      const MoeGgListTile lt = moe_gg_two_list_decode(row_off, tile_off, part_off, p.G, L, long_ids, tail_first, tail_s, BM, TC, split);
+      MoeGgListTile lt;
+      if constexpr (TALL) lt = moe_gg_two_list_decode_tall(row_off, tile_off, part_off, p.G, L, long_ids, tail_first, tail_s, BM, TC);
+      else lt = moe_gg_two_list_decode(row_off, tile_off, part_off, p.G, L, long_ids, tail_first, tail_s, BM, TC, split);
       g = lt.g; m0 = lt.m0; h = lt.h; n0 = lt.n0;
     }
     seq_tab[2 * i] = g | (h << 16) | ((nc / 32) << 26);
@@ -1075,7 +1149,7 @@ DEVINL void pingpong_body(const GgParams& p) {
 
   Shared sh{row_off, tile_off, part_off, seq_tab, lds, n_my};
   if constexpr (FOURWAVE) {
-    run_fourwave<OP>(p, sh);
+    run_fourwave<OP, TALL>(p, sh);
   } else {
     const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
     if (grp == 0) run_group<0, OP>(p, sh);
@@ -1089,6 +1163,10 @@ __global__ __launch_bounds__(W4_NT) void gg_bf16_fourwave(GgParams p) { pingpong
 __global__ __launch_bounds__(W4_NT) void gg_f16_fourwave(GgParams p) { pingpong_body<OP_F16, true>(p); }
 __global__ __launch_bounds__(W4_NT) void gg_bf16_fourwave_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU, true>(p); }
 __global__ __launch_bounds__(W4_NT) void gg_f16_fourwave_swiglu(GgParams p) { pingpong_body<OP_F16_SWIGLU, true>(p); }
+__global__ __launch_bounds__(W4_NT) void gg_bf16_fourwave_tall(GgParams p) { pingpong_body<OP_BF16, true, true>(p); }
+__global__ __launch_bounds__(W4_NT) void gg_f16_fourwave_tall(GgParams p) { pingpong_body<OP_F16, true, true>(p); }
+__global__ __launch_bounds__(W4_NT) void gg_bf16_fourwave_tall_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU, true, true>(p); }
+__global__ __launch_bounds__(W4_NT) void gg_f16_fourwave_tall_swiglu(GgParams p) { pingpong_body<OP_F16_SWIGLU, true, true>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad(GgParams p) { pingpong_body<OP_BF16_WGRAD>(p); }
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu(GgParams p) { pingpong_body<OP_BF16_SWIGLU>(p); }
 __global__ __launch_bounds__(NT) void gg_f16_pingpong_swiglu(GgParams p) { pingpong_body<OP_F16_SWIGLU>(p); }
@@ -1107,14 +1185,20 @@ hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t st
   return hipGetLastError();
 }
 
-hipError_t gg_bf16_fourwave_launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+hipError_t gg_bf16_fourwave_launch(const GgParams& p, bool tall, int num_wg, hipStream_t stream) {
+  if (tall) {
+    if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave_tall, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+    else hipLaunchKernelGGL(gg_bf16_fourwave_tall, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+  } else if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave, dim3(num_wg), dim3(W4_NT), 0, stream, p);
   else hipLaunchKernelGGL(gg_bf16_fourwave, dim3(num_wg), dim3(W4_NT), 0, stream, p);
   return hipGetLastError();
 }
 
-hipError_t gg_bf16_fourwave_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave_swiglu, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+hipError_t gg_bf16_fourwave_swiglu_launch(const GgParams& p, bool tall, int num_wg, hipStream_t stream) {
+  if (tall) {
+    if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave_tall_swiglu, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+    else hipLaunchKernelGGL(gg_bf16_fourwave_tall_swiglu, dim3(num_wg), dim3(W4_NT), 0, stream, p);
+  } else if (p.fp16) hipLaunchKernelGGL(gg_f16_fourwave_swiglu, dim3(num_wg), dim3(W4_NT), 0, stream, p);
   else hipLaunchKernelGGL(gg_bf16_fourwave_swiglu, dim3(num_wg), dim3(W4_NT), 0, stream, p);
   return hipGetLastError();
 }

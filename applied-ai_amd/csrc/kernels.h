@@ -44,9 +44,10 @@ int gg_bf16_tiled_block_n(int block_m);
 // and honours p.skip_rows.
 hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream);
 // The same tiles, tile order and LDS stages on four waves of 128 x 128 outputs each (bf16 / fp16 forward only).
-hipError_t gg_bf16_fourwave_launch(const GgParams& p, int num_wg, hipStream_t stream);
+// tall: tiles of up to 256 + 32 rows (the lists of moe_gg_tall_tail)
+hipError_t gg_bf16_fourwave_launch(const GgParams& p, bool tall, int num_wg, hipStream_t stream);
 // ... and its form with SiLU-and-mul in the epilogue (the arguments of gg_bf16_pingpong_swiglu_launch, no row gather).
-hipError_t gg_bf16_fourwave_swiglu_launch(const GgParams& p, int num_wg, hipStream_t stream);
+hipError_t gg_bf16_fourwave_swiglu_launch(const GgParams& p, bool tall, int num_wg, hipStream_t stream);
 hipError_t gg_fp8_pingpong_launch(const GgParams& p, int scale_mode, int num_wg, hipStream_t stream);
 hipError_t gg_bf16_generic_launch(const GgParams& p, hipStream_t stream);
 // Small-M split-K kernel; nf = 16-row weight fragments per wave (2 or 4), mf = 16-row activation

@@ -286,3 +286,63 @@ MOE_GG_HD MoeGgListTile moe_gg_two_list_decode(const int32_t* row_off, const int
   return t;
 }
 
+// ---- Tall tiles ------------------------------------------------------------------------------------
+// Lists of a kernel whose tiles may hold up to BM + MOE_GG_TALL_ROWS rows: a group with at least one full row tile and
+// at most MOE_GG_TALL_ROWS rows behind its last one gets no tile for those rows; its last full tile takes them along.
+// (Such a tail would otherwise stream the group's whole weight tile a second time, for a few rows, in every column
+// tile.) Everything else is the two-list order above without split tails.
+#define MOE_GG_TALL_ROWS 32
+MOE_GG_HD bool moe_gg_tall_tail(int rows, int BM) {
+  const int full = rows / BM, rem = rows - full * BM;
+  return full >= 1 && rem > 0 && rem <= MOE_GG_TALL_ROWS;
+}
+MOE_GG_HD int moe_gg_long_row_tiles_tall(int rows, int BM) {
+  return moe_gg_tall_tail(rows, BM) ? rows / BM : moe_gg_long_row_tiles(rows, BM);
+}
+MOE_GG_HD int moe_gg_low_row_tiles_tall(int rows, int BM) {
+  return moe_gg_tall_tail(rows, BM) ? 0 : moe_gg_low_row_tiles(rows, BM);
+}
+// moe_gg_two_list_decode for these lists: h may reach BM + MOE_GG_TALL_ROWS; of a tall tile cut into row pieces the
+// last piece takes the extra rows.
+MOE_GG_HD MoeGgListTile moe_gg_two_list_decode_tall(const int32_t* row_off, const int32_t* long_off, const int32_t* low_off,
+                                                    int G, int L, int long_ids, int tail_first, int tail_s, int BM, int TC) {
+  MoeGgListTile t;
+  int rows;
+  if (L < long_ids) {
+    int piece = 0;
+    if (L >= tail_first) {  // a piece of a tile of the last round
+      piece = (L - tail_first) % tail_s;
+      L = tail_first + (L - tail_first) / tail_s;
+    }
+    t.g = moe_gg_find_group(long_off, G, L);
+    const int idx = L - long_off[t.g];
+    rows = row_off[t.g + 1] - row_off[t.g];
+    int nf = moe_gg_long_row_tiles_tall(rows, BM);
+    if (nf < 1) nf = 1;
+    const int tn = idx / nf;
+    t.n0 = tn * TC;
+    t.m0 = (idx - tn * nf) * BM;
+    t.h = rows - t.m0 < BM ? rows - t.m0 : BM;
+    if (moe_gg_tall_tail(rows, BM) && t.m0 + BM == rows / BM * BM) t.h = rows - t.m0;  // the last full tile and the tail
+    if (tail_s > 1 && L >= tail_first) {
+      const int rv = t.h;
+      int off;
+      moe_gg_piece_rows(rv < BM ? rv : BM, tail_s, piece, &off, &t.h);
+      if (piece == tail_s - 1 && rv > BM) t.h += rv - BM;
+      if (t.h > 0) t.m0 += off;  // a piece without rows keeps the tile's first row: its loads must stay in bounds
+    }
+  } else {
+    const int Lp = L - long_ids;
+    t.g = moe_gg_find_group(low_off, G, Lp);
+    rows = row_off[t.g + 1] - row_off[t.g];
+    t.n0 = (Lp - low_off[t.g]) * TC;
+    t.m0 = rows / BM * BM;
+    t.h = rows - t.m0;
+  }
+  if (t.h < 0) t.h = 0;
+  if (t.m0 < 0 || t.m0 >= rows) { t.m0 = 0; t.h = 0; }
+  if (t.m0 + t.h > rows) t.h = rows - t.m0;
+  if (t.h > BM + MOE_GG_TALL_ROWS) t.h = BM + MOE_GG_TALL_ROWS;
+  return t;
+}
+

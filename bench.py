@@ -656,7 +656,7 @@ def printable(out):
 PIN_OPS = {"gg_bf16": 0, "gg_fp8": 1, "tile_order": 2, "w4a16": 3}
 HEADLINE_KERNELS = {-1: "gg_bf16_pingpong", 0: "gg_bf16_pingpong", 1: "gg_bf16_persistent<256x256>", 2: "gg_bf16_persistent<128x128>",
                     3: "gg_bf16_persistent<64x128>", 4: "gg_bf16_generic", 5: "gg_bf16_decode",
-                    6: "gg_bf16_persistent<256x256, four waves>", 7: "gg_bf16_fourwave"}
+                    6: "gg_bf16_persistent<256x256, four waves>", 7: "gg_bf16_fourwave", 8: "gg_bf16_fourwave_tall"}
 
 
 def parse_pins(items):

@@ -319,6 +319,10 @@ int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scale
                                     outputs each, loads and LDS reads placed behind single MFMAs (never chosen
                                     automatically); while pinned, moe_gg_grouped_gemm_swiglu_bf16 / _f16 run their
                                     four-wave form too */
+#define MOE_GG_GG_FOURWAVE_TALL 8 /* the same kernel with tiles of up to 256 + 32 rows: an expert's last full row tile
+                                     takes along up to 32 rows behind it, which otherwise are a low tile that streams
+                                     the expert's weight tile a second time (never chosen automatically; SiLU-and-mul
+                                     entry points as for 7; host enumerators: MOE_GG_ORDER_TALL_TILES) */
 #define MOE_GG_OP_GG_FP8 1
 /* variants of MOE_GG_OP_GG_FP8 */
 #define MOE_GG_FP8_TILED_128 0       /* 128x128 tiles for every expert */
@@ -332,6 +336,8 @@ int moe_gg_fp8_block128_quant(const void* in, int dtype, void* out, float* scale
 #define MOE_GG_ORDER_TWO_LISTS 0   /* long tiles, then low tiles; last round cut by its fill alone */
 #define MOE_GG_ORDER_SPLIT_TAILS 1 /* + a tall expert's last full tile and few rows become two half tiles; row
                                       pieces of the last round chosen with the second list in view */
+#define MOE_GG_ORDER_TALL_TILES 2  /* host enumerators only: the lists of MOE_GG_GG_FOURWAVE_TALL (the kernels take
+                                      this value as TWO_LISTS) */
 #define MOE_GG_OP_W4A16 3
 /* variants of MOE_GG_OP_W4A16 (bits, group size 128 and 16-bit output only; -1 and 0 are the default kernels) */
 #define MOE_GG_W4_ONE_PASS 1 /* 33-64 rows per expert: one pass of four activation fragments on four waves instead of

@@ -79,6 +79,13 @@ def _asm_rule(template, outs, ins, where):
     if re.fullmatch(r"\s*v_mad_u32_u24 %0, %1, %2, %3\s*", t):
         assert len(outs) == 1 and len(ins) == 3, where
         return "%s = ((%s) & 0xFFFFFFu) * ((%s) & 0xFFFFFFu) + (%s)" % (outs[0], ins[0], ins[1], ins[2])
+    m = re.fullmatch(r"\s*v_mfma_f32_16x16x32_(bf16|f16) %0, %1, %2, %0\s*", t)
+    if m:  # an MFMA with VGPR accumulators, written out: "+v"(c) : "v"(a), "v"(b)
+        assert len(outs) == 1 and len(ins) == 2, where
+        return "%s = mfma_16x16x32<%s>(__builtin_bit_cast(u32x4_t, %s), __builtin_bit_cast(u32x4_t, %s), %s)" % (
+            outs[0], "true" if m.group(1) == "f16" else "false", ins[0], ins[1], outs[0])
+    if re.fullmatch(r"\s*s_nop \d+(\s*s_nop \d+)*\s*", t):
+        return "((void)0)"  # wait states
     if t.strip() == "":
         return "((void)0)"  # an optimisation barrier on registers
     raise SystemExit("build_emu: no rule for the inline assembly at %s: %r" % (where, template))

@@ -12,7 +12,7 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 import harness as H  # noqa: E402
 from oracle import oracle as O  # noqa: E402
 
-EDGE = [0, 1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 320, 511, 512, 513, 530]
+EDGE = [0, 1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 272, 273, 288, 289, 320, 511, 512, 513, 530, 544]
 
 
 def sizes_of(rng, gmax=6, mmax=600):
@@ -46,7 +46,7 @@ def c_gemm(rng):
         N, K, variant = int(rng.integers(1, 200)), int(rng.integers(1, 200)), -1
     else:
         N, K = int(rng.choice([16, 64, 100, 128, 256, 264, 512])), int(rng.choice([64, 128, 192, 256]))
-        variant = int(rng.choice([-1, 0, 1, 2, 3, 4, 5, 6, 7, 7]))
+        variant = int(rng.choice([-1, 0, 1, 2, 3, 4, 5, 6, 7, 7, 8, 8]))
         if variant == 5 and K % 128:
             K = 128
     G, M = len(sizes), sum(sizes)
@@ -77,9 +77,10 @@ def c_swiglu(rng):
     G, M = len(sizes), sum(sizes)
     x = ints(rng, (M, K), -2, 3)
     w = (ints(rng, (G * 2 * n, K), -2, 3) * 0.125).astype(np.float32)
-    got = H.from16(H.grouped_gemm_swiglu(H.to16(x, fp16), H.to16(w, fp16), sizes, n, fp16), fp16)
+    variant = int(rng.choice([-1, -1, 7, 8]))     # the eight-wave kernel or one of its four-wave forms
+    got = H.from16(H.grouped_gemm_swiglu(H.to16(x, fp16), H.to16(w, fp16), sizes, n, fp16, variant=variant), fp16)
     want = O.silu_and_mul(O.grouped_gemm(x, w, sizes))
-    return bool(not np.isnan(got).any() and np.abs(got - want).max() <= 1e-2 * max(1.0, np.abs(want).max())), ("swiglu", sizes, n, K, fp16)
+    return bool(not np.isnan(got).any() and np.abs(got - want).max() <= 1e-2 * max(1.0, np.abs(want).max())), ("swiglu", sizes, n, K, fp16, variant)
 
 
 def c_backward(rng):

@@ -150,7 +150,7 @@ def grouped_gemm_fp8(xq, wq, x_scale, w_scale, mode, m_sizes, N, variant=-1):
 
 
 def grouped_gemm_swiglu(x16, w16, m_sizes, n, fp16=False, variant=-1):
-    """variant 7 (MOE_GG_GG_FOURWAVE_256 pinned for the grouped GEMM) selects the four-wave form of the fused kernel."""
+    """variant 7 or 8 (MOE_GG_GG_FOURWAVE_256 / _TALL pinned for the grouped GEMM) selects a four-wave form of the fused kernel."""
     L = lib()
     ms = i32(m_sizes)
     G, (M, K) = len(ms), x16.shape

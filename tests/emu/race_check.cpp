@@ -76,9 +76,9 @@ static int one_shape(const char* op, int N, int K, int G, char** sizes) {
     Buf<uint8_t> ws(wsb + 512);
     uint8_t* wsp = ws.p() + ((256 - ((uintptr_t)ws.p() & 255)) & 255);
     check(moe_gg_grouped_gemm_backward_bf16(go.p(), N, 0, x.p(), w.p(), ms.p(), G, M, N, K, gx.p(), gw.p(), wsp, wsb, nullptr), op);
-  } else if (!std::strcmp(op, "swigluw4")) {  // the fused kernel on four waves (N = output columns n, w [G, 2 n, K])
+  } else if (!std::strcmp(op, "swigluw4") || !std::strcmp(op, "swiglutall")) {  // the fused kernel on four waves (N = output columns n, w [G, 2 n, K])
     auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * 2 * N * K);
-    moe_gg_set_variant(MOE_GG_OP_GG_BF16, MOE_GG_GG_FOURWAVE_256);
+    moe_gg_set_variant(MOE_GG_OP_GG_BF16, !std::strcmp(op, "swiglutall") ? MOE_GG_GG_FOURWAVE_TALL : MOE_GG_GG_FOURWAVE_256);
     check(moe_gg_grouped_gemm_swiglu_bf16(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, nullptr), op);
     moe_gg_set_variant(MOE_GG_OP_GG_BF16, -1);
   } else if (!std::strcmp(op, "swiglu")) {
@@ -94,9 +94,10 @@ static int one_shape(const char* op, int N, int K, int G, char** sizes) {
   } else {
     const bool f16 = !std::strcmp(op, "f16") || !std::strcmp(op, "f16w4");
     const bool fourwave = !std::strcmp(op, "bf16w4") || !std::strcmp(op, "f16w4");
+    const bool tall = !std::strcmp(op, "bf16tall");
     auto x = f16 ? f16_small((size_t)M * K) : bf16_small((size_t)M * K);
     auto w = f16 ? f16_small((size_t)G * N * K) : bf16_small((size_t)G * N * K);
-    moe_gg_set_variant(MOE_GG_OP_GG_BF16, fourwave ? MOE_GG_GG_FOURWAVE_256 : MOE_GG_GG_PINGPONG_256);
+    moe_gg_set_variant(MOE_GG_OP_GG_BF16, tall ? MOE_GG_GG_FOURWAVE_TALL : fourwave ? MOE_GG_GG_FOURWAVE_256 : MOE_GG_GG_PINGPONG_256);
     check((f16 ? moe_gg_grouped_gemm_f16 : moe_gg_grouped_gemm_bf16)(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, MOE_GG_OUT_MN, nullptr), op);
   }
   return failures ? 1 : 0;
@@ -104,7 +105,8 @@ static int one_shape(const char* op, int N, int K, int G, char** sizes) {
 
 // race_check                       all entry points (exit status 0 unless the sanitizer reported something: then 66)
 // race_check selftest K B          control kernel K (0: stores, 1: global->LDS load), B = 1 with / 0 without the barrier
-// race_check shape OP N K m1 m2 .. one launch; OP = bf16 | f16 | swiglu | gather | fp8row | fp8block | bwd
+// race_check shape OP N K m1 m2 .. one launch; OP = bf16 | f16 | bf16w4 | f16w4 | bf16tall | swiglu | swigluw4 | swiglutall |
+//                                  gather | fp8row | fp8block | bwd
 int main(int argc, char** argv) {
   // EMU_TILE_ORDER = 0 / 1: the ping-pong kernels' tile order for this run (MOE_GG_OP_TILE_ORDER)
   if (const char* order = std::getenv("EMU_TILE_ORDER")) moe_gg_set_variant(MOE_GG_OP_TILE_ORDER, std::atoi(order));
@@ -120,7 +122,7 @@ int main(int argc, char** argv) {
     std::memcpy(ms.p(), sizes, sizeof(sizes));
     auto x = bf16_small((size_t)M * K), w = bf16_small((size_t)G * N * K);
     Buf<uint16_t> y((size_t)M * N * G);
-    for (int variant = -1; variant <= 7; ++variant) {
+    for (int variant = -1; variant <= 8; ++variant) {
       moe_gg_set_variant(MOE_GG_OP_GG_BF16, variant);
       check(moe_gg_grouped_gemm_bf16(x.p(), w.p(), y.p(), ms.p(), G, M, N, K, N, MOE_GG_OUT_MN, nullptr), "grouped_gemm_bf16 (every variant)");
     }

@@ -493,6 +493,18 @@ def test_traffic_implied_by_the_tile_order(lib):
     xb, wb, yb = _lockstep_traffic(lib, cfg2, 14336, 4096, fused_gate_up=True)
     alg = 8192 * 4096 * 2 + 8 * 2 * 14336 * 4096 * 2 + yb
     assert abs(xb - 14 * 8192 * 4096 * 2) < 0.02 * xb and 1.75 < (xb + wb + yb) / alg < 1.9
+    # tiles of up to 256 + 32 rows (the four-wave kernel's tall form): the four tails ride along with their experts' last
+    # full tiles, 1792 tiles = 7 per workgroup, every weight tile read once: 1.64 GB = 1.32 x; the fused GEMM 1.40 x
+    assert lib.moe_gg_set_variant(2, 2) == 0
+    try:
+        xb, wb, yb = _lockstep_traffic(lib, cfg2, 14336, 4096)
+        alg = 8192 * 4096 * 2 + 8 * 14336 * 4096 * 2 + yb
+        assert abs(wb - 8 * 14336 * 4096 * 2) < 0.01 * wb and 1.28 < (xb + wb + yb) / alg < 1.36
+        xb, wb, yb = _lockstep_traffic(lib, cfg2, 14336, 4096, fused_gate_up=True)
+        alg = 8192 * 4096 * 2 + 8 * 2 * 14336 * 4096 * 2 + yb
+        assert abs(wb - 8 * 2 * 14336 * 4096 * 2) < 0.01 * wb and 1.36 < (xb + wb + yb) / alg < 1.44
+    finally:
+        lib.moe_gg_set_variant(2, -1)
     # config 5 (fp8, 256 experts): dominated by weights that are read once; the order adds 7 %
     from applied_ai_amd import configs
 

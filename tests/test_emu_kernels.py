@@ -55,7 +55,7 @@ def tile_order(request):
 SIZES = [300, 0, 70, 530]   # a full tile + a low tile, an empty expert, a short one, a tall one whose tail is split
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, -1])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, -1])
 def test_bf16_every_kernel_variant(variant, tile_order):
     rng = np.random.default_rng(variant + 1)
     x, w = ints(rng, (sum(SIZES), 128)), ints(rng, (4 * 512, 128))
@@ -65,7 +65,7 @@ def test_bf16_every_kernel_variant(variant, tile_order):
 
 @pytest.mark.parametrize("K", [64, 128, 192, 320])
 @pytest.mark.parametrize("sizes,N", [([300, 0, 70, 530], 512), ([257, 1], 300), ([40], 64)])
-@pytest.mark.parametrize("variant", [6, 7])
+@pytest.mark.parametrize("variant", [6, 7, 8])
 def test_four_wave_kernels_over_k_steps(sizes, N, K, variant):
     """MOE_GG_GG_TILED_256_W4 and MOE_GG_GG_FOURWAVE_256 with 1, 2, 3 and 5 K steps per tile: their loops issue the
     slab loads behind the last slab too (masked to one line, into the buffer nobody reads again), and the second one
@@ -124,11 +124,23 @@ def test_fp8_every_kernel_variant(mode, variant, tile_order):
     assert exact16(y, O.grouped_gemm_fp8(xq, wq, xs, ws, sizes, mode))
 
 
+@pytest.mark.parametrize("sizes,N,K", [([257, 272, 273, 288, 289], 256, 128), ([530, 1, 544, 0, 800], 300, 64), ([270], 256, 192),
+                                       ([1036, 1012, 998], 512, 64), ([513] * 5, 128, 128)])
 @pytest.mark.parametrize("fp16", [False, True])
-@pytest.mark.parametrize("variant", [-1, 7])
+def test_four_wave_kernel_with_tall_tiles(sizes, N, K, fp16):
+    """MOE_GG_GG_FOURWAVE_TALL: tails of 1, 16, 17 and 32 rows ride along with the last full tile (33 do not), also when
+    the tile is cut into row pieces ([270] alone: four pieces on eight compute units, the last with 64 + 14 rows)."""
+    rng = np.random.default_rng(len(sizes) + N)
+    x, w = ints(rng, (sum(sizes), K)), ints(rng, (len(sizes) * N, K))
+    y = H.grouped_gemm(H.to16(x, fp16), H.to16(w, fp16), sizes, N, fp16=fp16, variant=8)
+    assert exact16(y, O.grouped_gemm(x, w, sizes), fp16)
+
+
+@pytest.mark.parametrize("fp16", [False, True])
+@pytest.mark.parametrize("variant", [-1, 7, 8])
 @pytest.mark.parametrize("n,K", [(192, 128), (64, 64), (328, 192)])
 def test_fused_silu_and_mul_gemm(fp16, variant, n, K, tile_order):
-    """The eight-wave kernel and (variant 7) its four-wave form: against the oracle, and the two against each other
+    """The eight-wave kernel and (variants 7, 8) its four-wave forms: against the oracle, and against each other
     bit for bit (the same products in the same order, the same roundings)."""
     rng = np.random.default_rng(5)
     x = (rng.standard_normal((sum(SIZES), K)) * 0.5).astype(np.float32)
@@ -138,7 +150,7 @@ def test_fused_silu_and_mul_gemm(fp16, variant, n, K, tile_order):
     got = H.from16(got16, fp16)
     want = O.silu_and_mul(O.grouped_gemm(H.from16(x16, fp16), H.from16(w16, fp16), SIZES))
     np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2)
-    if variant == 7:
+    if variant >= 7:
         assert (got16 == H.grouped_gemm_swiglu(x16, w16, SIZES, n, fp16)).all()
 
 
@@ -476,7 +488,8 @@ def test_no_data_race_between_the_waves_of_a_workgroup():
               ("fp8block", "384", "256", "1", "0", ["577", "33", "320"]), ("fp8row", "256", "128", "3", "9", ["129", "768", "1"]),
               ("f16", "384", "256", "2", "0", ["321", "511"]), ("bwd", "256", "128", "3", "4", ["300", "0", "41", "513"]),
               ("bf16w4", "512", "192", "1", "0", ["530", "300", "0", "70"]), ("f16w4", "384", "64", "2", "6", ["321", "511", "1"]),
-              ("swigluw4", "192", "128", "2", "1", ["300", "70", "0", "257"])]
+              ("swigluw4", "192", "128", "2", "1", ["300", "70", "0", "257"]),
+              ("bf16tall", "512", "192", "1", "0", ["530", "288", "0", "70", "257"]), ("swiglutall", "192", "128", "2", "1", ["270", "70", "0", "513"])]
     for i, (op, N, K, cus, seed, sizes) in enumerate(shapes):
         for order in ("0", "1"):
             procs.append(subprocess.Popen([exe, "shape", op, N, K] + sizes,

@@ -105,6 +105,27 @@ def test_hot_kernels_do_not_touch_scratch(asm):
             assert lds <= 160 << 10, (name, lds)        # the staged forms add 4 KB of LDS per wave and fragment
 
 
+def test_tall_tile_k_loop(asm):
+    """The four-wave kernels with tiles of up to 288 rows: the K-step loop has the 128 MFMAs of the plain form plus the
+    16 hand-written ones of the ninth activation fragment (VGPR accumulators), 34 fragment reads, 17 slab loads, and
+    still no accumulator moves and no scratch access; the hand-written MFMAs keep their accumulators in the same
+    registers in both half steps."""
+    for want in ("gg_bf16_fourwave_tallE", "gg_f16_fourwave_tallE", "gg_bf16_fourwave_tall_swigluE", "gg_f16_fourwave_tall_swigluE"):
+        (name, (lines, meta)), = [(n, v) for n, v in kernels(asm["gg_pingpong.hip"]).items() if want in n]
+        main = [seg for seg in loops(lines) if count(seg, "v_mfma") == 144 and count(seg, "global_load_lds_dwordx4") == 17]
+        assert main, name
+        seg = min(main, key=len)
+        assert count(seg, "ds_read_b128") == 34 and count(seg, "s_barrier") == 1
+        assert count(seg, "v_accvgpr") == 0 and count(seg, "scratch_") == 0
+        assert len(seg) <= 345, len(seg)
+        hand = [l for l in seg if re.match(r"v_mfma_f32_16x16x32_\w+ v\[", l)]       # VGPR destination: the hand-written ones
+        assert len(hand) == 16
+        dst = [re.match(r"v_mfma\S+ (v\[\d+:\d+\]), \S+ \S+ (v\[\d+:\d+\])", l).groups() for l in hand]
+        assert all(d == c for d, c in dst) and sorted(d for d, _ in dst[:8]) == sorted(d for d, _ in dst[8:])
+        lds = int(re.search(r"\.amdhsa_group_segment_fixed_size (\d+)", meta).group(1))
+        assert lds <= 160 << 10, lds
+
+
 def test_four_wave_k_loop_is_what_the_source_spells_out(asm):
     """gg_bf16_fourwave / gg_f16_fourwave and their SiLU-and-mul forms: one K-step loop of 128 MFMAs with 32 fragment reads and 16 slab loads
     between them, no accumulator moves, no scratch access, no branch but the back edge (and the one around the load

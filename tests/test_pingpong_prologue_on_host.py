@@ -46,7 +46,7 @@ template <class F> static void build_tile_prefix(const int32_t* row_off, int G, 
 }
 static void build_group_tables(const int32_t*, int, int, int, int, int32_t*, int32_t*, int, int) { abort(); }
 
-template <int OP>
+template <int OP, bool TALL = false>
 static void prologue(const GgParams& p, int32_t* seq_out, int* n_my_out) {
   static int32_t row_off[MOE_GG_MAX_GROUPS + 1], tile_off[MOE_GG_MAX_GROUPS + 1], part_off[MOE_GG_MAX_GROUPS + 1];
   static int32_t seq_tab[2 * MOE_GG_SEQ_CAP];
@@ -62,14 +62,18 @@ HARNESS_TAIL = r'''
 
 extern "C" int emu_prologue(int op, const int32_t* m_sizes, int G, int M, int N, int K, int skip_rows, int tails_apart,
                             int nwg, int xcds, int split_tails, int32_t* out, int cap) {
-  GgParams p{m_sizes, G, M, N, K, skip_rows, tails_apart, xcds, split_tails};
+  const bool tall = split_tails == 2;   // the four-wave kernel's lists with tiles of up to 256 + 32 rows
+  GgParams p{m_sizes, G, M, N, K, skip_rows, tails_apart, xcds, tall ? 0 : split_tails};
   gridDim.x = nwg;
   static int32_t seq[2 * MOE_GG_SEQ_CAP];
   int written = 0;
   for (int wg = 0; wg < nwg; ++wg) {
     blockIdx.x = wg;
     int n_my = 0;
-    if (op == OP_BF16) prologue<OP_BF16>(p, seq, &n_my);
+    if (op == OP_BF16 && tall) prologue<OP_BF16, true>(p, seq, &n_my);
+    else if (op == OP_BF16_SWIGLU && tall) prologue<OP_BF16_SWIGLU, true>(p, seq, &n_my);
+    else if (tall) return -1;
+    else if (op == OP_BF16) prologue<OP_BF16>(p, seq, &n_my);
     else if (op == OP_BF16_SWIGLU) prologue<OP_BF16_SWIGLU>(p, seq, &n_my);
     else if (op == OP_BF16_SWIGLU_GATHER) prologue<OP_BF16_SWIGLU_GATHER>(p, seq, &n_my);
     else if (op == OP_FP8_BLOCK) prologue<OP_FP8_BLOCK>(p, seq, &n_my);
@@ -162,6 +166,38 @@ def test_device_prologue_equals_the_host_mirror(emu, lib, split):
         for op in (4, 9):   # the fused gate/up kernel and its form with the row gather
             d = device_tiles(emu, op, sizes, 2 * n_out, 4096, nwg, split=split)
             assert h.shape == d.shape and (h == d).all(), ("swiglu", op, sizes[:8], n_out, nwg)
+
+
+def test_tall_tile_prologue_equals_the_host_mirror_and_covers_every_row_once(emu, lib):
+    """The lists of the four-wave kernel with tall tiles (MOE_GG_GG_FOURWAVE_TALL; host mirror: MOE_GG_ORDER_TALL_TILES):
+    an expert with 1 .. 32 rows behind its last full row tile has no tile for them, its last full tile is that much
+    taller; of a tall tile cut into row pieces the last piece takes the extra rows."""
+    assert lib.moe_gg_set_variant(2, 2) == 0
+    try:
+        tall_seen = 0
+        for sizes, N, nwg in shape_sets():
+            h = host_tiles(lib, sizes, N, 256, nwg)
+            d = device_tiles(emu, 0, sizes, N, 4096, nwg, split=2)
+            assert h.shape == d.shape and (h == d).all(), ("bf16", sizes[:8], N, nwg)
+            c = [np.zeros((max(m, 0), -(-N // 256)), dtype=np.int32) for m in sizes]
+            for wg, g, m0, hh, n0, nc in d.tolist():
+                assert m0 % 64 == 0 and 0 <= hh <= 288 and m0 + hh <= sizes[g], (g, m0, hh)
+                if hh > 256:
+                    assert 0 < sizes[g] % 256 <= 32 and m0 + hh == sizes[g]
+                    tall_seen += 1
+                if hh:
+                    c[g][m0:m0 + hh, n0 // 256] += 1
+            assert all((x == 1).all() for x in c), (sizes[:8], N, nwg)
+            for g, m in enumerate(sizes):     # no tile starts in the absorbed rows
+                if m >= 256 and 0 < m % 256 <= 32:
+                    assert not any(t[1] == g and t[2] >= m // 256 * 256 for t in d.tolist())
+            n_out = max(128, N // 2 // 128 * 128)
+            h = host_tiles(lib, sizes, n_out, 128, nwg)
+            d = device_tiles(emu, 4, sizes, 2 * n_out, 4096, nwg, split=2)
+            assert h.shape == d.shape and (h == d).all(), ("swiglu", sizes[:8], n_out, nwg)
+        assert tall_seen > 100
+    finally:
+        lib.moe_gg_set_variant(2, -1)
 
 
 def cover(tiles, sizes, N):
