@@ -928,8 +928,12 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
       cursor_next();
     }
     if constexpr (TALL) {
-      // the results of the last hand-written MFMAs must not be read before they are written (see mfma_vgpr)
-      if (tall) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+      // The results of the last hand-written MFMAs must not be read before they are written (see mfma_vgpr). The
+      // accumulators are operands of the statement, so that no instruction that reads one can be moved in front of it.
+      if (tall)
+        asm volatile("s_nop 15\n\ts_nop 15"
+                     : "+v"(acc[0][FMA - 1]), "+v"(acc[1][FMA - 1]), "+v"(acc[2][FMA - 1]), "+v"(acc[3][FMA - 1]),
+                       "+v"(acc[4][FMA - 1]), "+v"(acc[5][FMA - 1]), "+v"(acc[6][FMA - 1]), "+v"(acc[7][FMA - 1]));
     }
 
     // Epilogue: lane holds y[m][n .. n + 3] for m = (2 i + wm) * 16 + lane % 16, n = (8 wn + j) * 16 + 4 (lane / 16).

@@ -431,9 +431,9 @@ def test_every_entry_point_on_random_shapes_with_tensors_against_guard_pages():
 @pytest.mark.skipif(not os.environ.get("EMU_FULL_SIZE"), reason="20-40 minutes per case on one core each: set EMU_FULL_SIZE=1")
 def test_config2_at_full_size():
     """Benchmark config 2 at its real size with 256 emulated CUs (tests/emu/full_size.py): the ping-pong kernel in the
-    split-tail order and the four-wave kernel in both orders reproduce the exact bf16 output; the four-wave form of the
-    fused first GEMM gives the default kernel's bits."""
-    cases = [("gemm", "0", "1"), ("gemm", "7", "0"), ("gemm", "7", "1"), ("swiglu", "7", "0")]
+    split-tail order, the four-wave kernel in both orders and its tall-tile form reproduce the exact bf16 output; the
+    four-wave forms of the fused first GEMM give the default kernel's bits."""
+    cases = [("gemm", "0", "1"), ("gemm", "7", "0"), ("gemm", "7", "1"), ("gemm", "8", "0"), ("swiglu", "7", "0"), ("swiglu", "8", "0")]
     procs = [subprocess.Popen([sys.executable, os.path.join(EMU, "full_size.py"), kind, variant],
                               env=dict(os.environ, EMU_CUS="256", EMU_TILE_ORDER=order), stdout=subprocess.PIPE,
                               stderr=subprocess.STDOUT, cwd=ROOT) for kind, variant, order in cases]
