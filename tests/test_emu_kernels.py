@@ -445,12 +445,12 @@ def test_config2_at_full_size():
 def test_kernels_with_trapping_checks_of_alignment_shifts_overflow_and_bounds():
     """A second host build of the kernels in which every vector access checks its alignment, every shift its count,
     every signed operation its range and every index into a fixed-size array its bound, each ending in a trap
-    (EMU_UBSAN, tests/emu/build_emu.py): 120 random calls over all entry points, against guard pages, complete
+    (EMU_UBSAN, tests/emu/build_emu.py): 80 random calls over all entry points, against guard pages, complete
     without one. (An ordinary build would read a misaligned 16-byte LDS access without complaint; the GPU would not.)"""
     env = dict(os.environ, EMU_UBSAN="1", EMU_OUT=os.path.join(EMU, "_build", "ubsan"), EMU_GUARD="end", EMU_TRACE="1")
     b = subprocess.run([sys.executable, os.path.join(EMU, "build_emu.py")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT)
     assert b.returncode == 0, b.stdout.decode()[-2000:]
-    procs = [subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_all.py"), str(700 + i), "60"], stdout=subprocess.PIPE,
+    procs = [subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_all.py"), str(700 + i), "40"], stdout=subprocess.PIPE,
                               stderr=subprocess.STDOUT, cwd=ROOT, env=dict(env, EMU_TILE_ORDER=str(i), EMU_SEED=str(3 * i)))
              for i in range(2)]
     for i, p in enumerate(procs):
