@@ -1050,9 +1050,10 @@ DEVINL void run_fourwave(const GgParams& p, const Shared& sh) {
 
 // FOURWAVE: the workgroup is four waves running run_fourwave (one wave per SIMD, 128 x 128 outputs each) instead of the
 // two groups of four above; tables, tile order and LDS stages are the same.
-template <int OP, bool FOURWAVE = false, bool TALL = false>
+template <int OP, bool FOURWAVE = false, bool TALL = false, bool LISTS2 = FOURWAVE || op_gather(OP)>
 DEVINL void pingpong_body(const GgParams& p) {
   static_assert(!TALL || FOURWAVE, "tall tiles are the four-wave kernel's");
+  static_assert(LISTS2 || (!FOURWAVE && !TALL && !op_gather(OP)), "the first prologue knows the eight-wave kernels without a row gather");
   constexpr int NTB = FOURWAVE ? W4_NT : NT;  // threads of the workgroup
   __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE + (OP == OP_FP8_BLOCK ? 2 * SCALE_BYTES : 0) + (TALL ? 2 * TALL_BYTES : 0)];
   __shared__ int32_t row_off[MOE_GG_MAX_GROUPS + 1];
@@ -1061,93 +1062,195 @@ DEVINL void pingpong_body(const GgParams& p) {
   __shared__ int32_t seq_tab[2 * MOE_GG_SEQ_CAP];
   static_assert(2 * MOE_GG_SEQ_CAP >= MOE_GG_MAX_GROUPS + 1, "seq_tab doubles as a prefix table below");
 
-  int total, total_low = 0;
-  // Forward lists with p.split_tails: tall groups with a few rows beyond their last full tile get two half tiles for
-  // their last rows (moe_gg_split_tail), unless the small-M kernel of the same call takes the low tiles.
-  bool split = p.split_tails != 0;
-  bool apart = false;  // the low tiles are the small-M kernel's
-  if (OP == OP_BF16_WGRAD_DIRECT) {
-    build_row_offsets(p.m_sizes, p.G, p.M, row_off);
-    total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
-  } else if (OP == OP_BF16_WGRAD) {
-    // tile_off counts the 64-column blocks of the padded operands (at least one per expert).
-    build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
-    total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
-  } else {
-    const int ntn = op_swiglu(OP) ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
-    const int skip = p.skip_rows;
-    build_row_offsets(p.m_sizes, p.G, p.M, row_off);
-    if ((OP == OP_BF16 || OP == OP_F16) && p.tails_apart) {
-      // Few low tiles that would open a round of their own are computed by the small-M kernel of the same call,
-      // which takes the same decision from the same counts (the lists without split tails).
+  int n_my = 0;
+  if constexpr (!LISTS2) {
+    // The lists, sequence and tile decode of the kernels that run by default, kept word for word as they last ran on a
+    // GPU (the two-list order; row pieces of the last round by its fill alone).
+    int total, total_low = 0;
+    if (OP == OP_BF16_WGRAD_DIRECT) {
+      build_row_offsets(p.m_sizes, p.G, p.M, row_off);
+      total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
+    } else if (OP == OP_BF16_WGRAD) {
+      // tile_off counts the 64-column blocks of the padded operands (at least one per expert).
+      build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
+      total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
+    } else {
+      const int ntn = op_swiglu(OP) ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
+      const int skip = p.skip_rows;
+      build_row_offsets(p.m_sizes, p.G, p.M, row_off);
       build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
       build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
-      build_tile_prefix(row_off, p.G, seq_tab, [&](int rows) { return moe_gg_low_passes(rows, BM) * ntn; });
-      apart = moe_gg_tails_apart(uni(tile_off[p.G]), uni(part_off[p.G]), uni(seq_tab[p.G]), p.tails_apart);
-      if (apart) split = false;
-      __syncthreads();  // the tables are rewritten below
+      total_low = uni(part_off[p.G]);
+      total = uni(tile_off[p.G]);
+      if ((OP == OP_BF16 || OP == OP_F16) && p.tails_apart) {
+        // Few low tiles that would open a round of their own are computed by the small-M kernel of the same call.
+        build_tile_prefix(row_off, p.G, seq_tab, [&](int rows) { return moe_gg_low_passes(rows, BM) * ntn; });
+        if (moe_gg_tails_apart(total, total_low, uni(seq_tab[p.G]), p.tails_apart)) total_low = 0;
+        __syncthreads();  // seq_tab is rewritten below
+      }
     }
-    if constexpr (TALL) {
-      split = false;  // the lists of moe_gg_tall_tail
-      build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles_tall(rows, BM) * ntn : 0; });
-      build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles_tall(rows, BM) * ntn : 0; });
+    const int nwg = gridDim.x;
+    // Tiles of this workgroup in each list: rounds 0 .. n - 1 (tile ids grow with the round).
+    // (Forward kernels: the long tiles of a sparsely filled last round are cut into row pieces, moe_gg_tail_pieces.)
+    const bool fwd = OP != OP_BF16_WGRAD && OP != OP_BF16_WGRAD_DIRECT;
+    const int tail_s = fwd ? moe_gg_tail_pieces(total, nwg) : 1;
+    const int tail_first = fwd ? moe_gg_tail_first(total, nwg) : total;
+    const int long_ids = fwd ? moe_gg_long_ids(total, nwg) : total;
+    const int low_ids = total_low;
+    int n_long = 0, n_low = 0;
+    while (n_long * nwg < long_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < long_ids) ++n_long;
+    while ((n_long + n_low) * nwg < long_ids + low_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < long_ids + low_ids)
+      ++n_low;
+    if (n_long + n_low == 0) return;
+    // The sequence of this workgroup (moe_gg_seq_round), decoded once into a table: the arithmetic runs per thread
+    // here; in the K loop it would occupy scalar registers that the loop needs.
+    // Tile ids: the long tiles of all groups (group, then column tile, then row tile), then the low tiles (group,
+    // column tile; see moe_gg_long_row_tiles), dealt to the workgroups round-robin: every workgroup gets the same
+    // number (+- 1) of long tiles, and the low tiles go on where the long ones stopped.
+    n_my = min(n_long + n_low, MOE_GG_SEQ_CAP);
+    const int phase = moe_gg_low_phase(blockIdx.x, p.xcds);
+    for (int i = threadIdx.x; i < n_my; i += NT) {
+      int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
+      constexpr int TC = op_swiglu(OP) ? BN / 2 : BN;  // output columns of a tile
+      int g, m0, h, n0, nc = TC;  // group, first row inside the group, rows, first column, columns
+      if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
+        // Tiles of an expert in bands of four column tiles, column tile fastest inside a band: the 32 tiles an XCD
+        // works on at a time are 8 row tiles x 4 column tiles, which share 8 + 4 operand slabs per K step (with the
+        // row tile fastest they were 32 + 1: 3 % slower at the Mixtral shape, the reads from the fabric bound it).
+        const int ntm = moe_gg_cdiv(p.N, BM), ntn = moe_gg_cdiv(p.K, BN), tpg = ntm * ntn;
+        g = L / tpg;
+        const int rem = L - g * tpg;
+        const int band = rem / (4 * ntm), idx = rem - band * (4 * ntm);
+        const int wb = min(4, ntn - band * 4);  // column tiles of this band
+        const int tm = idx / wb;
+        n0 = (band * 4 + idx - tm * wb) * BN;
+        m0 = tm * BM;
+        h = min(p.N - m0, BM);
+      } else if (L < long_ids) {
+        int piece = 0;
+        if (L >= tail_first) {  // a piece of a tile of the last round
+          piece = (L - tail_first) % tail_s;
+          L = tail_first + (L - tail_first) / tail_s;
+        }
+        g = moe_gg_find_group(tile_off, p.G, L);
+        const int idx = L - tile_off[g];
+        const int rows = row_off[g + 1] - row_off[g];
+        const int nf = moe_gg_long_row_tiles(rows, BM);
+        const int tn = idx / nf;
+        n0 = tn * TC;
+        m0 = (idx - tn * nf) * BM;
+        h = min(rows - m0, BM);
+        if (tail_s > 1 && L >= tail_first) {
+          int off;
+          moe_gg_piece_rows(h, tail_s, piece, &off, &h);
+          if (h > 0) m0 += off;  // a piece without rows keeps the tile's first row: its loads must stay in bounds
+        }
+      } else {
+        // Low tiles. (Cutting few low tiles into column pieces for more workgroups was measured: no gain, a low
+        // tile is bound by the per-step cost of the K loop, not by the bytes it streams.)
+        const int Lp = L - long_ids;
+        g = moe_gg_find_group(part_off, p.G, Lp);
+        const int tn = Lp - part_off[g];
+        n0 = tn * TC;
+        const int rows = row_off[g + 1] - row_off[g];
+        m0 = rows / BM * BM;
+        h = rows - m0;
+      }
+      seq_tab[2 * i] = g | (h << 16) | ((nc / 32) << 26);
+      seq_tab[2 * i + 1] = (m0 / 64) | ((n0 / 32) << 16);
+    }
+  } else {
+    // The same with the selectable orders: split tails (p.split_tails), tall tiles (TALL); one decode function shared
+    // with the host mirror. Also the prologue of the kernels that came with it (four waves, row gather).
+    int total, total_low = 0;
+    // Forward lists with p.split_tails: tall groups with a few rows beyond their last full tile get two half tiles for
+    // their last rows (moe_gg_split_tail), unless the small-M kernel of the same call takes the low tiles.
+    bool split = p.split_tails != 0;
+    bool apart = false;  // the low tiles are the small-M kernel's
+    if (OP == OP_BF16_WGRAD_DIRECT) {
+      build_row_offsets(p.m_sizes, p.G, p.M, row_off);
+      total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
+    } else if (OP == OP_BF16_WGRAD) {
+      // tile_off counts the 64-column blocks of the padded operands (at least one per expert).
+      build_group_tables(p.m_sizes, p.G, p.skip_rows, 64, 1, row_off, tile_off, 0, 1);
+      total = p.G * moe_gg_cdiv(p.N, BM) * moe_gg_cdiv(p.K, BN);
     } else {
-    build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles2(rows, BM, split) * ntn : 0; });
-    build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles2(rows, BM, split) * ntn : 0; });
+      const int ntn = op_swiglu(OP) ? moe_gg_cdiv(p.N / 2, BN / 2) : moe_gg_cdiv(p.N, BN);
+      const int skip = p.skip_rows;
+      build_row_offsets(p.m_sizes, p.G, p.M, row_off);
+      if ((OP == OP_BF16 || OP == OP_F16) && p.tails_apart) {
+        // Few low tiles that would open a round of their own are computed by the small-M kernel of the same call,
+        // which takes the same decision from the same counts (the lists without split tails).
+        build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles(rows, BM) * ntn : 0; });
+        build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles(rows, BM) * ntn : 0; });
+        build_tile_prefix(row_off, p.G, seq_tab, [&](int rows) { return moe_gg_low_passes(rows, BM) * ntn; });
+        apart = moe_gg_tails_apart(uni(tile_off[p.G]), uni(part_off[p.G]), uni(seq_tab[p.G]), p.tails_apart);
+        if (apart) split = false;
+        __syncthreads();  // the tables are rewritten below
+      }
+      if constexpr (TALL) {
+        split = false;  // the lists of moe_gg_tall_tail
+        build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles_tall(rows, BM) * ntn : 0; });
+        build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles_tall(rows, BM) * ntn : 0; });
+      } else {
+      build_tile_prefix(row_off, p.G, tile_off, [&](int rows) { return rows > skip ? moe_gg_long_row_tiles2(rows, BM, split) * ntn : 0; });
+      build_tile_prefix(row_off, p.G, part_off, [&](int rows) { return rows > skip ? moe_gg_low_row_tiles2(rows, BM, split) * ntn : 0; });
+      }
+      total_low = apart ? 0 : uni(part_off[p.G]);
+      total = uni(tile_off[p.G]);
     }
-    total_low = apart ? 0 : uni(part_off[p.G]);
-    total = uni(tile_off[p.G]);
-  }
-  const int nwg = gridDim.x;
-  // Tiles of this workgroup in each list: rounds 0 .. n - 1 (tile ids grow with the round).
-  // (Forward kernels: the long tiles of a sparsely filled last round are cut into row pieces: by the fill of that
-  // round alone (moe_gg_tail_pieces), or, with p.split_tails, as many as make the busiest workgroup's load smallest
-  // with the second list dealt behind them, moe_gg_tail_pieces_low.)
-  const bool fwd = OP != OP_BF16_WGRAD && OP != OP_BF16_WGRAD_DIRECT;
-  const int tail_s = !fwd ? 1 : (p.split_tails && !TALL) ? moe_gg_tail_pieces_low(total, total_low, nwg) : moe_gg_tail_pieces(total, nwg);
-  const int tail_first = moe_gg_tail_first_s(total, nwg, tail_s);
-  const int long_ids = moe_gg_long_ids_s(total, nwg, tail_s);
-  const int low_ids = total_low;
-  int n_long = 0, n_low = 0;
-  while (n_long * nwg < long_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < long_ids) ++n_long;
-  while ((n_long + n_low) * nwg < long_ids + low_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < long_ids + low_ids)
-    ++n_low;
-  if (n_long + n_low == 0) return;
-  // The sequence of this workgroup (moe_gg_seq_round), decoded once into a table: the arithmetic runs per thread
-  // here; in the K loop it would occupy scalar registers that the loop needs.
-  // Tile ids: the long tiles of all groups (group, then column tile, then row tile), then the second list (group,
-  // column tile, then the group's low tile or its two half tiles; see moe_gg_long_row_tiles, moe_gg_split_tail),
-  // dealt to the workgroups round-robin: every workgroup gets the same number (+- 1) of long tiles, and the second
-  // list goes on where the long ones stopped.
-  const int n_my = min(n_long + n_low, MOE_GG_SEQ_CAP), phase = moe_gg_low_phase(blockIdx.x, p.xcds);
-  for (int i = threadIdx.x; i < n_my; i += NTB) {
-    int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
-    constexpr int TC = op_swiglu(OP) ? BN / 2 : BN;  // output columns of a tile
-    int g, m0, h, n0, nc = TC;  // group, first row inside the group, rows, first column, columns
-    if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
-      // Tiles of an expert in bands of four column tiles, column tile fastest inside a band: the 32 tiles an XCD
-      // works on at a time are 8 row tiles x 4 column tiles, which share 8 + 4 operand slabs per K step (with the
-      // row tile fastest they were 32 + 1: 3 % slower at the Mixtral shape, the reads from the fabric bound it).
-      const int ntm = moe_gg_cdiv(p.N, BM), ntn = moe_gg_cdiv(p.K, BN), tpg = ntm * ntn;
-      g = L / tpg;
-      const int rem = L - g * tpg;
-      const int band = rem / (4 * ntm), idx = rem - band * (4 * ntm);
-      const int wb = min(4, ntn - band * 4);  // column tiles of this band
-      const int tm = idx / wb;
-      n0 = (band * 4 + idx - tm * wb) * BN;
-      m0 = tm * BM;
-      h = min(p.N - m0, BM);
-    } else {
-      // Long tiles (the last round cut into row pieces when it is sparsely filled), then the second list.
-      // (Cutting few low tiles into column pieces for more workgroups was measured: no gain, a low tile is bound
-      // by the per-step cost of the K loop, not by the bytes it streams.)
-      MoeGgListTile lt;
-      if constexpr (TALL) lt = moe_gg_two_list_decode_tall(row_off, tile_off, part_off, p.G, L, long_ids, tail_first, tail_s, BM, TC);
-      else lt = moe_gg_two_list_decode(row_off, tile_off, part_off, p.G, L, long_ids, tail_first, tail_s, BM, TC, split);
-      g = lt.g; m0 = lt.m0; h = lt.h; n0 = lt.n0;
+    const int nwg = gridDim.x;
+    // Tiles of this workgroup in each list: rounds 0 .. n - 1 (tile ids grow with the round).
+    // (Forward kernels: the long tiles of a sparsely filled last round are cut into row pieces: by the fill of that
+    // round alone (moe_gg_tail_pieces), or, with p.split_tails, as many as make the busiest workgroup's load smallest
+    // with the second list dealt behind them, moe_gg_tail_pieces_low.)
+    const bool fwd = OP != OP_BF16_WGRAD && OP != OP_BF16_WGRAD_DIRECT;
+    const int tail_s = !fwd ? 1 : (p.split_tails && !TALL) ? moe_gg_tail_pieces_low(total, total_low, nwg) : moe_gg_tail_pieces(total, nwg);
+    const int tail_first = moe_gg_tail_first_s(total, nwg, tail_s);
+    const int long_ids = moe_gg_long_ids_s(total, nwg, tail_s);
+    const int low_ids = total_low;
+    int n_long = 0, n_low = 0;
+    while (n_long * nwg < long_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long) < long_ids) ++n_long;
+    while ((n_long + n_low) * nwg < long_ids + low_ids && moe_gg_tile_of(blockIdx.x, nwg, p.xcds, n_long + n_low) < long_ids + low_ids)
+      ++n_low;
+    if (n_long + n_low == 0) return;
+    // The sequence of this workgroup (moe_gg_seq_round), decoded once into a table: the arithmetic runs per thread
+    // here; in the K loop it would occupy scalar registers that the loop needs.
+    // Tile ids: the long tiles of all groups (group, then column tile, then row tile), then the second list (group,
+    // column tile, then the group's low tile or its two half tiles; see moe_gg_long_row_tiles, moe_gg_split_tail),
+    // dealt to the workgroups round-robin: every workgroup gets the same number (+- 1) of long tiles, and the second
+    // list goes on where the long ones stopped.
+    n_my = min(n_long + n_low, MOE_GG_SEQ_CAP);
+    const int phase = moe_gg_low_phase(blockIdx.x, p.xcds);
+    for (int i = threadIdx.x; i < n_my; i += NTB) {
+      int L = moe_gg_tile_of(blockIdx.x, nwg, p.xcds, moe_gg_seq_round(i, n_long + n_low, n_low, phase));
+      constexpr int TC = op_swiglu(OP) ? BN / 2 : BN;  // output columns of a tile
+      int g, m0, h, n0, nc = TC;  // group, first row inside the group, rows, first column, columns
+      if (OP == OP_BF16_WGRAD || OP == OP_BF16_WGRAD_DIRECT) {
+        // Tiles of an expert in bands of four column tiles, column tile fastest inside a band: the 32 tiles an XCD
+        // works on at a time are 8 row tiles x 4 column tiles, which share 8 + 4 operand slabs per K step (with the
+        // row tile fastest they were 32 + 1: 3 % slower at the Mixtral shape, the reads from the fabric bound it).
+        const int ntm = moe_gg_cdiv(p.N, BM), ntn = moe_gg_cdiv(p.K, BN), tpg = ntm * ntn;
+        g = L / tpg;
+        const int rem = L - g * tpg;
+        const int band = rem / (4 * ntm), idx = rem - band * (4 * ntm);
+        const int wb = min(4, ntn - band * 4);  // column tiles of this band
+        const int tm = idx / wb;
+        n0 = (band * 4 + idx - tm * wb) * BN;
+        m0 = tm * BM;
+        h = min(p.N - m0, BM);
+      } else {
+        // Long tiles (the last round cut into row pieces when it is sparsely filled), then the second list.
+        // (Cutting few low tiles into column pieces for more workgroups was measured: no gain, a low tile is bound
+        // by the per-step cost of the K loop, not by the bytes it streams.)
+        MoeGgListTile lt;
+        if constexpr (TALL) lt = moe_gg_two_list_decode_tall(row_off, tile_off, part_off, p.G, L, long_ids, tail_first, tail_s, BM, TC);
+        else lt = moe_gg_two_list_decode(row_off, tile_off, part_off, p.G, L, long_ids, tail_first, tail_s, BM, TC, split);
+        g = lt.g; m0 = lt.m0; h = lt.h; n0 = lt.n0;
+      }
+      seq_tab[2 * i] = g | (h << 16) | ((nc / 32) << 26);
+      seq_tab[2 * i + 1] = (m0 / 64) | ((n0 / 32) << 16);
     }
-    seq_tab[2 * i] = g | (h << 16) | ((nc / 32) << 26);
-    seq_tab[2 * i + 1] = (m0 / 64) | ((n0 / 32) << 16);
   }
   __syncthreads();
 
@@ -1180,11 +1283,23 @@ __global__ __launch_bounds__(NT) void gg_bf16_pingpong_nt(GgParams p) { pingpong
 __global__ __launch_bounds__(NT) void gg_bf16_pingpong_wgrad_direct(GgParams p) { pingpong_body<OP_BF16_WGRAD_DIRECT>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise(GgParams p) { pingpong_body<OP_FP8_ROW>(p); }
 __global__ __launch_bounds__(NT) void gg_fp8_pingpong_block(GgParams p) { pingpong_body<OP_FP8_BLOCK>(p); }
+// The forward eight-wave kernels behind the second prologue, for the split-tail order (p.split_tails): the K loops are
+// the same source as above.
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong_split(GgParams p) { pingpong_body<OP_BF16, false, false, true>(p); }
+__global__ __launch_bounds__(NT) void gg_f16_pingpong_split(GgParams p) { pingpong_body<OP_F16, false, false, true>(p); }
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong_swiglu_split(GgParams p) { pingpong_body<OP_BF16_SWIGLU, false, false, true>(p); }
+__global__ __launch_bounds__(NT) void gg_f16_pingpong_swiglu_split(GgParams p) { pingpong_body<OP_F16_SWIGLU, false, false, true>(p); }
+__global__ __launch_bounds__(NT) void gg_bf16_pingpong_nt_split(GgParams p) { pingpong_body<OP_BF16_NT, false, false, true>(p); }
+__global__ __launch_bounds__(NT) void gg_fp8_pingpong_rowwise_split(GgParams p) { pingpong_body<OP_FP8_ROW, false, false, true>(p); }
+__global__ __launch_bounds__(NT) void gg_fp8_pingpong_block_split(GgParams p) { pingpong_body<OP_FP8_BLOCK, false, false, true>(p); }
 
 }  // namespace
 
 hipError_t gg_bf16_pingpong_launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
+  if (p.split_tails) {
+    if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong_split, dim3(num_wg), dim3(NT), 0, stream, p);
+    else hipLaunchKernelGGL(gg_bf16_pingpong_split, dim3(num_wg), dim3(NT), 0, stream, p);
+  } else if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
   else hipLaunchKernelGGL(gg_bf16_pingpong, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
@@ -1216,13 +1331,17 @@ hipError_t gg_bf16_pingpong_swiglu_launch(const GgParams& p, int num_wg, hipStre
   if (p.gather_perm) {
     if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong_swiglu_gather, dim3(num_wg), dim3(NT), 0, stream, p);
     else hipLaunchKernelGGL(gg_bf16_pingpong_swiglu_gather, dim3(num_wg), dim3(NT), 0, stream, p);
+  } else if (p.split_tails) {
+    if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong_swiglu_split, dim3(num_wg), dim3(NT), 0, stream, p);
+    else hipLaunchKernelGGL(gg_bf16_pingpong_swiglu_split, dim3(num_wg), dim3(NT), 0, stream, p);
   } else if (p.fp16) hipLaunchKernelGGL(gg_f16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
   else hipLaunchKernelGGL(gg_bf16_pingpong_swiglu, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
 
 hipError_t gg_bf16_pingpong_nt_launch(const GgParams& p, int num_wg, hipStream_t stream) {
-  hipLaunchKernelGGL(gg_bf16_pingpong_nt, dim3(num_wg), dim3(NT), 0, stream, p);
+  if (p.split_tails) hipLaunchKernelGGL(gg_bf16_pingpong_nt_split, dim3(num_wg), dim3(NT), 0, stream, p);
+  else hipLaunchKernelGGL(gg_bf16_pingpong_nt, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -1232,7 +1351,10 @@ hipError_t gg_bf16_pingpong_wgrad_direct_launch(const GgParams& p, int num_wg, h
 }
 
 hipError_t gg_fp8_pingpong_launch(const GgParams& p, int scale_mode, int num_wg, hipStream_t stream) {
-  if (scale_mode == 0) hipLaunchKernelGGL(gg_fp8_pingpong_rowwise, dim3(num_wg), dim3(NT), 0, stream, p);
+  if (p.split_tails) {
+    if (scale_mode == 0) hipLaunchKernelGGL(gg_fp8_pingpong_rowwise_split, dim3(num_wg), dim3(NT), 0, stream, p);
+    else hipLaunchKernelGGL(gg_fp8_pingpong_block_split, dim3(num_wg), dim3(NT), 0, stream, p);
+  } else if (scale_mode == 0) hipLaunchKernelGGL(gg_fp8_pingpong_rowwise, dim3(num_wg), dim3(NT), 0, stream, p);
   else hipLaunchKernelGGL(gg_fp8_pingpong_block, dim3(num_wg), dim3(NT), 0, stream, p);
   return hipGetLastError();
 }

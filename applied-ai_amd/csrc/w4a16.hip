@@ -209,12 +209,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_splitk_anygroup(W4Params p) 
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
-  // The two constants of the nibble unpack live in registers (the mask in a scalar, the exponent pattern in a vector
-  // one), hidden from constant folding: mask-and-or is then one v_and_or_b32, which takes no literal and one scalar
-  // operand; with literals it is an and and an or.
-  uint32_t nib_mask = 0x000F000Fu, magic = E::MAGIC;
-  asm volatile("" : "+s"(nib_mask));
-  asm volatile("" : "+v"(magic));
+  const uint32_t nib_mask = 0x000F000Fu, magic = E::MAGIC;  // the two constants of the nibble unpack
   const W4View v = w4_view(p);
   const int N = p.N, K = p.K, M = v.M;
   constexpr int CB = QOUT ? 2 : 1;                 // 64-column blocks per workgroup
@@ -365,12 +360,15 @@ __global__ __launch_bounds__(64 * (NWAVES + WARM)) void w4a16_splitk_g128(W4Para
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int fr = lane & 15, fq = lane >> 4;
-  // The two constants of the nibble unpack live in registers (the mask in a scalar, the exponent pattern in a vector
-  // one), hidden from constant folding: mask-and-or is then one v_and_or_b32, which takes no literal and one scalar
-  // operand; with literals it is an and and an or.
+  // The two constants of the nibble unpack. In the selectable forms (one pass, warm-up waves, staged activations) they
+  // live in registers, the mask in a scalar and the exponent pattern in a vector one, hidden from constant folding:
+  // mask-and-or is then one v_and_or_b32, which takes no literal and one scalar operand; with literals, as in the
+  // kernels that run by default, it is an and and an or.
   uint32_t nib_mask = 0x000F000Fu, magic = E::MAGIC;
-  asm volatile("" : "+s"(nib_mask));
-  asm volatile("" : "+v"(magic));
+  if constexpr (WARM > 0 || STAGE || MF == 4) {
+    asm volatile("" : "+s"(nib_mask));
+    asm volatile("" : "+v"(magic));
+  }
   const W4View v = w4_view(p);
   const int N = p.N, K = p.K, M = v.M;
   constexpr int CB = QOUT ? 2 : 1;                      // 64-column blocks per workgroup

@@ -164,3 +164,29 @@ def test_pingpong_k_loops_keep_their_instruction_mix(asm):
         for seg in loops(lines):
             if count(seg, "v_mfma") >= 32 and len(seg) < 1500:
                 assert count(seg, "scratch_") == 0 and count(seg, "v_accvgpr") == 0, (name, len(seg))
+
+
+def test_default_kernels_are_the_gpu_tested_code():
+    """Every kernel of the last commit whose tree passed the GPU suite on an MI355X (tests/golden/isa_fingerprints.json,
+    made by tests/golden/make_isa_fingerprints.py) compiles from the working tree to the same instruction stream: the
+    kernels that run by default are that code, and what was written since lives in kernels of its own (selectable
+    variants). The normalisation is the generator's: labels, the offset of the first hidden kernel argument, the order
+    inside runs of scalar register copies."""
+    import importlib.util
+    import json
+
+    spec = importlib.util.spec_from_file_location("make_isa_fingerprints", os.path.join(ROOT, "tests", "golden", "make_isa_fingerprints.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    golden = json.load(open(os.path.join(ROOT, "tests", "golden", "isa_fingerprints.json")))
+    now = gen.compile_tree(CSRC)
+    checked = 0
+    for f, ks in golden["kernels"].items():
+        for name, fp in ks.items():
+            # the group-size-128 W4A16 kernel has two more template arguments now: <..., WARM = 0, STAGE = false>
+            new = name.replace("EEEv8W4Params", "ELi0ELb0EEEv8W4Params") if "w4a16_splitk_g128" in name else name
+            assert new in now[f], (f, name)
+            assert now[f][new] == fp, (f, name)
+            checked += 1
+    assert checked >= 80
+

@@ -46,7 +46,7 @@ template <class F> static void build_tile_prefix(const int32_t* row_off, int G, 
 }
 static void build_group_tables(const int32_t*, int, int, int, int, int32_t*, int32_t*, int, int) { abort(); }
 
-template <int OP, bool TALL = false>
+template <int OP, bool TALL = false, bool LISTS2 = false>
 static void prologue(const GgParams& p, int32_t* seq_out, int* n_my_out) {
   static int32_t row_off[MOE_GG_MAX_GROUPS + 1], tile_off[MOE_GG_MAX_GROUPS + 1], part_off[MOE_GG_MAX_GROUPS + 1];
   static int32_t seq_tab[2 * MOE_GG_SEQ_CAP];
@@ -61,7 +61,7 @@ HARNESS_TAIL = r'''
 }
 
 extern "C" int emu_prologue(int op, const int32_t* m_sizes, int G, int M, int N, int K, int skip_rows, int tails_apart,
-                            int nwg, int xcds, int split_tails, int32_t* out, int cap) {
+                            int nwg, int xcds, int split_tails, int lists2, int32_t* out, int cap) {
   const bool tall = split_tails == 2;   // the four-wave kernel's lists with tiles of up to 256 + 32 rows
   GgParams p{m_sizes, G, M, N, K, skip_rows, tails_apart, xcds, tall ? 0 : split_tails};
   gridDim.x = nwg;
@@ -70,12 +70,19 @@ extern "C" int emu_prologue(int op, const int32_t* m_sizes, int G, int M, int N,
   for (int wg = 0; wg < nwg; ++wg) {
     blockIdx.x = wg;
     int n_my = 0;
-    if (op == OP_BF16 && tall) prologue<OP_BF16, true>(p, seq, &n_my);
-    else if (op == OP_BF16_SWIGLU && tall) prologue<OP_BF16_SWIGLU, true>(p, seq, &n_my);
+    // As the launchers choose: the first prologue for the kernels that run by default, the second one for the
+    // split-tail order, the row gather and the four-wave kernels (lists2 = 1 forces it: those kernels also run the
+    // plain two-list order through it).
+    const bool second = lists2 || p.split_tails;
+    if (op == OP_BF16 && tall) prologue<OP_BF16, true, true>(p, seq, &n_my);
+    else if (op == OP_BF16_SWIGLU && tall) prologue<OP_BF16_SWIGLU, true, true>(p, seq, &n_my);
     else if (tall) return -1;
+    else if (op == OP_BF16 && second) prologue<OP_BF16, false, true>(p, seq, &n_my);
     else if (op == OP_BF16) prologue<OP_BF16>(p, seq, &n_my);
+    else if (op == OP_BF16_SWIGLU && second) prologue<OP_BF16_SWIGLU, false, true>(p, seq, &n_my);
     else if (op == OP_BF16_SWIGLU) prologue<OP_BF16_SWIGLU>(p, seq, &n_my);
-    else if (op == OP_BF16_SWIGLU_GATHER) prologue<OP_BF16_SWIGLU_GATHER>(p, seq, &n_my);
+    else if (op == OP_BF16_SWIGLU_GATHER) prologue<OP_BF16_SWIGLU_GATHER, false, true>(p, seq, &n_my);
+    else if (op == OP_FP8_BLOCK && second) prologue<OP_FP8_BLOCK, false, true>(p, seq, &n_my);
     else if (op == OP_FP8_BLOCK) prologue<OP_FP8_BLOCK>(p, seq, &n_my);
     else return -1;
     for (int i = 0; i < n_my; ++i) {
@@ -95,13 +102,13 @@ extern "C" int emu_prologue(int op, const int32_t* m_sizes, int G, int M, int N,
 @pytest.fixture(scope="module")
 def emu(tmp_path_factory):
     src = open(os.path.join(CSRC, "gg_pingpong.hip")).read()
-    begin = "  int total, total_low = 0;\n"
+    begin = "  int n_my = 0;\n  if constexpr (!LISTS2) {\n"
     end = "  __syncthreads();\n\n  Shared sh{row_off"
     assert src.count(begin) == 1 and src.count(end) == 1, "markers of the prologue moved"
-    body = src[src.index(begin):src.index(end)]
-    early = "  if (n_long + n_low == 0) return;"
-    assert body.count(early) == 1
-    body = body.replace(early, "  if (n_long + n_low == 0) { *n_my_out = 0; return; }")
+    body = src[src.index(begin):src.index(end)]      # both prologues: the default kernels' and the second one
+    early = "    if (n_long + n_low == 0) return;"
+    assert body.count(early) == 2
+    body = body.replace(early, "    if (n_long + n_low == 0) { *n_my_out = 0; return; }")
     d = tmp_path_factory.mktemp("emu")
     cpp = d / "emu.cpp"
     cpp.write_text(HARNESS_HEAD + body + HARNESS_TAIL)
@@ -109,7 +116,7 @@ def emu(tmp_path_factory):
     subprocess.run(["g++", "-O1", "-std=c++17", "-shared", "-fPIC", "-I", CSRC, "-o", str(so), str(cpp)], check=True)
     lib = ctypes.CDLL(str(so))
     lib.emu_prologue.restype = ctypes.c_int
-    lib.emu_prologue.argtypes = [ctypes.c_int, I32P] + [ctypes.c_int] * 9 + [I32P, ctypes.c_int]
+    lib.emu_prologue.argtypes = [ctypes.c_int, I32P] + [ctypes.c_int] * 10 + [I32P, ctypes.c_int]
     return lib
 
 
@@ -123,11 +130,11 @@ def split(lib, request):
         lib.moe_gg_set_variant(2, -1)
 
 
-def device_tiles(emu, op, sizes, N, K, nwg, skip=0, tails=0, M=None, split=0):
+def device_tiles(emu, op, sizes, N, K, nwg, skip=0, tails=0, M=None, split=0, lists2=0):
     ms = np.ascontiguousarray(sizes, dtype=np.int32)
     out = np.zeros((CAP, 6), dtype=np.int32)
     n = emu.emu_prologue(op, ms.ctypes.data_as(I32P), len(ms), int(ms.sum()) if M is None else M, N, K, skip, tails, nwg, 8,
-                         split, out.ctypes.data_as(I32P), CAP)
+                         split, lists2, out.ctypes.data_as(I32P), CAP)
     assert 0 <= n < CAP
     return out[:n]
 
@@ -159,8 +166,9 @@ def shape_sets():
 def test_device_prologue_equals_the_host_mirror(emu, lib, split):
     for sizes, N, nwg in shape_sets():
         h = host_tiles(lib, sizes, N, 256, nwg)
-        d = device_tiles(emu, 0, sizes, N, 4096, nwg, split=split).copy()
-        assert h.shape == d.shape and (h == d).all(), ("bf16", sizes[:8], N, nwg)
+        for lists2 in (0, 1):   # the default kernels' prologue and the second one (four-wave kernels run it in both orders)
+            d = device_tiles(emu, 0, sizes, N, 4096, nwg, split=split, lists2=lists2).copy()
+            assert h.shape == d.shape and (h == d).all(), ("bf16", sizes[:8], N, nwg, lists2)
         n_out = max(128, N // 2 // 128 * 128)       # fused gate/up kernel: p.N = 2 n, tiles of 128 output columns
         h = host_tiles(lib, sizes, n_out, 128, nwg)
         for op in (4, 9):   # the fused gate/up kernel and its form with the row gather
