@@ -462,10 +462,11 @@ def test_corrupt_m_sizes_are_clamped_by_every_kernel():
     """Negative sizes, sums beyond M, a size of 2^30: every kernel that reads m_sizes (all GEMM variants, fp8, SwiGLU,
     backward, W4A16 grouped) computes the rows of the clamped sizes, leaves the other rows alone and, with every tensor
     against a guard page, touches nothing outside them."""
-    for order in ("0", "1"):
-        env = dict(os.environ, EMU_GUARD="end", EMU_TRACE="1", EMU_TILE_ORDER=order)
-        p = subprocess.run([sys.executable, os.path.join(EMU, "corrupt_sizes.py")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT)
-        assert p.returncode == 0, (order, p.stdout.decode()[-2000:])
+    procs = [subprocess.Popen([sys.executable, os.path.join(EMU, "corrupt_sizes.py")], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT,
+                              env=dict(os.environ, EMU_GUARD="end", EMU_TRACE="1", EMU_TILE_ORDER=order)) for order in ("0", "1")]
+    for order, p in enumerate(procs):
+        log = p.communicate()[0].decode()
+        assert p.returncode == 0, (order, log[-2000:])
 
 
 def test_no_data_race_between_the_waves_of_a_workgroup():
