@@ -358,8 +358,9 @@ int moe_gg_host_enumerate_tiles(const int32_t* m_sizes_host, int G, int64_t M, i
  * its tiles of the second list spread between its long ones, and cut the long tiles of a sparsely filled last
  * round into row pieces. Six int32 per tile here: (workgroup,
  * group, first row inside the group, rows, first column, columns), for each workgroup in the order in which it
- * computes them; a piece may have 0 rows, and the columns may reach beyond N. The tile decode is the kernels' own
- * code (compiled for the host). */
+ * computes them; a piece may have 0 rows, and the columns may reach beyond N. With MOE_GG_ORDER_TALL_TILES pinned the
+ * lists are those of MOE_GG_GG_FOURWAVE_TALL: rows may be up to 256 + 32. The tile decode is the kernels' own code
+ * (compiled for the host). */
 int moe_gg_host_enumerate_tiles_two_lists(const int32_t* m_sizes_host, int G, int64_t M, int N, int block_m,
                                           int block_n, int num_workgroups, int xcds, int32_t* out,
                                           int max_tiles);
