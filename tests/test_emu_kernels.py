@@ -395,35 +395,52 @@ def test_committed_golden_vectors():
 
 FUZZ = [  # (compute units, load-landing model, wave order seed): few units = long tile sequences per workgroup
     ("1", "late", "0"), ("2", "early", "0"), ("3", "late", "5"), ("8", "early", "9"), ("16", "late", "0"), ("5", "late", "77")]
+GUARDED = [("end", "8", "late", "0"), ("start", "8", "early", "3"), ("end", "2", "late", "11"), ("start", "13", "late", "0")]
+UBSAN_ENV = dict(EMU_UBSAN="1", EMU_OUT=os.path.join(EMU, "_build", "ubsan"), EMU_GUARD="end", EMU_TRACE="1")
 
 
-def test_pingpong_random_shapes_over_unit_counts_and_schedules():
-    procs = []
+def _child(script, args, **env):
+    return subprocess.Popen([sys.executable, os.path.join(EMU, script)] + list(args), env=dict(os.environ, **env), stdout=subprocess.PIPE,
+                            stderr=subprocess.STDOUT, cwd=ROOT)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def children():
+    """The random-launch runs of this file are child processes of their own; they are started when the first test of the
+    file runs (the emulated library is built by then) and collected by the tests at its end, so that they run beside
+    the tests in between instead of after them."""
+    build_emu.build()
+    c = {}
     for i, (cus, dma, seed) in enumerate(FUZZ):
-        env = dict(os.environ, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed, EMU_TILE_ORDER=str(i % 2))
-        procs.append(subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_pingpong.py"), str(100 + i), "20"], env=env,
-                                      stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT))
-    for cfg, p in zip(FUZZ, procs):
+        c["pingpong", i] = _child("fuzz_pingpong.py", [str(100 + i), "20"], EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed, EMU_TILE_ORDER=str(i % 2))
+    for i, (guard, cus, dma, seed) in enumerate(GUARDED):
+        env = dict(EMU_GUARD=guard, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed, EMU_TRACE="1", EMU_TILE_ORDER=str(i % 2))
+        if i >= 2:
+            env["EMU_LDS_POISON"] = "1"      # workgroups start with NaN patterns in LDS instead of a predecessor's data
+        c["guarded", i] = _child("fuzz_all.py", [str(200 + i), "40"], **env)
+    for order in ("0", "1"):
+        c["corrupt", order] = _child("corrupt_sizes.py", [], EMU_GUARD="end", EMU_TRACE="1", EMU_TILE_ORDER=order)
+    c["ubsan build"] = _child("build_emu.py", [], **UBSAN_ENV)     # the build with trapping checks; its runs follow in the test
+    yield c
+    for p in c.values():
+        if p.poll() is None:
+            p.kill()
+
+
+def test_pingpong_random_shapes_over_unit_counts_and_schedules(children):
+    for i, cfg in enumerate(FUZZ):
+        p = children["pingpong", i]
         log = p.communicate()[0].decode()
         assert p.returncode == 0, (cfg, log[-2000:])
 
 
-GUARDED = [("end", "8", "late", "0"), ("start", "8", "early", "3"), ("end", "2", "late", "11"), ("start", "13", "late", "0")]
-
-
-def test_every_entry_point_on_random_shapes_with_tensors_against_guard_pages():
+def test_every_entry_point_on_random_shapes_with_tensors_against_guard_pages(children):
     """Inputs, outputs and the workspace end (or begin) at an inaccessible page: a kernel that touches memory outside a
     tensor, by one element or by one 16-byte load, ends the child process with a memory fault. Two of the four runs
     start every workgroup with LDS full of NaN patterns: a result that depends on LDS bytes its workgroup never wrote
     fails the comparison."""
-    procs = []
-    for i, (guard, cus, dma, seed) in enumerate(GUARDED):
-        env = dict(os.environ, EMU_GUARD=guard, EMU_CUS=cus, EMU_DMA=dma, EMU_SEED=seed, EMU_TRACE="1", EMU_TILE_ORDER=str(i % 2))
-        if i >= 2:
-            env["EMU_LDS_POISON"] = "1"      # workgroups start with NaN patterns in LDS instead of a predecessor's data
-        procs.append(subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_all.py"), str(200 + i), "40"], env=env,
-                                      stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT))
-    for cfg, p in zip(GUARDED, procs):
+    for i, cfg in enumerate(GUARDED):
+        p = children["guarded", i]
         log = p.communicate()[0].decode()
         assert p.returncode == 0, (cfg, log[-2000:])
 
@@ -442,29 +459,26 @@ def test_config2_at_full_size():
         assert p.returncode == 0, (case, log[-2000:])
 
 
-def test_kernels_with_trapping_checks_of_alignment_shifts_overflow_and_bounds():
+def test_kernels_with_trapping_checks_of_alignment_shifts_overflow_and_bounds(children):
     """A second host build of the kernels in which every vector access checks its alignment, every shift its count,
     every signed operation its range and every index into a fixed-size array its bound, each ending in a trap
     (EMU_UBSAN, tests/emu/build_emu.py): 80 random calls over all entry points, against guard pages, complete
     without one. (An ordinary build would read a misaligned 16-byte LDS access without complaint; the GPU would not.)"""
-    env = dict(os.environ, EMU_UBSAN="1", EMU_OUT=os.path.join(EMU, "_build", "ubsan"), EMU_GUARD="end", EMU_TRACE="1")
-    b = subprocess.run([sys.executable, os.path.join(EMU, "build_emu.py")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT)
-    assert b.returncode == 0, b.stdout.decode()[-2000:]
-    procs = [subprocess.Popen([sys.executable, os.path.join(EMU, "fuzz_all.py"), str(700 + i), "40"], stdout=subprocess.PIPE,
-                              stderr=subprocess.STDOUT, cwd=ROOT, env=dict(env, EMU_TILE_ORDER=str(i), EMU_SEED=str(3 * i)))
-             for i in range(2)]
+    b = children["ubsan build"]
+    log = b.communicate()[0].decode()
+    assert b.returncode == 0, log[-2000:]
+    procs = [_child("fuzz_all.py", [str(700 + i), "40"], EMU_TILE_ORDER=str(i), EMU_SEED=str(3 * i), **UBSAN_ENV) for i in range(2)]
     for i, p in enumerate(procs):
         log = p.communicate()[0].decode()
         assert p.returncode == 0, (i, log[-2000:])
 
 
-def test_corrupt_m_sizes_are_clamped_by_every_kernel():
+def test_corrupt_m_sizes_are_clamped_by_every_kernel(children):
     """Negative sizes, sums beyond M, a size of 2^30: every kernel that reads m_sizes (all GEMM variants, fp8, SwiGLU,
     backward, W4A16 grouped) computes the rows of the clamped sizes, leaves the other rows alone and, with every tensor
     against a guard page, touches nothing outside them."""
-    procs = [subprocess.Popen([sys.executable, os.path.join(EMU, "corrupt_sizes.py")], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, cwd=ROOT,
-                              env=dict(os.environ, EMU_GUARD="end", EMU_TRACE="1", EMU_TILE_ORDER=order)) for order in ("0", "1")]
-    for order, p in enumerate(procs):
+    for order in ("0", "1"):
+        p = children["corrupt", order]
         log = p.communicate()[0].decode()
         assert p.returncode == 0, (order, log[-2000:])
 

@@ -26,28 +26,45 @@ SKIP = ("not config4 and not mixtral and not invalid and not rejects and not err
         "and not prefill_rows and not m_sizes5 and not sizes1-1032")
 
 
-def test_gpu_tests_pass_against_the_emulated_library():
+SMOKE = ("import sys; sys.path.insert(0, 'tests/emu'); sys.path.insert(0, '.'); import gpu_tests_on_emu as g; g.install(); "
+         "import __graft_entry__ as e; e.smoke()")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def children():
+    """The three child processes of this file, started together when its first test runs."""
     build_emu.build()
-    p = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "emu", "gpu_tests_on_emu.py")] + FILES + ["-k", SKIP],
-                       cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=1500)
-    log = p.stdout.decode()
+    emu = os.path.join(ROOT, "tests", "emu")
+    c = {"tests": subprocess.Popen([sys.executable, os.path.join(emu, "gpu_tests_on_emu.py")] + FILES + ["-k", SKIP], cwd=ROOT,
+                                   stdout=subprocess.PIPE, stderr=subprocess.STDOUT),
+         "bench": subprocess.Popen([sys.executable, os.path.join(emu, "bench_on_emu.py")], cwd=ROOT, stdout=subprocess.PIPE,
+                                   stderr=subprocess.PIPE),
+         "smoke": subprocess.Popen([sys.executable, "-c", SMOKE], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)}
+    yield c
+    for p in c.values():
+        if p.poll() is None:
+            p.kill()
+
+
+def test_gpu_tests_pass_against_the_emulated_library(children):
+    p = children["tests"]
+    log = p.communicate(timeout=1500)[0].decode()
     assert p.returncode == 0, log[-3000:]
     m = re.search(r"(\d+) passed", log)
     assert m and int(m.group(1)) >= 100, log[-1000:]
 
 
-def test_bench_py_runs_end_to_end_against_the_emulated_library():
+def test_bench_py_runs_end_to_end_against_the_emulated_library(children):
     """bench.py's main() and every secondary workload (with CPU baselines and the optional sweep) at reduced shapes,
     through the real ctypes calls into the emulated kernels: one JSON line with the contract's fields, no workload
     ending in an "error" entry, the baselines attached after the device legs."""
     import json
 
-    build_emu.build()
-    p = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "emu", "bench_on_emu.py")], cwd=ROOT, stdout=subprocess.PIPE,
-                       stderr=subprocess.PIPE, timeout=1500)
-    assert p.returncode == 0, p.stderr.decode()[-3000:]
-    lines = [ln for ln in p.stdout.decode().splitlines() if ln.startswith("{")]
-    assert len(lines) == 1, p.stdout.decode()[-2000:]
+    p = children["bench"]
+    out, err = p.communicate(timeout=1500)
+    assert p.returncode == 0, err.decode()[-3000:]
+    lines = [ln for ln in out.decode().splitlines() if ln.startswith("{")]
+    assert len(lines) == 1, out.decode()[-2000:]
     d = json.loads(lines[0])
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
                 "dtype", "data", "config", "roofline", "cpu_baseline", "secondary", "dense_gemm_library", "wall_s"):
@@ -63,9 +80,8 @@ def test_bench_py_runs_end_to_end_against_the_emulated_library():
     assert sec[-1]["rows"] and sec[-1]["rows"][0]["m"] == 1
 
 
-def test_smoke_entry_point_against_the_emulated_library():
+def test_smoke_entry_point_against_the_emulated_library(children):
     """__graft_entry__.smoke() (one small grouped GEMM through the Python entry function, checked against the oracle)."""
-    code = ("import sys; sys.path.insert(0, 'tests/emu'); sys.path.insert(0, '.'); import gpu_tests_on_emu as g; g.install(); "
-            "import __graft_entry__ as e; e.smoke()")
-    p = subprocess.run([sys.executable, "-c", code], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=600)
-    assert p.returncode == 0 and "smoke ok" in p.stdout.decode(), p.stdout.decode()[-2000:]
+    p = children["smoke"]
+    log = p.communicate(timeout=600)[0].decode()
+    assert p.returncode == 0 and "smoke ok" in log, log[-2000:]
